@@ -1,0 +1,235 @@
+"""numpy/ctypes front end of the CPU oracle (``md_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``.  The product package never imports it.
+
+Every function takes and returns numpy arrays with the reference's layouts
+(positions ``(N,3) f32``, cell ``(B,3,3) f32`` rows = lattice vectors, pbc ``(B,3) bool``,
+``batch_ptr (B+1) i32``, ``batch_idx (N) i32``; see nvalchemi/neighbors.py:239-266).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_HERE = Path(__file__).resolve().parent
+_LIB_PATH = _HERE / "libmd_oracle.so"
+_lib = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+
+
+def build(force: bool = False) -> Path:
+    """Compile ``md_oracle.c`` with gcc (``make -C oracle``)."""
+    if force and _LIB_PATH.exists():
+        _LIB_PATH.unlink()
+    subprocess.run(["make", "-C", str(_HERE), "-s"], check=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            build()
+        L = ctypes.CDLL(str(_LIB_PATH))
+        L.orc_nl_brute.restype = ctypes.c_int64
+        L.orc_nl_brute.argtypes = [_f32p, _f32p, _u8p, _i32p, ctypes.c_int32, ctypes.c_double,
+                                   ctypes.c_int32, ctypes.c_int64, _i32p]
+        L.orc_nl_cell.restype = ctypes.c_int32
+        L.orc_nl_cell.argtypes = [_f32p, _f32p, _u8p, _i32p, ctypes.c_int32, ctypes.c_double,
+                                  ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, _i32p, _i32p, _i32p]
+        L.orc_lj_matrix.restype = ctypes.c_int32
+        L.orc_lj_matrix.argtypes = [_f32p, _f32p, _i32p, _i32p, _i32p, _i32p, ctypes.c_int32,
+                                    ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                    ctypes.c_double, ctypes.c_double, ctypes.c_double,
+                                    ctypes.c_int32, _f32p, _f32p, _f32p, _f32p]
+        L.orc_vv_pre.restype = None
+        L.orc_vv_pre.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _i32p, _u8p, ctypes.c_int32]
+        L.orc_vv_post.restype = None
+        L.orc_vv_post.argtypes = [_f32p, _f32p, _f32p, _f32p, _i32p, _u8p, ctypes.c_int32]
+        L.orc_fire_step.restype = None
+        L.orc_fire_step.argtypes = [_f32p, _f32p, _f32p, _f32p] + [_f32p] * 7 + [_i32p, _i32p] + \
+            [_f32p] * 5 + [_i32p, _u8p, ctypes.c_int32, ctypes.c_int32]
+        L.orc_fmax.restype = None
+        L.orc_fmax.argtypes = [_f32p, _i32p, ctypes.c_int32, ctypes.c_int32, _f32p]
+        L.orc_num_threads.restype = ctypes.c_int32
+        _lib = L
+    return _lib
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _u8(a):
+    return np.ascontiguousarray(a, dtype=np.uint8)
+
+
+def _p(a, t):
+    return None if a is None else a.ctypes.data_as(t)
+
+
+def set_threads(n: int) -> None:
+    """Thread count of the OpenMP loops (read by libgomp at the next parallel region)."""
+    os.environ["OMP_NUM_THREADS"] = str(n)
+    try:
+        ctypes.CDLL("libgomp.so.1").omp_set_num_threads(int(n))
+    except OSError:
+        pass
+
+
+def num_threads() -> int:
+    return int(lib().orc_num_threads())
+
+
+def batch_idx_from_ptr(batch_ptr) -> np.ndarray:
+    ptr = np.asarray(batch_ptr, dtype=np.int64)
+    return np.repeat(np.arange(len(ptr) - 1, dtype=np.int32), np.diff(ptr)).astype(np.int32)
+
+
+def canonical_edges(edges: np.ndarray) -> np.ndarray:
+    """Sort ``(E,5)`` records ``(i, j, sx, sy, sz)`` lexicographically."""
+    e = np.asarray(edges, dtype=np.int64).reshape(-1, 5)
+    if len(e) == 0:
+        return e
+    order = np.lexsort((e[:, 4], e[:, 3], e[:, 2], e[:, 1], e[:, 0]))
+    return e[order]
+
+
+def matrix_to_edges(nm, nn, shifts=None) -> np.ndarray:
+    """Dense ``(N,K)`` matrix + counts (+ ``(N,K,3)`` shifts) -> canonical ``(E,5)`` records.
+
+    Rows are read in ``[0, min(count, K))`` as the reference does
+    (nvalchemi/models/_ops/neighbor_filter.py:255-283).
+    """
+    nm = np.asarray(nm)
+    nn = np.asarray(nn)
+    N, K = nm.shape
+    cols = np.arange(K)[None, :]
+    valid = cols < np.minimum(nn, K)[:, None]
+    ii, kk = np.nonzero(valid)
+    out = np.zeros((len(ii), 5), dtype=np.int64)
+    out[:, 0] = ii
+    out[:, 1] = nm[ii, kk]
+    if shifts is not None:
+        out[:, 2:] = np.asarray(shifts)[ii, kk]
+    return canonical_edges(out)
+
+
+def nl_brute(positions, cell, pbc, batch_ptr, cutoff: float, half: bool = False) -> np.ndarray:
+    """All ``(i, j, S)`` with ``|r_j - r_i + S.cell| < cutoff`` by brute force; canonical order."""
+    pos = _f32(positions)
+    ptr = _i32(batch_ptr)
+    B = len(ptr) - 1
+    c = None if cell is None else _f32(cell).reshape(B, 9)
+    p = None if (pbc is None or cell is None) else _u8(pbc).reshape(B, 3)
+    L = lib()
+    args = (_p(pos, _f32p), _p(c, _f32p), _p(p, _u8p), _p(ptr, _i32p), B, float(cutoff), int(half))
+    total = L.orc_nl_brute(*args, 0, None)
+    out = np.zeros((max(total, 1), 5), dtype=np.int32)
+    total2 = L.orc_nl_brute(*args, total, _p(out, _i32p))
+    assert total2 == total
+    return canonical_edges(out[:total])
+
+
+def nl_cell(positions, cell, pbc, batch_ptr, cutoff: float, max_neighbors: int, half: bool = False):
+    """Cell-list build into ``(neighbor_matrix, num_neighbors, shifts)`` (reference layout)."""
+    pos = _f32(positions)
+    ptr = _i32(batch_ptr)
+    B = len(ptr) - 1
+    N = pos.shape[0]
+    K = int(max_neighbors)
+    c = None if cell is None else _f32(cell).reshape(B, 9)
+    p = None if (pbc is None or cell is None) else _u8(pbc).reshape(B, 3)
+    nm = np.empty((N, K), dtype=np.int32)
+    nn = np.empty(N, dtype=np.int32)
+    sh = np.empty((N, K, 3), dtype=np.int32)
+    lib().orc_nl_cell(_p(pos, _f32p), _p(c, _f32p), _p(p, _u8p), _p(ptr, _i32p), B, float(cutoff),
+                      int(half), K, N, _p(nm, _i32p), _p(nn, _i32p), _p(sh, _i32p))
+    return nm, nn, sh
+
+
+def lj_matrix(positions, cells, neighbor_matrix, shifts, num_neighbors, batch_idx, fill_value,
+              epsilon, sigma, cutoff, half=False, virial=False):
+    """LJ over the dense matrix -> dict(atomic_energies, forces, energy[, virials])."""
+    pos = _f32(positions)
+    N = pos.shape[0]
+    nm = _i32(neighbor_matrix)
+    K = nm.shape[1] if nm.ndim == 2 else 0
+    cells = _f32(cells).reshape(-1, 9)
+    B = cells.shape[0]
+    sh = None if shifts is None else _i32(shifts)
+    nn = _i32(num_neighbors)
+    bi = _i32(batch_idx)
+    e = np.zeros(N, dtype=np.float32)
+    f = np.zeros((N, 3), dtype=np.float32)
+    w = np.zeros((B, 9), dtype=np.float32) if virial else None
+    es = np.zeros(B, dtype=np.float32)
+    lib().orc_lj_matrix(_p(pos, _f32p), _p(cells, _f32p), _p(nm, _i32p), _p(sh, _i32p), _p(nn, _i32p),
+                        _p(bi, _i32p), N, K, B, int(fill_value), float(epsilon), float(sigma),
+                        float(cutoff), int(half), _p(e, _f32p), _p(f, _f32p), _p(w, _f32p),
+                        _p(es, _f32p))
+    out = {"atomic_energies": e, "forces": f, "energy": es}
+    if virial:
+        out["virials"] = w
+    return out
+
+
+def vv_pre(positions, velocities, forces, masses, dt, batch_idx, active=None):
+    """In-place first half of velocity Verlet on float32 arrays."""
+    for a in (positions, velocities):
+        assert a.dtype == np.float32 and a.flags.c_contiguous
+    act = None if active is None else _u8(active)
+    lib().orc_vv_pre(_p(positions, _f32p), _p(velocities, _f32p), _p(_f32(forces), _f32p),
+                     _p(_f32(masses), _f32p), _p(_f32(dt), _f32p), _p(_i32(batch_idx), _i32p),
+                     _p(act, _u8p), positions.shape[0])
+
+
+def vv_post(velocities, forces, masses, dt, batch_idx, active=None):
+    """In-place second half of velocity Verlet on float32 arrays."""
+    assert velocities.dtype == np.float32 and velocities.flags.c_contiguous
+    act = None if active is None else _u8(active)
+    lib().orc_vv_post(_p(velocities, _f32p), _p(_f32(forces), _f32p), _p(_f32(masses), _f32p),
+                      _p(_f32(dt), _f32p), _p(_i32(batch_idx), _i32p), _p(act, _u8p),
+                      velocities.shape[0])
+
+
+def fire_step(positions, velocities, forces, masses, state: dict, batch_idx, active=None):
+    """In-place FIRE step.  ``state`` holds float32 ``alpha, dt, alpha_start, f_alpha, dt_min,
+    dt_max, maxstep, f_dec, f_inc, vf, vv, ff`` and int32 ``n_steps_positive, n_min`` arrays
+    of length M; ``alpha, dt, n_steps_positive, vf, vv, ff`` are updated."""
+    for a in (positions, velocities):
+        assert a.dtype == np.float32 and a.flags.c_contiguous
+    for k in ("alpha", "dt", "vf", "vv", "ff"):
+        assert state[k].dtype == np.float32
+    assert state["n_steps_positive"].dtype == np.int32
+    M = state["alpha"].shape[0]
+    act = None if active is None else _u8(active)
+    g = lambda k: _p(_f32(state[k]), _f32p)  # noqa: E731
+    lib().orc_fire_step(_p(positions, _f32p), _p(velocities, _f32p), _p(_f32(forces), _f32p),
+                        _p(_f32(masses), _f32p), _p(state["alpha"], _f32p), _p(state["dt"], _f32p),
+                        g("alpha_start"), g("f_alpha"), g("dt_min"), g("dt_max"), g("maxstep"),
+                        _p(state["n_steps_positive"], _i32p), _p(_i32(state["n_min"]), _i32p),
+                        g("f_dec"), g("f_inc"), _p(state["vf"], _f32p), _p(state["vv"], _f32p),
+                        _p(state["ff"], _f32p), _p(_i32(batch_idx), _i32p), _p(act, _u8p),
+                        positions.shape[0], M)
+
+
+def fmax(forces, batch_idx, n_systems: int) -> np.ndarray:
+    f = _f32(forces)
+    out = np.empty(n_systems, dtype=np.float32)
+    lib().orc_fmax(_p(f, _f32p), _p(_i32(batch_idx), _i32p), f.shape[0], int(n_systems),
+                   _p(out, _f32p))
+    return out

@@ -1,0 +1,548 @@
+/*
+ * md_oracle.c -- CPU restatement of the batched-MD inner loop of nvalchemi-toolkit.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the parity checker for the HIP path: it may be
+ * loaded by tests/, by __graft_entry__.smoke() and by bench.py's cpu_baseline leg, and by
+ * nothing else.  The product library never links, imports or calls it.
+ *
+ * The arithmetic of this path lives in a third-party wheel that is absent from the
+ * reference tree (nvalchemi-toolkit-ops==0.4.0, pinned in uv.lock:186-189,4168), so every
+ * function below restates the published algorithm and anchors on the reference's own call
+ * sites, docstrings and tests:
+ *
+ *   orc_nl_brute / orc_nl_cell   nvalchemi/neighbors.py:244-273 (output layout, overflow
+ *                                protocol), nvalchemi/models/_ops/neighbor_filter.py:98-119
+ *                                (pair geometry r_ij = r_j - r_i + S.cell, row-vector cell,
+ *                                strict d2 < rc2), nvalchemi/hooks/neighbor_list.py:685-704
+ *                                (bin -> histogram -> scan -> scatter -> stencil search)
+ *   orc_lj_matrix                nvalchemi/models/_ops/lj.py:31-54,116-216,246-321 and
+ *                                nvalchemi/models/lj.py:464-477 (fp64 per-system sum)
+ *   orc_vv_pre / orc_vv_post     nvalchemi/dynamics/_ops/velocity_verlet.py:63-64,112
+ *   orc_fire_step                nvalchemi/dynamics/_ops/fire.py:245-362,
+ *                                nvalchemi/dynamics/optimizers/fire.py:69-76,182-219,
+ *                                nvalchemi/distributed/_dynamics_coordinator.py:296-322
+ *   orc_fmax                     nvalchemi/dynamics/base.py:304-349
+ *
+ * Pinning status (what checks each function; see tests/test_oracle_*.py):
+ *   orc_nl_brute   pinned: hand geometries restated from the reference tests
+ *                  (test/hooks/test_neighbor_list_hook.py:65-105,630-719,
+ *                  test/models/test_neighbor_filter.py:182-215), invariants (symmetry,
+ *                  no self pair, no cross-system pair), lattice coordination numbers.
+ *   orc_nl_cell    pinned against orc_nl_brute (set equality on random periodic,
+ *                  triclinic, mixed-pbc, small-cell and non-periodic inputs).
+ *   orc_lj_matrix  pinned: closed forms (u(sigma)=0, u(2^(1/6)sigma)=-eps with zero
+ *                  force, literal dimer value), F = -dE/dr by fp64 finite differences,
+ *                  W = -dE/d(strain) by finite differences, sum F = 0.
+ *                  Still unpinned by anything the reference holds: whether the truncated
+ *                  potential is energy-shifted at the cutoff (taken as NOT shifted), the
+ *                  C2 switching polynomial for switch_width > 0 (not implemented), the
+ *                  half-list energy attribution.
+ *   orc_vv_*       pinned: harmonic-oscillator closed form, time reversibility.
+ *   orc_fire_step  PARITY UNPINNED against the reference: the exact ordering of FIRE's
+ *                  sub-steps is only visible inside the absent wheel.  The restatement
+ *                  follows Bitzek 2006 / ASE ordering, constrained by the reference's
+ *                  notes (reductions at entry; mixing with the stored alpha; per-atom
+ *                  maxstep clamp; vanilla branch only).  Checked by invariants only.
+ *   orc_fmax       pinned: in-tree Torch definition is complete; literal cases.
+ *
+ * Numerical definition of the neighbor set: the pair (i, j, S) is a neighbor iff
+ *   d = (r_j - r_i) + (S0*a0 + S1*a1 + S2*a2),  d.d < rc*rc
+ * evaluated in IEEE double on the given float32 inputs (each operation rounded once,
+ * no fused multiply-add), i.e. to within 1e-15 of exact arithmetic on the inputs.
+ * Compile with -ffp-contract=off.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------------------------
+ * per-system geometry
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    double h[9];    /* rows = lattice vectors */
+    double hinv[9]; /* inverse, so frac = r . hinv (row vector times matrix) */
+    double width[3]; /* perpendicular width of the cell along each lattice direction */
+    int per[3];
+    int has_cell;
+} orc_sys_t;
+
+static void orc_inv3(const double* m, double* inv) {
+    double c00 = m[4] * m[8] - m[5] * m[7];
+    double c01 = m[5] * m[6] - m[3] * m[8];
+    double c02 = m[3] * m[7] - m[4] * m[6];
+    double det = m[0] * c00 + m[1] * c01 + m[2] * c02;
+    double id = 1.0 / det;
+    inv[0] = c00 * id;
+    inv[1] = (m[2] * m[7] - m[1] * m[8]) * id;
+    inv[2] = (m[1] * m[5] - m[2] * m[4]) * id;
+    inv[3] = c01 * id;
+    inv[4] = (m[0] * m[8] - m[2] * m[6]) * id;
+    inv[5] = (m[2] * m[3] - m[0] * m[5]) * id;
+    inv[6] = c02 * id;
+    inv[7] = (m[1] * m[6] - m[0] * m[7]) * id;
+    inv[8] = (m[0] * m[4] - m[1] * m[3]) * id;
+}
+
+static void orc_sys_init(orc_sys_t* s, const float* cell, const uint8_t* pbc) {
+    int d, k;
+    if (cell) {
+        for (k = 0; k < 9; ++k) s->h[k] = (double)cell[k];
+        s->has_cell = 1;
+    } else {
+        for (k = 0; k < 9; ++k) s->h[k] = (k % 4 == 0) ? 1.0 : 0.0;
+        s->has_cell = 0;
+    }
+    orc_inv3(s->h, s->hinv);
+    for (d = 0; d < 3; ++d) {
+        /* column d of hinv is the reciprocal vector of lattice direction d */
+        double nx = s->hinv[0 + d], ny = s->hinv[3 + d], nz = s->hinv[6 + d];
+        s->width[d] = 1.0 / sqrt(nx * nx + ny * ny + nz * nz);
+        s->per[d] = (cell && pbc) ? (pbc[d] != 0) : 0;
+    }
+}
+
+static inline void orc_frac(const orc_sys_t* s, const float* r, double* f) {
+    double x = r[0], y = r[1], z = r[2];
+    f[0] = x * s->hinv[0] + y * s->hinv[3] + z * s->hinv[6];
+    f[1] = x * s->hinv[1] + y * s->hinv[4] + z * s->hinv[7];
+    f[2] = x * s->hinv[2] + y * s->hinv[5] + z * s->hinv[8];
+}
+
+/* the one definition of the pair separation, shared by the neighbor test and LJ */
+static inline double orc_pair_d2(const float* ri, const float* rj, const int* S, const double* h,
+                                 double* d) {
+    double tx = ((double)S[0] * h[0] + (double)S[1] * h[3]) + (double)S[2] * h[6];
+    double ty = ((double)S[0] * h[1] + (double)S[1] * h[4]) + (double)S[2] * h[7];
+    double tz = ((double)S[0] * h[2] + (double)S[1] * h[5]) + (double)S[2] * h[8];
+    d[0] = ((double)rj[0] - (double)ri[0]) + tx;
+    d[1] = ((double)rj[1] - (double)ri[1]) + ty;
+    d[2] = ((double)rj[2] - (double)ri[2]) + tz;
+    return (d[0] * d[0] + d[1] * d[1]) + d[2] * d[2];
+}
+
+static inline int orc_half_keep(int i, int j, const int* S) {
+    /* half list: each undirected pair once; i<j, and for self images the
+       lexicographically positive shift */
+    if (i != j) return i < j;
+    if (S[0] != 0) return S[0] > 0;
+    if (S[1] != 0) return S[1] > 0;
+    return S[2] > 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * brute-force neighbor enumeration: every pair of the same system, every image in range.
+ * Writes records (i, j, sx, sy, sz) into out (capacity cap records); returns the total count
+ * (which may exceed cap: nothing is written past cap).
+ * ---------------------------------------------------------------------------------------- */
+ORC_API int64_t orc_nl_brute(const float* pos, const float* cell, const uint8_t* pbc,
+                             const int32_t* batch_ptr, int32_t n_systems, double cutoff,
+                             int32_t half, int64_t cap, int32_t* out) {
+    int64_t total = 0;
+    double rc2 = cutoff * cutoff;
+    for (int s = 0; s < n_systems; ++s) {
+        orc_sys_t sys;
+        orc_sys_init(&sys, cell ? cell + 9 * s : NULL, pbc ? pbc + 3 * s : NULL);
+        int a0 = batch_ptr[s], a1 = batch_ptr[s + 1];
+        int n = a1 - a0;
+        int Q[3];
+        for (int d = 0; d < 3; ++d)
+            Q[d] = sys.per[d] ? (int)floor(cutoff / sys.width[d] * (1.0 + 1e-9)) + 1 : 0;
+        int* wrap = (int*)malloc(sizeof(int) * 3 * (n > 0 ? n : 1));
+        for (int i = 0; i < n; ++i) {
+            double f[3];
+            orc_frac(&sys, pos + 3 * (a0 + i), f);
+            for (int d = 0; d < 3; ++d) wrap[3 * i + d] = sys.per[d] ? (int)floor(f[d]) : 0;
+        }
+        for (int i = 0; i < n; ++i) {
+            const float* ri = pos + 3 * (a0 + i);
+            for (int j = 0; j < n; ++j) {
+                const float* rj = pos + 3 * (a0 + j);
+                for (int qx = -Q[0]; qx <= Q[0]; ++qx)
+                    for (int qy = -Q[1]; qy <= Q[1]; ++qy)
+                        for (int qz = -Q[2]; qz <= Q[2]; ++qz) {
+                            int S[3];
+                            double d[3];
+                            S[0] = qx - wrap[3 * j + 0] + wrap[3 * i + 0];
+                            S[1] = qy - wrap[3 * j + 1] + wrap[3 * i + 1];
+                            S[2] = qz - wrap[3 * j + 2] + wrap[3 * i + 2];
+                            if (i == j && S[0] == 0 && S[1] == 0 && S[2] == 0) continue;
+                            if (!(orc_pair_d2(ri, rj, S, sys.h, d) < rc2)) continue;
+                            if (half && !orc_half_keep(a0 + i, a0 + j, S)) continue;
+                            if (total < cap) {
+                                int32_t* o = out + 5 * total;
+                                o[0] = a0 + i;
+                                o[1] = a0 + j;
+                                o[2] = S[0];
+                                o[3] = S[1];
+                                o[4] = S[2];
+                            }
+                            ++total;
+                        }
+            }
+        }
+        free(wrap);
+    }
+    return total;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * cell-list neighbor build into the reference's dense layout:
+ *   neighbor_matrix (N,K) int32, rows valid in [0, num_neighbors[i]), the rest = fill (N)
+ *   num_neighbors   (N)   int32, counts keep running past K (overflow signalling)
+ *   shifts          (N,K,3) int32 or NULL
+ * Steps: bin (wrapped fractional coordinates; bounding box on non-periodic axes) ->
+ * histogram -> exclusive scan -> counting-sort scatter -> stencil search with the exact test.
+ * ---------------------------------------------------------------------------------------- */
+static inline int orc_floordiv(int a, int b) {
+    int q = a / b, r = a % b;
+    return (r != 0 && ((r < 0) != (b < 0))) ? q - 1 : q;
+}
+
+ORC_API int32_t orc_nl_cell(const float* pos, const float* cell, const uint8_t* pbc,
+                            const int32_t* batch_ptr, int32_t n_systems, double cutoff,
+                            int32_t half, int32_t K, int32_t n_total, int32_t* nm, int32_t* nn,
+                            int32_t* shifts) {
+    double rc2 = cutoff * cutoff;
+    double rcb = cutoff * (1.0 + 1.0 / 1024.0); /* binning margin: candidates are a superset */
+    for (int64_t t = 0; t < (int64_t)n_total * K; ++t) nm[t] = n_total;
+    if (shifts) memset(shifts, 0, sizeof(int32_t) * 3 * (size_t)n_total * K);
+    memset(nn, 0, sizeof(int32_t) * (size_t)n_total);
+
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int s = 0; s < n_systems; ++s) {
+        orc_sys_t sys;
+        orc_sys_init(&sys, cell ? cell + 9 * s : NULL, pbc ? pbc + 3 * s : NULL);
+        int a0 = batch_ptr[s], a1 = batch_ptr[s + 1];
+        int n = a1 - a0;
+        if (n <= 0) continue;
+        double* fr = (double*)malloc(sizeof(double) * 3 * n);
+        int* wrap = (int*)malloc(sizeof(int) * 3 * n);
+        double lo[3] = {0, 0, 0}, ext[3] = {1, 1, 1};
+        double fmin[3] = {1e300, 1e300, 1e300}, fmax[3] = {-1e300, -1e300, -1e300};
+        for (int i = 0; i < n; ++i) {
+            orc_frac(&sys, pos + 3 * (a0 + i), fr + 3 * i);
+            for (int d = 0; d < 3; ++d) {
+                if (fr[3 * i + d] < fmin[d]) fmin[d] = fr[3 * i + d];
+                if (fr[3 * i + d] > fmax[d]) fmax[d] = fr[3 * i + d];
+            }
+        }
+        int nc[3], R[3];
+        for (int d = 0; d < 3; ++d) {
+            if (!sys.per[d]) {
+                lo[d] = fmin[d];
+                ext[d] = fmax[d] - fmin[d];
+                if (!(ext[d] > 0)) ext[d] = 1e-30;
+            }
+            double span = ext[d] * sys.width[d]; /* perpendicular extent of the binned slab */
+            int c = (int)floor(span / rcb);
+            if (c < 1) c = 1;
+            if (c > 1024) c = 1024;
+            nc[d] = c;
+        }
+        while ((int64_t)nc[0] * nc[1] * nc[2] > (int64_t)(n > 8 ? n : 8)) {
+            int m = 0;
+            if (nc[1] > nc[m]) m = 1;
+            if (nc[2] > nc[m]) m = 2;
+            if (nc[m] == 1) break;
+            nc[m] = (nc[m] + 1) / 2;
+        }
+        for (int d = 0; d < 3; ++d) {
+            double cw = ext[d] * sys.width[d] / nc[d];
+            if (!sys.per[d] && nc[d] == 1) { R[d] = 0; continue; }
+            R[d] = (int)ceil(rcb / cw);
+            if (!sys.per[d] && R[d] > nc[d] - 1) R[d] = nc[d] - 1;
+        }
+        int ncell = nc[0] * nc[1] * nc[2];
+        int* cid = (int*)malloc(sizeof(int) * n);
+        int* start = (int*)calloc((size_t)ncell + 1, sizeof(int));
+        int* order = (int*)malloc(sizeof(int) * n);
+        for (int i = 0; i < n; ++i) {
+            int c[3];
+            for (int d = 0; d < 3; ++d) {
+                double f = fr[3 * i + d];
+                int w = 0;
+                if (sys.per[d]) {
+                    w = (int)floor(f);
+                    f -= (double)w;
+                }
+                wrap[3 * i + d] = w;
+                int b = (int)floor((f - lo[d]) / ext[d] * nc[d]);
+                if (b < 0) b = 0;
+                if (b > nc[d] - 1) b = nc[d] - 1;
+                c[d] = b;
+            }
+            cid[i] = (c[0] * nc[1] + c[1]) * nc[2] + c[2];
+            start[cid[i] + 1]++;
+        }
+        for (int c = 0; c < ncell; ++c) start[c + 1] += start[c];
+        int* fill = (int*)malloc(sizeof(int) * (ncell > 0 ? ncell : 1));
+        memcpy(fill, start, sizeof(int) * ncell);
+        for (int i = 0; i < n; ++i) order[fill[cid[i]]++] = i;
+
+        for (int i = 0; i < n; ++i) {
+            const float* ri = pos + 3 * (a0 + i);
+            int ci = cid[i];
+            int cz = ci % nc[2], cy = (ci / nc[2]) % nc[1], cx = ci / (nc[2] * nc[1]);
+            int count = 0;
+            int32_t* row = nm + (int64_t)(a0 + i) * K;
+            int32_t* srow = shifts ? shifts + (int64_t)(a0 + i) * K * 3 : NULL;
+            for (int ox = -R[0]; ox <= R[0]; ++ox) {
+                int gx = cx + ox, qx = 0;
+                if (sys.per[0]) { qx = orc_floordiv(gx, nc[0]); gx -= qx * nc[0]; }
+                else if (gx < 0 || gx >= nc[0]) continue;
+                for (int oy = -R[1]; oy <= R[1]; ++oy) {
+                    int gy = cy + oy, qy = 0;
+                    if (sys.per[1]) { qy = orc_floordiv(gy, nc[1]); gy -= qy * nc[1]; }
+                    else if (gy < 0 || gy >= nc[1]) continue;
+                    for (int oz = -R[2]; oz <= R[2]; ++oz) {
+                        int gz = cz + oz, qz = 0;
+                        if (sys.per[2]) { qz = orc_floordiv(gz, nc[2]); gz -= qz * nc[2]; }
+                        else if (gz < 0 || gz >= nc[2]) continue;
+                        int c2 = (gx * nc[1] + gy) * nc[2] + gz;
+                        for (int t = start[c2]; t < start[c2 + 1]; ++t) {
+                            int j = order[t];
+                            int S[3];
+                            double d[3];
+                            S[0] = qx - wrap[3 * j + 0] + wrap[3 * i + 0];
+                            S[1] = qy - wrap[3 * j + 1] + wrap[3 * i + 1];
+                            S[2] = qz - wrap[3 * j + 2] + wrap[3 * i + 2];
+                            if (i == j && S[0] == 0 && S[1] == 0 && S[2] == 0) continue;
+                            if (!(orc_pair_d2(ri, pos + 3 * (a0 + j), S, sys.h, d) < rc2))
+                                continue;
+                            if (half && !orc_half_keep(a0 + i, a0 + j, S)) continue;
+                            if (count < K) {
+                                row[count] = a0 + j;
+                                if (srow) {
+                                    srow[3 * count + 0] = S[0];
+                                    srow[3 * count + 1] = S[1];
+                                    srow[3 * count + 2] = S[2];
+                                }
+                            }
+                            ++count;
+                        }
+                    }
+                }
+            }
+            nn[a0 + i] = count;
+        }
+        free(fill); free(order); free(start); free(cid); free(wrap); free(fr);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Lennard-Jones over the dense neighbor matrix.  Pair math in double on the float32 inputs,
+ * one rounding to float32 on output (reference: "Internal math is performed in float64",
+ * nvalchemi/models/_ops/lj.py:49-50).  Plain truncation at the cutoff, no energy shift.
+ *   u(r)  = 4 eps [ (sigma/r)^12 - (sigma/r)^6 ]
+ *   e_i   = 1/2 sum_j u(r_ij)         (full list)   -> atomic_energies (N)
+ *   F_i   = sum_j u'(r_ij) d_ij / r_ij,  d_ij = r_j - r_i + S.cell
+ *   W     = -dE/d(strain) = -1/2 sum_ij u'(r) d (x) d / r   per system, row-major (B,9)
+ *   E_sys = fp64 sum over the system's atoms of the float32-rounded e_i, then cast
+ *           (nvalchemi/models/lj.py:467-477)
+ * Half list: each pair once; e split half/half, force applied to both atoms.
+ * ---------------------------------------------------------------------------------------- */
+ORC_API int32_t orc_lj_matrix(const float* pos, const float* cells, const int32_t* nm,
+                              const int32_t* shifts, const int32_t* nn, const int32_t* batch_idx,
+                              int32_t n_atoms, int32_t K, int32_t n_systems, int32_t fill_value,
+                              double epsilon, double sigma, double cutoff, int32_t half,
+                              float* atomic_energies, float* forces, float* virials,
+                              float* system_energies) {
+    double rc2 = cutoff * cutoff, sig2 = sigma * sigma;
+    double* e = (double*)calloc((size_t)n_atoms, sizeof(double));
+    double* f = (double*)calloc((size_t)n_atoms * 3, sizeof(double));
+    double* w = (double*)calloc((size_t)n_systems * 9, sizeof(double));
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        double h[9];
+        for (int k = 0; k < 9; ++k) h[k] = (double)cells[9 * s + k];
+        int cnt = nn[i] < K ? nn[i] : K;
+        for (int k = 0; k < cnt; ++k) {
+            int j = nm[(int64_t)i * K + k];
+            if (j >= fill_value || j < 0) continue;
+            int S[3] = {0, 0, 0};
+            double d[3];
+            if (shifts) {
+                const int32_t* sp = shifts + ((int64_t)i * K + k) * 3;
+                S[0] = sp[0]; S[1] = sp[1]; S[2] = sp[2];
+            }
+            double r2 = orc_pair_d2(pos + 3 * i, pos + 3 * j, S, h, d);
+            if (!(r2 < rc2)) continue;
+            double ir2 = 1.0 / r2;
+            double s2 = sig2 * ir2, s6 = s2 * s2 * s2, s12 = s6 * s6;
+            double u = 4.0 * epsilon * (s12 - s6);
+            double g = -24.0 * epsilon * (2.0 * s12 - s6) * ir2; /* u'(r)/r */
+            double pf = half ? 1.0 : 0.5;
+            if (half) {
+                e[i] += 0.5 * u;
+                e[j] += 0.5 * u;
+                for (int a = 0; a < 3; ++a) { f[3 * i + a] += g * d[a]; f[3 * j + a] -= g * d[a]; }
+            } else {
+                e[i] += 0.5 * u;
+                for (int a = 0; a < 3; ++a) f[3 * i + a] += g * d[a];
+            }
+            for (int a = 0; a < 3; ++a)
+                for (int b = 0; b < 3; ++b) w[9 * s + 3 * a + b] -= pf * g * d[a] * d[b];
+        }
+    }
+    for (int i = 0; i < n_atoms; ++i) {
+        atomic_energies[i] = (float)e[i];
+        for (int a = 0; a < 3; ++a) forces[3 * i + a] = (float)f[3 * i + a];
+    }
+    if (virials)
+        for (int k = 0; k < 9 * n_systems; ++k) virials[k] = (float)w[k];
+    if (system_energies) {
+        double* acc = (double*)calloc((size_t)n_systems, sizeof(double));
+        for (int i = 0; i < n_atoms; ++i) acc[batch_idx[i]] += (double)atomic_energies[i];
+        for (int s = 0; s < n_systems; ++s) system_energies[s] = (float)acc[s];
+        free(acc);
+    }
+    free(e); free(f); free(w);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * velocity Verlet halves, float32, per-system dt (reference docstrings:
+ *   r(t+dt) = r + v dt + 1/2 (F/m) dt^2 ;  v(t+dt/2) = v + 1/2 (F/m) dt ;  v(t+dt) = v + 1/2 (F'/m) dt)
+ * Association used (each operation rounded once, no fma):
+ *   a = F/m ; vh = v + a*(0.5*dt) ; r' = r + vh*dt
+ * `active` (n_systems bytes or NULL): systems with 0 are left untouched.
+ * ---------------------------------------------------------------------------------------- */
+ORC_API void orc_vv_pre(float* pos, float* vel, const float* forces, const float* masses,
+                        const float* dt, const int32_t* batch_idx, const uint8_t* active,
+                        int32_t n_atoms) {
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float h = dt[s], hh = 0.5f * h, m = masses[i];
+        for (int a = 0; a < 3; ++a) {
+            float acc = forces[3 * i + a] / m;
+            float kick = acc * hh;
+            float vh = vel[3 * i + a] + kick;
+            float dr = vh * h;
+            vel[3 * i + a] = vh;
+            pos[3 * i + a] = pos[3 * i + a] + dr;
+        }
+    }
+}
+
+ORC_API void orc_vv_post(float* vel, const float* forces, const float* masses, const float* dt,
+                         const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms) {
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float hh = 0.5f * dt[s], m = masses[i];
+        for (int a = 0; a < 3; ++a) {
+            float acc = forces[3 * i + a] / m;
+            float kick = acc * hh;
+            vel[3 * i + a] = vel[3 * i + a] + kick;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * FIRE step (vanilla branch).  Reductions vf, vv, ff per system in double at entry, then
+ *   P > 0 : v <- (1-alpha) v + alpha sqrt(vv/ff) F   with the STORED alpha;
+ *           n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max), alpha *= f_alpha
+ *   else  : v <- 0 ; n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
+ *   MD    : v += dt F/m ; dr = dt v ; |dr| > maxstep -> dr *= maxstep/|dr| ; r += dr
+ * Every atom of a system uses the same pre-update scalars.  vf/vv/ff outputs are the
+ * float32-rounded reductions.
+ * ---------------------------------------------------------------------------------------- */
+ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const float* masses,
+                           float* alpha, float* dt, const float* alpha_start,
+                           const float* f_alpha, const float* dt_min, const float* dt_max,
+                           const float* maxstep, int32_t* n_pos, const int32_t* n_min,
+                           const float* f_dec, const float* f_inc, float* vf, float* vv,
+                           float* ff, const int32_t* batch_idx, const uint8_t* active,
+                           int32_t n_atoms, int32_t n_systems) {
+    double* acc = (double*)calloc((size_t)n_systems * 3, sizeof(double));
+    float* mixa = (float*)malloc(sizeof(float) * n_systems);
+    float* mixb = (float*)malloc(sizeof(float) * n_systems);
+    float* dtn = (float*)malloc(sizeof(float) * n_systems);
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        for (int a = 0; a < 3; ++a) {
+            double v = vel[3 * i + a], f = forces[3 * i + a];
+            acc[3 * s + 0] += f * v;
+            acc[3 * s + 1] += v * v;
+            acc[3 * s + 2] += f * f;
+        }
+    }
+    for (int s = 0; s < n_systems; ++s) {
+        double P = acc[3 * s], VV = acc[3 * s + 1], FF = acc[3 * s + 2];
+        vf[s] = (float)P; vv[s] = (float)VV; ff[s] = (float)FF;
+        dtn[s] = dt[s]; mixa[s] = 1.0f; mixb[s] = 0.0f;
+        if (active && !active[s]) continue;
+        if (P > 0.0) {
+            float al = alpha[s];
+            mixa[s] = 1.0f - al;
+            mixb[s] = (FF > 0.0) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
+            n_pos[s] += 1;
+            if (n_pos[s] > n_min[s]) {
+                float nd = dt[s] * f_inc[s];
+                dt[s] = nd < dt_max[s] ? nd : dt_max[s];
+                alpha[s] = al * f_alpha[s];
+            }
+        } else {
+            mixa[s] = 0.0f; mixb[s] = 0.0f;
+            n_pos[s] = 0;
+            float nd = dt[s] * f_dec[s];
+            dt[s] = nd > dt_min[s] ? nd : dt_min[s];
+            alpha[s] = alpha_start[s];
+        }
+        dtn[s] = dt[s];
+    }
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float h = dtn[s], m = masses[i], ms = maxstep[s];
+        float dr[3], v[3];
+        for (int a = 0; a < 3; ++a) {
+            float f = forces[3 * i + a];
+            float vm = (mixa[s] * vel[3 * i + a]) + (mixb[s] * f);
+            float acc1 = f / m;
+            v[a] = vm + (h * acc1);
+            dr[a] = h * v[a];
+        }
+        float n2 = (dr[0] * dr[0] + dr[1] * dr[1]) + dr[2] * dr[2];
+        float nrm = sqrtf(n2);
+        if (nrm > ms) {
+            float sc = ms / nrm;
+            for (int a = 0; a < 3; ++a) dr[a] = dr[a] * sc;
+        }
+        for (int a = 0; a < 3; ++a) {
+            vel[3 * i + a] = v[a];
+            pos[3 * i + a] = pos[3 * i + a] + dr[a];
+        }
+    }
+    free(acc); free(mixa); free(mixb); free(dtn);
+}
+
+/* per-system max over atoms of the float32 force norm (reference: vector_norm then
+ * scatter amax, nvalchemi/dynamics/base.py:266,336-349); systems with no atoms give -inf */
+ORC_API void orc_fmax(const float* forces, const int32_t* batch_idx, int32_t n_atoms,
+                      int32_t n_systems, float* fmax) {
+    for (int s = 0; s < n_systems; ++s) fmax[s] = -INFINITY;
+    for (int i = 0; i < n_atoms; ++i) {
+        const float* f = forces + 3 * i;
+        float n = sqrtf((f[0] * f[0] + f[1] * f[1]) + f[2] * f[2]);
+        int s = batch_idx[i];
+        if (n > fmax[s]) fmax[s] = n;
+    }
+}
+
+ORC_API int32_t orc_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

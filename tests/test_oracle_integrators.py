@@ -1,0 +1,145 @@
+"""Pins the oracle's integrators (CPU only).
+
+Velocity Verlet: literal one-step values from the reference's docstring formulas
+(nvalchemi/dynamics/_ops/velocity_verlet.py:63-64,112), the closed form of the discrete
+harmonic oscillator and time reversibility.  FIRE: hand-worked first steps of the
+restated algorithm and its invariants (dt bounds, counters, descent to the minimum);
+the ordering inside the reference's FIRE kernel is not visible in the reference tree, so
+these checks pin the restatement, not the reference.  fmax: literal cases of
+nvalchemi/dynamics/base.py:304-349.
+"""
+
+import numpy as np
+import pytest
+
+import oracle
+
+
+def test_vv_literal_single_step():
+    r = np.array([[1.0, 0, 0]], dtype=np.float32)
+    v = np.array([[2.0, 0, 0]], dtype=np.float32)
+    F = np.array([[3.0, 0, 0]], dtype=np.float32)
+    m = np.array([4.0], dtype=np.float32)
+    dt = np.array([0.5], dtype=np.float32)
+    oracle.vv_pre(r, v, F, m, dt, [0])
+    # r + v dt + 1/2 (F/m) dt^2 = 1 + 1 + 0.09375 ; v + 1/2 (F/m) dt = 2 + 0.1875
+    assert r[0, 0] == np.float32(2.09375) and v[0, 0] == np.float32(2.1875)
+    oracle.vv_post(v, np.array([[-1.0, 0, 0]], dtype=np.float32), m, dt, [0])
+    assert v[0, 0] == np.float32(2.125)
+
+
+def test_vv_per_system_dt_and_active_mask():
+    r = np.zeros((3, 3), dtype=np.float32)
+    v = np.ones((3, 3), dtype=np.float32)
+    F = np.zeros((3, 3), dtype=np.float32)
+    m = np.ones(3, dtype=np.float32)
+    dt = np.array([0.5, 2.0, 1.0], dtype=np.float32)
+    oracle.vv_pre(r, v, F, m, dt, [0, 1, 2], active=[1, 1, 0])
+    assert np.array_equal(r[:, 0], np.array([0.5, 2.0, 0.0], dtype=np.float32))
+
+
+def test_vv_harmonic_oscillator_closed_form_and_reversibility():
+    k, m0, h, n = 2.0, 1.5, 0.05, 400
+    r = np.array([[1.0, -0.5, 0.25]], dtype=np.float32)
+    v = np.zeros((1, 3), dtype=np.float32)
+    r0 = r.copy()
+    m = np.array([m0], dtype=np.float32)
+    dt = np.array([h], dtype=np.float32)
+    F = (-k * r).astype(np.float32)
+    for _ in range(n):
+        oracle.vv_pre(r, v, F, m, dt, [0])
+        F = (-k * r).astype(np.float32)
+        oracle.vv_post(v, F, m, dt, [0])
+    # velocity Verlet on a harmonic force is a rotation by theta per step, cos(theta) = 1 - (w h)^2/2
+    w2 = k / m0
+    theta = np.arccos(1.0 - w2 * h * h / 2)
+    assert np.allclose(r, r0 * np.cos(n * theta), atol=2e-4)
+    v *= -1
+    for _ in range(n):
+        oracle.vv_pre(r, v, F, m, dt, [0])
+        F = (-k * r).astype(np.float32)
+        oracle.vv_post(v, F, m, dt, [0])
+    assert np.allclose(r, r0, atol=2e-4) and np.abs(v).max() < 2e-4
+
+
+def _fire_state(M, dt=0.1, **kw):
+    f32 = lambda x: np.full(M, x, dtype=np.float32)  # noqa: E731
+    st = dict(alpha=f32(0.1), dt=f32(dt), alpha_start=f32(0.1), f_alpha=f32(0.99),
+              dt_min=f32(0.02 * dt), dt_max=f32(10 * dt), maxstep=f32(0.2), f_dec=f32(0.5),
+              f_inc=f32(1.1), vf=f32(0), vv=f32(0), ff=f32(0),
+              n_steps_positive=np.zeros(M, dtype=np.int32), n_min=np.full(M, 5, dtype=np.int32))
+    for k_, v_ in kw.items():
+        st[k_][:] = v_
+    return st
+
+
+def test_fire_hand_worked_first_two_steps():
+    r = np.zeros((1, 3), dtype=np.float32)
+    v = np.zeros((1, 3), dtype=np.float32)
+    F = np.array([[2.0, 0, 0]], dtype=np.float32)
+    m = np.ones(1, dtype=np.float32)
+    st = _fire_state(1)
+    oracle.fire_step(r, v, F, m, st, [0])
+    # P = 0 is not > 0: dt halves, alpha resets, v zeroed; then v = dt F/m, r += dt v
+    assert st["dt"][0] == np.float32(0.05) and st["n_steps_positive"][0] == 0
+    assert v[0, 0] == pytest.approx(0.1, rel=1e-6) and r[0, 0] == pytest.approx(0.005, rel=1e-6)
+    assert st["vf"][0] == 0 and st["ff"][0] == 4
+    oracle.fire_step(r, v, F, m, st, [0])
+    # P = 0.2 > 0: v <- 0.9*0.1 + 0.1*(0.1/2)*2 = 0.1 ; n+ = 1 <= n_min ; v += 0.05*2 ; r += 0.05*0.2
+    assert st["vf"][0] == pytest.approx(0.2, rel=1e-6) and st["n_steps_positive"][0] == 1
+    assert st["dt"][0] == np.float32(0.05) and st["alpha"][0] == np.float32(0.1)
+    assert v[0, 0] == pytest.approx(0.2, rel=1e-6) and r[0, 0] == pytest.approx(0.015, rel=1e-6)
+
+
+def test_fire_dt_growth_after_n_min_and_caps():
+    r = np.zeros((1, 3), dtype=np.float32)
+    v = np.zeros((1, 3), dtype=np.float32)
+    F = np.array([[1e-3, 0, 0]], dtype=np.float32)
+    m = np.ones(1, dtype=np.float32)
+    st = _fire_state(1, dt=0.1)
+    dts, alphas = [], []
+    for _ in range(60):
+        oracle.fire_step(r, v, F, m, st, [0])
+        dts.append(float(st["dt"][0]))
+        alphas.append(float(st["alpha"][0]))
+    # step 1 shrinks; steps 2..6 are positive steps 1..5 (no growth); growth starts at the 6th
+    assert dts[0] == pytest.approx(0.05) and dts[5] == pytest.approx(0.05)
+    assert dts[6] == pytest.approx(0.05 * 1.1, rel=1e-6) and alphas[6] == pytest.approx(0.099, rel=1e-6)
+    assert max(dts) == pytest.approx(1.0, rel=1e-6)  # dt_max = 10 dt
+    assert all(b >= a for a, b in zip(dts[1:], dts[2:]))
+
+
+def test_fire_maxstep_clamp_is_per_atom():
+    r = np.zeros((2, 3), dtype=np.float32)
+    v = np.zeros((2, 3), dtype=np.float32)
+    F = np.array([[3e4, 4e4, 0], [1e-3, 0, 0]], dtype=np.float32)
+    m = np.ones(2, dtype=np.float32)
+    st = _fire_state(1)
+    oracle.fire_step(r, v, F, m, st, [0, 0])
+    assert np.linalg.norm(r[0]) == pytest.approx(0.2, rel=1e-5)
+    assert r[0, 0] / r[0, 1] == pytest.approx(0.75, rel=1e-5)
+    assert r[1, 0] == pytest.approx(0.05 * 0.05 * 1e-3, rel=1e-5)
+
+
+def test_fire_relaxes_a_quadratic_bowl_and_respects_masks():
+    rng = np.random.default_rng(0)
+    n = 40
+    r = rng.normal(0, 1, (n, 3)).astype(np.float32)
+    v = np.zeros((n, 3), dtype=np.float32)
+    m = rng.uniform(1, 3, n).astype(np.float32)
+    bi = np.repeat(np.arange(4), 10).astype(np.int32)
+    st = _fire_state(4, dt=0.05)
+    frozen = r[bi == 3].copy()
+    active = np.array([1, 1, 1, 0], dtype=np.uint8)
+    for _ in range(300):
+        F = (-1.5 * r).astype(np.float32)
+        oracle.fire_step(r, v, F, m, st, bi, active=active)
+        assert np.all(st["dt"] >= st["dt_min"]) and np.all(st["dt"] <= st["dt_max"])
+    assert np.array_equal(r[bi == 3], frozen)
+    assert oracle.fmax(-1.5 * r, bi, 4)[:3].max() < 1e-3
+
+
+def test_fmax_is_max_atom_force_norm_per_system():
+    F = np.array([[3, 4, 0], [0, 0, 1], [0, 0, 0], [1, 2, 2]], dtype=np.float32)
+    out = oracle.fmax(F, [0, 0, 2, 2], 3)
+    assert out[0] == 5 and out[1] == -np.inf and out[2] == 3
