@@ -1,0 +1,165 @@
+/*
+ * nvalchemi_amd.h -- C ABI of the MI355X (gfx950) batched-MD inner loop.
+ *
+ * One shared library, libnvalchemi_amd.so, exports these entry points.  They are what the
+ * reference's Python binds for this path: the reference reaches its kernels through
+ * torch custom ops and plain calls into an ops wheel; each declaration cites the reference
+ * interface it replaces.  All pointers are DEVICE pointers unless stated otherwise; every
+ * buffer is allocated and owned by the caller; outputs are written in place; work is
+ * enqueued on `stream` (a hipStream_t, NULL = the default stream) and no entry point
+ * synchronises.  Every function returns NVAMD_OK or an error code; nvamd_last_error()
+ * holds a message for the calling thread.  Nothing throws across this boundary.
+ *
+ * Layouts (reference: nvalchemi/neighbors.py:239-266, nvalchemi/models/_ops/lj.py:135-151):
+ *   positions (N,3) f32 | cell (B,3,3) f32, rows = lattice vectors | pbc (B,3) u8 (bool)
+ *   batch_ptr (B+1) i32 | batch_idx (N) i32, non-decreasing
+ *   neighbor_matrix (N,K) i32 padded with N | num_neighbors (N) i32
+ *   neighbor_matrix_shifts (N,K,3) i32, zero in the padding
+ * Pair geometry: r_ij = r_j - r_i + S . cell ; neighbor iff |r_ij|^2 < cutoff^2 (strict),
+ * evaluated in double on the float32 inputs.
+ */
+#ifndef NVALCHEMI_AMD_H
+#define NVALCHEMI_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NVAMD_OK 0
+#define NVAMD_ERR_INVALID_ARGUMENT 1
+#define NVAMD_ERR_WORKSPACE_TOO_SMALL 2
+#define NVAMD_ERR_HIP 3
+#define NVAMD_ERR_UNSUPPORTED 4
+
+#define NVAMD_ABI_VERSION 1
+
+/* Library identification and the last error message of the calling thread. */
+int32_t nvamd_abi_version(void);
+const char* nvamd_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Neighbor list.  Replaces nvalchemiops.torch.neighbors.neighbor_list(...) as called at
+ * nvalchemi/neighbors.py:253-266 and nvalchemi/hooks/neighbor_list.py:328-343, together with
+ * its scratch allocators (allocate_cell_list / estimate_batch_cell_list_sizes,
+ * nvalchemi/hooks/neighbor_list.py:682-704) and the hook's stale-slot masking (:377-380).
+ *
+ * nvamd_nl_workspace_bytes: size of the scratch buffer nvamd_nl_build needs for at most
+ *   n_atoms atoms in n_systems systems (host-only computation, no device access).
+ *
+ * nvamd_nl_build:
+ *   cell, pbc            NULL together = non-periodic (positions are never wrapped).
+ *   rebuild_flags        (B) u8 or NULL; systems with 0 keep their rows and counts.
+ *   max_neighbors        K.  Counting continues past K, nothing is written past K; the
+ *                        caller treats max(num_neighbors) >= K as overflow and retries.
+ *   half_fill            0 = both directions; 1 = each pair once (i<j; self images by the
+ *                        lexicographically positive shift).
+ *   tail_mode            what to do with slots k >= num_neighbors[i] of a rebuilt row:
+ *                        0 = trust that slots beyond the PREVIOUS count already hold the
+ *                            padding (reset only [new, old)); valid for buffers that were
+ *                            prefilled once and are only ever written by this function;
+ *                        1 = write the padding over the whole tail [new, K).
+ *                        num_neighbors must hold the previous counts (zeros at first use).
+ *   neighbor_matrix_shifts may be NULL when cell is NULL.
+ * ---------------------------------------------------------------------------------------- */
+int32_t nvamd_nl_workspace_bytes(int32_t n_atoms, int32_t n_systems, size_t* bytes);
+
+int32_t nvamd_nl_build(const float* positions, const float* cell, const uint8_t* pbc,
+                       const int32_t* batch_ptr, const int32_t* batch_idx,
+                       const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                       double cutoff, int32_t max_neighbors, int32_t half_fill,
+                       int32_t tail_mode, int32_t* neighbor_matrix, int32_t* num_neighbors,
+                       int32_t* neighbor_matrix_shifts, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
+/* Dense -> COO compaction in row-major order (atom ascending, slot ascending).  Replaces
+ * nvalchemiops.torch.neighbors.neighbor_utils.get_neighbor_list_from_neighbor_matrix as
+ * called at nvalchemi/neighbors.py:92-103, in two steps so the caller can size the output:
+ *   nvamd_nl_edge_ptr       edge_ptr (N+1) i32 = exclusive scan of min(num_neighbors, K);
+ *                           edge_ptr[N] = E.  workspace: nvamd_coo_workspace_bytes(n_atoms).
+ *   nvamd_nl_matrix_to_coo  neighbor_list (E_cap,2) i32 rows [i, j]; neighbor_list_shifts
+ *                           (E_cap,3) i32 or NULL; edges at or beyond E_cap are not written.
+ */
+int32_t nvamd_coo_workspace_bytes(int32_t n_atoms, size_t* bytes);
+int32_t nvamd_nl_edge_ptr(const int32_t* num_neighbors, int32_t n_atoms, int32_t max_neighbors,
+                          int32_t* edge_ptr, void* workspace, size_t workspace_bytes,
+                          void* stream);
+int32_t nvamd_nl_matrix_to_coo(const int32_t* neighbor_matrix,
+                               const int32_t* neighbor_matrix_shifts, const int32_t* edge_ptr,
+                               int32_t n_atoms, int32_t max_neighbors, int64_t edge_capacity,
+                               int32_t* neighbor_list, int32_t* neighbor_list_shifts,
+                               void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Lennard-Jones pair kernel over the neighbor matrix.  Replaces the Warp launches inside
+ * nvalchemi::lj_energy_forces_batch and nvalchemi::lj_energy_forces_virial_batch
+ * (nvalchemi/models/_ops/lj.py:116-216, 246-321) and fuses the per-system fp64 energy
+ * scatter of nvalchemi/models/lj.py:467-477.
+ *   neighbor_matrix_shifts NULL = all shifts zero.
+ *   atomic_energies (N) f32, forces (N,3) f32: overwritten.
+ *   virials (B,9) f32 or NULL: W = -sum r_ij (x) F_ij, row-major, overwritten.
+ *   system_energies (B) f32 or NULL: fp64 sum of the float32 atomic energies, overwritten.
+ *   switch_width must be 0 (the C2 switching function is not implemented).
+ *   workspace: nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list).
+ * ---------------------------------------------------------------------------------------- */
+int32_t nvamd_lj_workspace_bytes(int32_t n_atoms, int32_t n_systems, int32_t half_list,
+                                 size_t* bytes);
+
+int32_t nvamd_lj_energy_forces(const float* positions, const float* cells,
+                               const int32_t* neighbor_matrix,
+                               const int32_t* neighbor_matrix_shifts,
+                               const int32_t* num_neighbors, const int32_t* batch_idx,
+                               int32_t n_atoms, int32_t max_neighbors, int32_t n_systems,
+                               int32_t fill_value, double epsilon, double sigma, double cutoff,
+                               double switch_width, int32_t half_list, float* atomic_energies,
+                               float* forces, float* virials, float* system_energies,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Velocity Verlet halves.  Replace nvalchemi::vv_position_update and
+ * nvalchemi::vv_velocity_finalize (nvalchemi/dynamics/_ops/velocity_verlet.py:50-92,102-138).
+ *   dt (M) f32 per system; `active` (M) u8 or NULL: systems with 0 are left untouched (the
+ *   in-kernel form of the save/restore masking of nvalchemi/dynamics/base.py:1849-1891).
+ * ---------------------------------------------------------------------------------------- */
+int32_t nvamd_vv_position_update(float* positions, float* velocities, const float* forces,
+                                 const float* masses, const float* dt, const int32_t* batch_idx,
+                                 const uint8_t* active, int32_t n_atoms, int32_t n_systems,
+                                 void* stream);
+
+int32_t nvamd_vv_velocity_finalize(float* velocities, const float* forces_new,
+                                   const float* masses, const float* dt,
+                                   const int32_t* batch_idx, const uint8_t* active,
+                                   int32_t n_atoms, int32_t n_systems, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * FIRE step.  Replaces nvalchemi::_fire_step_op (nvalchemi/dynamics/_ops/fire.py:79-140).
+ *   All per-system arrays have M entries; alpha, dt, n_steps_positive, vf, vv, ff and
+ *   positions, velocities are updated.  compute_reductions = 0 consumes vf/vv/ff as given.
+ *   uphill_flag is accepted for signature parity; only the vanilla branch exists, entries
+ *   other than 0 are ignored.  `active` as above.
+ *   workspace: nvamd_fire_workspace_bytes(n_systems).
+ * ---------------------------------------------------------------------------------------- */
+int32_t nvamd_fire_workspace_bytes(int32_t n_systems, size_t* bytes);
+
+int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces,
+                        const float* masses, float* alpha, float* dt, const float* alpha_start,
+                        const float* f_alpha, const float* dt_min, const float* dt_max,
+                        const float* maxstep, int32_t* n_steps_positive, const int32_t* n_min,
+                        const float* f_dec, const float* f_inc, const int32_t* uphill_flag,
+                        float* vf, float* vv, float* ff, const int32_t* batch_idx,
+                        int32_t compute_reductions, const uint8_t* active, int32_t n_atoms,
+                        int32_t n_systems, void* workspace, size_t workspace_bytes,
+                        void* stream);
+
+/* Per-system maximum atomic force norm (the default convergence criterion,
+ * nvalchemi/dynamics/base.py:258-349: vector_norm over xyz, scatter amax over atoms).
+ * fmax (M) f32; systems without atoms give -inf. */
+int32_t nvamd_segment_fmax(const float* forces, const int32_t* batch_idx, int32_t n_atoms,
+                           int32_t n_systems, float* fmax, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NVALCHEMI_AMD_H */

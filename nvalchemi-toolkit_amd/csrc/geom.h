@@ -1,0 +1,44 @@
+// Pair geometry shared by the neighbor search and the pair kernel.
+//
+// The separation of atom j (image S) from atom i is defined on the float32 inputs as
+//   d = (r_j - r_i) + (S0*a0 + S1*a1 + S2*a2),   a_k = rows of the cell,
+// evaluated in double with one rounding per operation (no fused multiply-add), in exactly
+// this association.  Both kernels decide "inside the cutoff" from this one expression, so a
+// pair the list holds is a pair the potential sees.
+// Convention: nvalchemi/models/_ops/neighbor_filter.py:98-119 (r_j - r_i + shift . cell,
+// row-vector cell, strict <).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace nvamd {
+
+struct Cell64 {
+    double h[9];
+};
+
+__device__ __forceinline__ double pair_d2_exact(float xi, float yi, float zi, float xj, float yj,
+                                                float zj, int s0, int s1, int s2,
+                                                const double* __restrict__ h, double& d0,
+                                                double& d1, double& d2) {
+#pragma clang fp contract(off)
+    double a = (double)s0, b = (double)s1, c = (double)s2;
+    double tx = (a * h[0] + b * h[3]) + c * h[6];
+    double ty = (a * h[1] + b * h[4]) + c * h[7];
+    double tz = (a * h[2] + b * h[5]) + c * h[8];
+    d0 = ((double)xj - (double)xi) + tx;
+    d1 = ((double)yj - (double)yi) + ty;
+    d2 = ((double)zj - (double)zi) + tz;
+    return (d0 * d0 + d1 * d1) + d2 * d2;
+}
+
+// blockIdx -> logical block so that each of the 8 XCDs (which receive consecutive
+// workgroups round-robin) walks one contiguous eighth of the index space and keeps its
+// own slice of the gathered data in its L2.
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned b, unsigned n_blocks) {
+    constexpr unsigned kXcd = 8;
+    unsigned per = (n_blocks + kXcd - 1) / kXcd;
+    return (b % kXcd) * per + b / kXcd;  // may be >= n_blocks: caller skips
+}
+
+}  // namespace nvamd

@@ -1,0 +1,426 @@
+// Velocity Verlet, FIRE and the per-system max-force reduction for gfx950.
+//
+// All three are pure streaming kernels bounded by HBM bandwidth.  The velocity-Verlet
+// halves treat the (N,3) arrays as flat float streams and move 16 bytes per lane; the
+// per-atom operands (mass, system index, time step) come through the vector L1.
+// Arithmetic is float32 with one rounding per operation (no fused multiply-add) so that
+// results do not depend on how the compiler schedules the expression.
+//
+// Reference interfaces: nvalchemi/dynamics/_ops/velocity_verlet.py:50-138,
+// nvalchemi/dynamics/_ops/fire.py:79-140, nvalchemi/dynamics/base.py:304-349.
+#include "common.h"
+
+#pragma clang fp contract(off)
+
+namespace nvamd {
+namespace {
+
+constexpr int kBlock = 256;
+
+// ---- velocity Verlet ----------------------------------------------------------------------
+// a = F/m ; v(t+dt/2) = v + a*(dt/2) ; r(t+dt) = r + v(t+dt/2)*dt
+__device__ __forceinline__ void vv_pre_elem(float& r, float& v, float f, float m, float h) {
+    float a = f / m;
+    float kick = a * (0.5f * h);
+    float vh = v + kick;
+    float dr = vh * h;
+    v = vh;
+    r = r + dr;
+}
+__device__ __forceinline__ void vv_post_elem(float& v, float f, float m, float h) {
+    float a = f / m;
+    float kick = a * (0.5f * h);
+    v = v + kick;
+}
+
+struct AtomOperands {
+    float m, h;
+    bool on;
+};
+
+__device__ __forceinline__ AtomOperands load_atom(uint32_t atom, const float* __restrict__ masses,
+                                                  const float* __restrict__ dt,
+                                                  const int32_t* __restrict__ bidx,
+                                                  const uint8_t* __restrict__ active) {
+    AtomOperands o;
+    int s = bidx[atom];
+    o.m = masses[atom];
+    o.h = dt[s];
+    o.on = active ? (active[s] != 0) : true;
+    return o;
+}
+
+// One lane owns four consecutive floats of the flat (3N) stream: at most two atoms.
+template <bool PRE>
+__global__ __launch_bounds__(kBlock) void vv_flat_kernel(
+    float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
+    const float* __restrict__ masses, const float* __restrict__ dt,
+    const int32_t* __restrict__ bidx, const uint8_t* __restrict__ active, uint32_t n_elems) {
+    uint32_t t = blockIdx.x * kBlock + threadIdx.x;
+    uint32_t e0 = 4u * t;
+    if (e0 >= n_elems) return;
+    uint32_t a0 = e0 / 3u;
+    uint32_t rem = e0 - 3u * a0;  // position of e0 inside atom a0
+    if (e0 + 4u <= n_elems) {
+        uint32_t a1 = (e0 + 3u) / 3u;
+        AtomOperands o0 = load_atom(a0, masses, dt, bidx, active);
+        AtomOperands o1 = (a1 != a0) ? load_atom(a1, masses, dt, bidx, active) : o0;
+        float4 v4 = reinterpret_cast<const float4*>(vel)[t];
+        float4 f4 = reinterpret_cast<const float4*>(frc)[t];
+        float v[4] = {v4.x, v4.y, v4.z, v4.w};
+        float f[4] = {f4.x, f4.y, f4.z, f4.w};
+        float r[4];
+        if (PRE) {
+            float4 r4 = reinterpret_cast<const float4*>(pos)[t];
+            r[0] = r4.x; r[1] = r4.y; r[2] = r4.z; r[3] = r4.w;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            bool second = (rem + k) >= 3u;
+            const AtomOperands& o = second ? o1 : o0;
+            if (o.on) {
+                if (PRE) vv_pre_elem(r[k], v[k], f[k], o.m, o.h);
+                else vv_post_elem(v[k], f[k], o.m, o.h);
+            }
+        }
+        reinterpret_cast<float4*>(vel)[t] = make_float4(v[0], v[1], v[2], v[3]);
+        if (PRE) reinterpret_cast<float4*>(pos)[t] = make_float4(r[0], r[1], r[2], r[3]);
+    } else {
+        for (uint32_t e = e0; e < n_elems; ++e) {
+            AtomOperands o = load_atom(e / 3u, masses, dt, bidx, active);
+            if (!o.on) continue;
+            if (PRE) vv_pre_elem(pos[e], vel[e], frc[e], o.m, o.h);
+            else vv_post_elem(vel[e], frc[e], o.m, o.h);
+        }
+    }
+}
+
+// Fallback for buffers that are not 16-byte aligned: one lane per float.
+template <bool PRE>
+__global__ __launch_bounds__(kBlock) void vv_scalar_kernel(
+    float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
+    const float* __restrict__ masses, const float* __restrict__ dt,
+    const int32_t* __restrict__ bidx, const uint8_t* __restrict__ active, uint32_t n_elems) {
+    uint32_t e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= n_elems) return;
+    AtomOperands o = load_atom(e / 3u, masses, dt, bidx, active);
+    if (!o.on) return;
+    if (PRE) vv_pre_elem(pos[e], vel[e], frc[e], o.m, o.h);
+    else vv_post_elem(vel[e], frc[e], o.m, o.h);
+}
+
+template <bool PRE>
+int32_t launch_vv(float* pos, float* vel, const float* frc, const float* masses, const float* dt,
+                  const int32_t* bidx, const uint8_t* active, int32_t n_atoms, void* stream) {
+    if (n_atoms < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "n_atoms < 0");
+    if (n_atoms == 0) return NVAMD_OK;
+    if ((PRE && !pos) || !vel || !frc || !masses || !dt || !bidx)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "velocity Verlet: null buffer");
+    if ((int64_t)n_atoms * 3 > 0x7fffffff)
+        return fail(NVAMD_ERR_UNSUPPORTED, "velocity Verlet: more than 2^31/3 atoms");
+    uint32_t n_elems = 3u * (uint32_t)n_atoms;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    bool vec = aligned16(vel) && aligned16(frc) && (!PRE || aligned16(pos));
+    if (vec) {
+        uint32_t n_threads = (n_elems + 3u) / 4u;
+        dim3 grid((n_threads + kBlock - 1) / kBlock);
+        hipLaunchKernelGGL(vv_flat_kernel<PRE>, grid, dim3(kBlock), 0, st, pos, vel, frc, masses, dt,
+                           bidx, active, n_elems);
+    } else {
+        dim3 grid((n_elems + kBlock - 1) / kBlock);
+        hipLaunchKernelGGL(vv_scalar_kernel<PRE>, grid, dim3(kBlock), 0, st, pos, vel, frc, masses,
+                           dt, bidx, active, n_elems);
+    }
+    NVAMD_LAUNCH_CHECK("velocity Verlet launch");
+    return NVAMD_OK;
+}
+
+// ---- segmented wave reductions ------------------------------------------------------------
+// batch_idx is non-decreasing, so inside a wave every system is one run of lanes.  After
+// log2(64) steps the first lane of each run holds the run's total.
+template <int NV>
+__device__ __forceinline__ bool wave_segmented_sum(int seg, double (&v)[NV]) {
+    int lane = lane_id();
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        int seg_up = __shfl_down(seg, o, kWave);
+        bool take = (lane + o < kWave) && (seg_up == seg);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            double up = __shfl_down(v[k], o, kWave);
+            if (take) v[k] += up;
+        }
+    }
+    int seg_prev = __shfl_up(seg, 1, kWave);
+    return lane == 0 || seg_prev != seg;
+}
+
+__device__ __forceinline__ bool wave_segmented_max(int seg, float& v) {
+    int lane = lane_id();
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        int seg_up = __shfl_down(seg, o, kWave);
+        float up = __shfl_down(v, o, kWave);
+        // NaN must win, as it does in a max reduction over the values
+        if ((lane + o < kWave) && (seg_up == seg)) v = (up > v || up != up) ? up : v;
+    }
+    int seg_prev = __shfl_up(seg, 1, kWave);
+    return lane == 0 || seg_prev != seg;
+}
+
+// ---- FIRE -----------------------------------------------------------------------------------
+struct FireScratch {
+    double* acc;   // (M,3): sum F.v, sum v.v, sum F.F
+    float* mix_a;  // (M) factor on v
+    float* mix_b;  // (M) factor on F
+    float* dt_use; // (M) time step of the MD sub-step
+};
+
+__global__ __launch_bounds__(kBlock) void fire_clear_kernel(double* acc, int n) {
+    int t = blockIdx.x * kBlock + threadIdx.x;
+    if (t < n) acc[t] = 0.0;
+}
+
+__global__ __launch_bounds__(kBlock) void fire_reduce_kernel(const float* __restrict__ vel,
+                                                             const float* __restrict__ frc,
+                                                             const int32_t* __restrict__ bidx,
+                                                             double* __restrict__ acc, int n_atoms) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    double v[3] = {0.0, 0.0, 0.0};
+    int seg = -1 - (i - n_atoms);  // distinct negative ids past the end: never merged
+    if (i < n_atoms) {
+        seg = bidx[i];
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            double vv = (double)vel[3 * (size_t)i + a], ff = (double)frc[3 * (size_t)i + a];
+            v[0] += ff * vv;
+            v[1] += vv * vv;
+            v[2] += ff * ff;
+        }
+    }
+    bool head = wave_segmented_sum<3>(seg, v);
+    if (head && i < n_atoms) {
+        atomic_add_f64(acc + 3 * (size_t)seg + 0, v[0]);
+        atomic_add_f64(acc + 3 * (size_t)seg + 1, v[1]);
+        atomic_add_f64(acc + 3 * (size_t)seg + 2, v[2]);
+    }
+}
+
+// caller-supplied vf/vv/ff (compute_reductions = 0): widen them into the accumulator
+__global__ __launch_bounds__(kBlock) void fire_import_kernel(const float* vf, const float* vv,
+                                                             const float* ff, double* acc, int m) {
+    int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    acc[3 * s + 0] = (double)vf[s];
+    acc[3 * s + 1] = (double)vv[s];
+    acc[3 * s + 2] = (double)ff[s];
+}
+
+__global__ __launch_bounds__(kBlock) void fire_params_kernel(
+    float* __restrict__ alpha, float* __restrict__ dt, const float* __restrict__ alpha_start,
+    const float* __restrict__ f_alpha, const float* __restrict__ dt_min,
+    const float* __restrict__ dt_max, int32_t* __restrict__ n_pos, const int32_t* __restrict__ n_min,
+    const float* __restrict__ f_dec, const float* __restrict__ f_inc, float* __restrict__ vf,
+    float* __restrict__ vv, float* __restrict__ ff, const uint8_t* __restrict__ active,
+    FireScratch ws, int write_reductions, int m) {
+    int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+    if (write_reductions) {
+        vf[s] = (float)P;
+        vv[s] = (float)VV;
+        ff[s] = (float)FF;
+    }
+    float h = dt[s];
+    float ma = 1.0f, mb = 0.0f;
+    if (!active || active[s]) {
+        if (P > 0.0) {
+            float al = alpha[s];
+            ma = 1.0f - al;
+            mb = (FF > 0.0) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
+            int np = n_pos[s] + 1;
+            n_pos[s] = np;
+            if (np > n_min[s]) {
+                float nd = h * f_inc[s];
+                float cap = dt_max[s];
+                h = nd < cap ? nd : cap;
+                alpha[s] = al * f_alpha[s];
+            }
+        } else {
+            ma = 0.0f;
+            mb = 0.0f;
+            n_pos[s] = 0;
+            float nd = h * f_dec[s];
+            float lo = dt_min[s];
+            h = nd > lo ? nd : lo;
+            alpha[s] = alpha_start[s];
+        }
+        dt[s] = h;
+    }
+    ws.mix_a[s] = ma;
+    ws.mix_b[s] = mb;
+    ws.dt_use[s] = h;
+}
+
+__global__ __launch_bounds__(kBlock) void fire_update_kernel(
+    float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
+    const float* __restrict__ masses, const float* __restrict__ maxstep,
+    const int32_t* __restrict__ bidx, const uint8_t* __restrict__ active, FireScratch ws,
+    int n_atoms) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_atoms) return;
+    int s = bidx[i];
+    if (active && !active[s]) return;
+    float ma = ws.mix_a[s], mb = ws.mix_b[s], h = ws.dt_use[s], ms = maxstep[s], m = masses[i];
+    size_t b = 3 * (size_t)i;
+    float v[3], dr[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float f = frc[b + a];
+        float vm = (ma * vel[b + a]) + (mb * f);
+        float acc = f / m;
+        v[a] = vm + (h * acc);
+        dr[a] = h * v[a];
+    }
+    float n2 = (dr[0] * dr[0] + dr[1] * dr[1]) + dr[2] * dr[2];
+    float nrm = sqrtf(n2);
+    if (nrm > ms) {
+        float sc = ms / nrm;
+#pragma unroll
+        for (int a = 0; a < 3; ++a) dr[a] = dr[a] * sc;
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        vel[b + a] = v[a];
+        pos[b + a] = pos[b + a] + dr[a];
+    }
+}
+
+// ---- per-system max force norm ------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void fmax_init_kernel(float* fmax, int m) {
+    int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s < m) fmax[s] = -INFINITY;
+}
+
+__global__ __launch_bounds__(kBlock) void fmax_kernel(const float* __restrict__ frc,
+                                                      const int32_t* __restrict__ bidx,
+                                                      float* __restrict__ fmax, int n_atoms) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    int seg = -1 - (i - n_atoms);
+    float nrm = 0.0f;
+    if (i < n_atoms) {
+        seg = bidx[i];
+        size_t b = 3 * (size_t)i;
+        float x = frc[b], y = frc[b + 1], z = frc[b + 2];
+        nrm = sqrtf((x * x + y * y) + z * z);
+    }
+    bool head = wave_segmented_max(seg, nrm);
+    if (head && i < n_atoms) {
+        // norms are >= 0 (or NaN): their bit patterns order like signed integers, and the
+        // bit pattern of -inf is below all of them
+        atomicMax(reinterpret_cast<int*>(fmax) + seg, __float_as_int(nrm));
+    }
+}
+
+}  // namespace
+}  // namespace nvamd
+
+using namespace nvamd;
+
+NVAMD_EXPORT int32_t nvamd_vv_position_update(float* positions, float* velocities,
+                                              const float* forces, const float* masses,
+                                              const float* dt, const int32_t* batch_idx,
+                                              const uint8_t* active, int32_t n_atoms,
+                                              int32_t n_systems, void* stream) {
+    (void)n_systems;
+    return launch_vv<true>(positions, velocities, forces, masses, dt, batch_idx, active, n_atoms,
+                           stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_vv_velocity_finalize(float* velocities, const float* forces_new,
+                                                const float* masses, const float* dt,
+                                                const int32_t* batch_idx, const uint8_t* active,
+                                                int32_t n_atoms, int32_t n_systems, void* stream) {
+    (void)n_systems;
+    return launch_vv<false>(nullptr, velocities, forces_new, masses, dt, batch_idx, active, n_atoms,
+                            stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_fire_workspace_bytes(int32_t n_systems, size_t* bytes) {
+    if (!bytes || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire workspace: bad argument");
+    size_t m = (size_t)(n_systems > 0 ? n_systems : 1);
+    *bytes = align_up(m * 3 * sizeof(double)) + 3 * align_up(m * sizeof(float));
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces,
+                                     const float* masses, float* alpha, float* dt,
+                                     const float* alpha_start, const float* f_alpha,
+                                     const float* dt_min, const float* dt_max, const float* maxstep,
+                                     int32_t* n_steps_positive, const int32_t* n_min,
+                                     const float* f_dec, const float* f_inc,
+                                     const int32_t* uphill_flag, float* vf, float* vv, float* ff,
+                                     const int32_t* batch_idx, int32_t compute_reductions,
+                                     const uint8_t* active, int32_t n_atoms, int32_t n_systems,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    (void)uphill_flag;
+    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire: negative size");
+    if (n_systems == 0) return NVAMD_OK;
+    if (!alpha || !dt || !alpha_start || !f_alpha || !dt_min || !dt_max || !maxstep ||
+        !n_steps_positive || !n_min || !f_dec || !f_inc || !vf || !vv || !ff)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire: null per-system buffer");
+    if (n_atoms > 0 && (!positions || !velocities || !forces || !masses || !batch_idx))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire: null per-atom buffer");
+    size_t need = 0;
+    nvamd_fire_workspace_bytes(n_systems, &need);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "fire: workspace %zu < %zu bytes", workspace_bytes, need);
+    size_t m = (size_t)n_systems;
+    char* w = static_cast<char*>(workspace);
+    FireScratch ws;
+    ws.acc = reinterpret_cast<double*>(w);
+    w += align_up(m * 3 * sizeof(double));
+    ws.mix_a = reinterpret_cast<float*>(w);
+    w += align_up(m * sizeof(float));
+    ws.mix_b = reinterpret_cast<float*>(w);
+    w += align_up(m * sizeof(float));
+    ws.dt_use = reinterpret_cast<float*>(w);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 blk(kBlock);
+    dim3 grid_m((n_systems + kBlock - 1) / kBlock);
+    dim3 grid_n((n_atoms + kBlock - 1) / kBlock);
+    if (compute_reductions) {
+        int n3 = 3 * n_systems;
+        hipLaunchKernelGGL(fire_clear_kernel, dim3((n3 + kBlock - 1) / kBlock), blk, 0, st, ws.acc, n3);
+        if (n_atoms > 0)
+            hipLaunchKernelGGL(fire_reduce_kernel, grid_n, blk, 0, st, velocities, forces, batch_idx,
+                               ws.acc, n_atoms);
+    } else {
+        hipLaunchKernelGGL(fire_import_kernel, grid_m, blk, 0, st, vf, vv, ff, ws.acc, n_systems);
+    }
+    hipLaunchKernelGGL(fire_params_kernel, grid_m, blk, 0, st, alpha, dt, alpha_start, f_alpha, dt_min,
+                       dt_max, n_steps_positive, n_min, f_dec, f_inc, vf, vv, ff, active, ws,
+                       compute_reductions ? 1 : 0, n_systems);
+    if (n_atoms > 0)
+        hipLaunchKernelGGL(fire_update_kernel, grid_n, blk, 0, st, positions, velocities, forces, masses,
+                           maxstep, batch_idx, active, ws, n_atoms);
+    NVAMD_LAUNCH_CHECK("fire launch");
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_segment_fmax(const float* forces, const int32_t* batch_idx,
+                                        int32_t n_atoms, int32_t n_systems, float* fmax,
+                                        void* stream) {
+    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fmax: negative size");
+    if (n_systems == 0) return NVAMD_OK;
+    if (!fmax || (n_atoms > 0 && (!forces || !batch_idx)))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "fmax: null buffer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(fmax_init_kernel, dim3((n_systems + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+                       fmax, n_systems);
+    if (n_atoms > 0)
+        hipLaunchKernelGGL(fmax_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+                           forces, batch_idx, fmax, n_atoms);
+    NVAMD_LAUNCH_CHECK("fmax launch");
+    return NVAMD_OK;
+}

@@ -1,0 +1,408 @@
+// Lennard-Jones energy / force / virial over the dense neighbor matrix, gfx950.
+//
+// Reference interface: nvalchemi::lj_energy_forces_batch and
+// nvalchemi::lj_energy_forces_virial_batch (nvalchemi/models/_ops/lj.py:116-216,246-321),
+// plus the per-system fp64 energy scatter of nvalchemi/models/lj.py:467-477, fused here.
+//
+// Bound: HBM.  Per directed edge the kernel must read the neighbor index (4 B) and the
+// shift (12 B); per atom it reads its position once through the row owner and writes
+// energy and force.  Work decomposition: LPR lanes of a wavefront own one row of the
+// matrix (LPR = 8..64 chosen from the row width), so the row and its shifts are read as
+// contiguous segments, the neighbor positions are gathered through L2 (a system's atoms
+// are contiguous in index space, and workgroups are laid out so that one XCD's L2 serves
+// one contiguous slice of atoms), and the row sum is a shuffle reduction inside the
+// wavefront.  Per-system energy and virial go through one fp64 atomic per run of rows
+// of the same system per workgroup.  Pair math is double on the float32 inputs
+// ("internal math is performed in float64", nvalchemi/models/_ops/lj.py:49-50).
+#include "common.h"
+#include "geom.h"
+
+namespace nvamd {
+namespace {
+
+constexpr int kBlock = 256;
+
+struct LjArgs {
+    const float* pos;
+    const float* cells;
+    const int32_t* nm;
+    const int32_t* shifts;
+    const int32_t* nn;
+    const int32_t* bidx;
+    int32_t n_atoms, K, n_systems, fill;
+    double c4eps, c24eps, sig2, rc2;
+    float* e_atom;
+    float* forces;
+    double* sys_acc;  // (B, 1 + 9): energy then virial, fp64, zeroed before the launch
+    unsigned n_blocks;
+};
+
+template <int LPR>
+__device__ __forceinline__ double group_sum(double v) {
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS>
+__global__ __launch_bounds__(kBlock) void lj_matrix_kernel(LjArgs a) {
+    constexpr int G = kBlock / LPR;  // rows per workgroup
+    __shared__ int s_sys[G];
+    __shared__ double s_val[G][VIRIAL ? 7 : 1];
+
+    unsigned lb = xcd_contiguous_block(blockIdx.x, a.n_blocks);
+    if (lb >= a.n_blocks) return;
+    const int g = threadIdx.x / LPR;
+    const int sub = threadIdx.x % LPR;
+    const int i = (int)(lb * G) + g;
+    const bool row_ok = i < a.n_atoms;
+
+    double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
+    double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;  // xx xy xz yy yz zz
+    int sys = -1 - g;
+    if (row_ok) {
+        sys = a.bidx[i];
+        int cnt = a.nn[i];
+        cnt = cnt < a.K ? cnt : a.K;
+        const float* pi = a.pos + 3 * (size_t)i;
+        const float xi = pi[0], yi = pi[1], zi = pi[2];
+        double h[9];
+        if (SHIFTS) {
+            const float* c = a.cells + 9 * (size_t)sys;
+#pragma unroll
+            for (int k = 0; k < 9; ++k) h[k] = (double)c[k];
+        } else {
+#pragma unroll
+            for (int k = 0; k < 9; ++k) h[k] = 0.0;
+        }
+        const int32_t* row = a.nm + (size_t)i * a.K;
+        const int32_t* srow = SHIFTS ? a.shifts + (size_t)i * a.K * 3 : nullptr;
+        for (int k = sub; k < cnt; k += LPR) {
+            int j = row[k];
+            if (j < 0 || j >= a.fill) continue;
+            int s0 = 0, s1 = 0, s2 = 0;
+            if (SHIFTS) {
+                s0 = srow[3 * k + 0];
+                s1 = srow[3 * k + 1];
+                s2 = srow[3 * k + 2];
+            }
+            const float* pj = a.pos + 3 * (size_t)j;
+            double d0, d1, d2;
+            double r2 = pair_d2_exact(xi, yi, zi, pj[0], pj[1], pj[2], s0, s1, s2, h, d0, d1, d2);
+            if (!(r2 < a.rc2)) continue;
+            double ir2 = 1.0 / r2;
+            double q2 = a.sig2 * ir2;
+            double q6 = q2 * q2 * q2;
+            double q12 = q6 * q6;
+            e += 0.5 * (a.c4eps * (q12 - q6));
+            double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
+            fx += gg * d0;
+            fy += gg * d1;
+            fz += gg * d2;
+            if (VIRIAL) {
+                double hg = -0.5 * gg;
+                w0 += hg * d0 * d0;
+                w1 += hg * d0 * d1;
+                w2 += hg * d0 * d2;
+                w3 += hg * d1 * d1;
+                w4 += hg * d1 * d2;
+                w5 += hg * d2 * d2;
+            }
+        }
+    }
+    e = group_sum<LPR>(e);
+    fx = group_sum<LPR>(fx);
+    fy = group_sum<LPR>(fy);
+    fz = group_sum<LPR>(fz);
+    if (VIRIAL) {
+        w0 = group_sum<LPR>(w0);
+        w1 = group_sum<LPR>(w1);
+        w2 = group_sum<LPR>(w2);
+        w3 = group_sum<LPR>(w3);
+        w4 = group_sum<LPR>(w4);
+        w5 = group_sum<LPR>(w5);
+    }
+    if (sub == 0) {
+        float ef = (float)e;
+        if (row_ok) {
+            a.e_atom[i] = ef;
+            float* fo = a.forces + 3 * (size_t)i;
+            fo[0] = (float)fx;
+            fo[1] = (float)fy;
+            fo[2] = (float)fz;
+        }
+        if (SYS) {
+            s_sys[g] = sys;
+            s_val[g][0] = (double)ef;  // the reference sums the rounded atomic energies
+            if (VIRIAL) {
+                s_val[g][1] = w0; s_val[g][2] = w1; s_val[g][3] = w2;
+                s_val[g][4] = w3; s_val[g][5] = w4; s_val[g][6] = w5;
+            }
+        }
+    }
+    if (SYS) {
+        __syncthreads();
+        // rows of one system are consecutive: the first row of each run adds the run up
+        if (threadIdx.x < G) {
+            int t = threadIdx.x;
+            int s = s_sys[t];
+            bool head = s >= 0 && (t == 0 || s_sys[t - 1] != s);
+            if (head) {
+                constexpr int NV = VIRIAL ? 7 : 1;
+                double acc[NV];
+#pragma unroll
+                for (int k = 0; k < NV; ++k) acc[k] = 0.0;
+                for (int u = t; u < G && s_sys[u] == s; ++u) {
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) acc[k] += s_val[u][k];
+                }
+                double* out = a.sys_acc + 10 * (size_t)s;
+                atomic_add_f64(out + 0, acc[0]);
+                if (VIRIAL) {
+                    atomic_add_f64(out + 1, acc[1]);
+                    atomic_add_f64(out + 2, acc[2]);
+                    atomic_add_f64(out + 3, acc[3]);
+                    atomic_add_f64(out + 5, acc[4]);
+                    atomic_add_f64(out + 6, acc[5]);
+                    atomic_add_f64(out + 9, acc[6]);
+                }
+            }
+        }
+    }
+}
+
+// Half list: each pair once, both atoms updated.  Accumulates in fp64 scratch through
+// atomics; one lane per row.  Not tuned: the reference's LJ default is the full list
+// (nvalchemi/models/lj.py:115).
+struct LjHalfArgs {
+    LjArgs a;
+    double* atom_acc;  // (N,4): e, fx, fy, fz
+};
+
+template <bool VIRIAL, bool SHIFTS>
+__global__ __launch_bounds__(kBlock) void lj_half_kernel(LjHalfArgs p) {
+    const LjArgs& a = p.a;
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.n_atoms) return;
+    int sys = a.bidx[i];
+    int cnt = a.nn[i];
+    cnt = cnt < a.K ? cnt : a.K;
+    const float* pi = a.pos + 3 * (size_t)i;
+    double h[9];
+    const float* c = a.cells + 9 * (size_t)sys;
+    for (int k = 0; k < 9; ++k) h[k] = SHIFTS ? (double)c[k] : 0.0;
+    double e = 0, fx = 0, fy = 0, fz = 0, w[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = 0; k < cnt; ++k) {
+        int j = a.nm[(size_t)i * a.K + k];
+        if (j < 0 || j >= a.fill) continue;
+        int s0 = 0, s1 = 0, s2 = 0;
+        if (SHIFTS) {
+            const int32_t* sp = a.shifts + ((size_t)i * a.K + k) * 3;
+            s0 = sp[0]; s1 = sp[1]; s2 = sp[2];
+        }
+        const float* pj = a.pos + 3 * (size_t)j;
+        double d[3];
+        double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1, s2, h, d[0], d[1], d[2]);
+        if (!(r2 < a.rc2)) continue;
+        double ir2 = 1.0 / r2;
+        double q2 = a.sig2 * ir2, q6 = q2 * q2 * q2, q12 = q6 * q6;
+        double u = a.c4eps * (q12 - q6);
+        double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;
+        e += 0.5 * u;
+        fx += gg * d[0]; fy += gg * d[1]; fz += gg * d[2];
+        double* aj = p.atom_acc + 4 * (size_t)j;
+        atomic_add_f64(aj + 0, 0.5 * u);
+        atomic_add_f64(aj + 1, -gg * d[0]);
+        atomic_add_f64(aj + 2, -gg * d[1]);
+        atomic_add_f64(aj + 3, -gg * d[2]);
+        if (VIRIAL)
+            for (int x = 0; x < 3; ++x)
+                for (int y = 0; y < 3; ++y) w[3 * x + y] -= gg * d[x] * d[y];
+    }
+    double* ai = p.atom_acc + 4 * (size_t)i;
+    atomic_add_f64(ai + 0, e);
+    atomic_add_f64(ai + 1, fx);
+    atomic_add_f64(ai + 2, fy);
+    atomic_add_f64(ai + 3, fz);
+    if (VIRIAL && a.sys_acc)
+        for (int k = 0; k < 9; ++k)
+            if (w[k] != 0.0) atomic_add_f64(a.sys_acc + 10 * (size_t)sys + 1 + k, w[k]);
+}
+
+__global__ __launch_bounds__(kBlock) void lj_half_finish_kernel(const double* __restrict__ atom_acc,
+                                                                const int32_t* __restrict__ bidx,
+                                                                float* __restrict__ e_atom,
+                                                                float* __restrict__ forces,
+                                                                double* __restrict__ sys_acc,
+                                                                int n_atoms) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_atoms) return;
+    const double* ai = atom_acc + 4 * (size_t)i;
+    float ef = (float)ai[0];
+    e_atom[i] = ef;
+    forces[3 * (size_t)i + 0] = (float)ai[1];
+    forces[3 * (size_t)i + 1] = (float)ai[2];
+    forces[3 * (size_t)i + 2] = (float)ai[3];
+    if (sys_acc) atomic_add_f64(sys_acc + 10 * (size_t)bidx[i], (double)ef);
+}
+
+__global__ __launch_bounds__(kBlock) void clear_f64_kernel(double* p, size_t n) {
+    size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t < n) p[t] = 0.0;
+}
+
+__global__ __launch_bounds__(kBlock) void lj_sys_finish_kernel(const double* __restrict__ sys_acc,
+                                                               float* __restrict__ sys_e,
+                                                               float* __restrict__ virials, int m) {
+    int t = blockIdx.x * kBlock + threadIdx.x;
+    if (t >= m * 10) return;
+    int s = t / 10, k = t % 10;
+    double v = sys_acc[t];
+    if (k == 0) {
+        if (sys_e) sys_e[s] = (float)v;
+    } else if (virials) {
+        // the symmetric half was accumulated: mirror it
+        int c = k - 1;
+        int r = c / 3, q = c % 3;
+        if (r > q) v = sys_acc[10 * (size_t)s + 1 + 3 * q + r];
+        virials[9 * (size_t)s + c] = (float)v;
+    }
+}
+
+template <int LPR>
+void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_t st) {
+    constexpr int G = kBlock / LPR;
+    LjArgs b = a;
+    b.n_blocks = (unsigned)((a.n_atoms + G - 1) / G);
+    unsigned per = (b.n_blocks + 7) / 8;
+    dim3 grid(per * 8), blk(kBlock);
+#define NVAMD_LJ_CASE(V, S, Y)                                                          \
+    if (virial == V && shifts == S && sys == Y) {                                       \
+        hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y>), grid, blk, 0, st, b);      \
+        return;                                                                         \
+    }
+    NVAMD_LJ_CASE(false, false, false)
+    NVAMD_LJ_CASE(false, false, true)
+    NVAMD_LJ_CASE(false, true, false)
+    NVAMD_LJ_CASE(false, true, true)
+    NVAMD_LJ_CASE(true, false, true)
+    NVAMD_LJ_CASE(true, true, true)
+#undef NVAMD_LJ_CASE
+}
+
+int lanes_per_row(int K) {
+    static int forced = [] {
+        const char* e = getenv("NVAMD_LJ_LANES_PER_ROW");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced == 8 || forced == 16 || forced == 32 || forced == 64) return forced;
+    if (K <= 16) return 8;
+    if (K <= 256) return 16;
+    return 32;
+}
+
+}  // namespace
+}  // namespace nvamd
+
+using namespace nvamd;
+
+NVAMD_EXPORT int32_t nvamd_lj_workspace_bytes(int32_t n_atoms, int32_t n_systems, int32_t half_list,
+                                              size_t* bytes) {
+    if (!bytes || n_atoms < 0 || n_systems < 0)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj workspace: bad argument");
+    size_t b = align_up((size_t)(n_systems > 0 ? n_systems : 1) * 10 * sizeof(double));
+    if (half_list) b += align_up((size_t)(n_atoms > 0 ? n_atoms : 1) * 4 * sizeof(double));
+    *bytes = b;
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float* cells,
+                                            const int32_t* neighbor_matrix,
+                                            const int32_t* neighbor_matrix_shifts,
+                                            const int32_t* num_neighbors, const int32_t* batch_idx,
+                                            int32_t n_atoms, int32_t max_neighbors,
+                                            int32_t n_systems, int32_t fill_value, double epsilon,
+                                            double sigma, double cutoff, double switch_width,
+                                            int32_t half_list, float* atomic_energies, float* forces,
+                                            float* virials, float* system_energies, void* workspace,
+                                            size_t workspace_bytes, void* stream) {
+    if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
+    if (switch_width != 0.0)
+        return fail(NVAMD_ERR_UNSUPPORTED, "lj: switch_width > 0 (C2 switching) is not implemented");
+    if (n_atoms > 0 && (!positions || !num_neighbors || !batch_idx || !atomic_energies || !forces))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: null per-atom buffer");
+    if (n_atoms > 0 && max_neighbors > 0 && !neighbor_matrix)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: null neighbor matrix");
+    if (neighbor_matrix_shifts && !cells)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: shifts given without cells");
+    size_t need = 0;
+    nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list, &need);
+    const bool want_sys = (virials != nullptr) || (system_energies != nullptr);
+    if ((want_sys || half_list) && (!workspace || workspace_bytes < need))
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "lj: workspace %zu < %zu bytes", workspace_bytes, need);
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    LjArgs a;
+    a.pos = positions;
+    a.cells = cells;
+    a.nm = neighbor_matrix;
+    a.shifts = neighbor_matrix_shifts;
+    a.nn = num_neighbors;
+    a.bidx = batch_idx;
+    a.n_atoms = n_atoms;
+    a.K = max_neighbors;
+    a.n_systems = n_systems;
+    a.fill = fill_value < n_atoms ? fill_value : n_atoms;  // indices at or above are padding
+    a.c4eps = 4.0 * epsilon;
+    a.c24eps = 24.0 * epsilon;
+    a.sig2 = sigma * sigma;
+    a.rc2 = cutoff * cutoff;
+    a.e_atom = atomic_energies;
+    a.forces = forces;
+    a.sys_acc = nullptr;
+    a.n_blocks = 0;
+    const bool shifts = neighbor_matrix_shifts != nullptr;
+    char* w = static_cast<char*>(workspace);
+    if (want_sys && n_systems > 0) {
+        a.sys_acc = reinterpret_cast<double*>(w);
+        size_t n = (size_t)n_systems * 10;
+        hipLaunchKernelGGL(clear_f64_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           st, a.sys_acc, n);
+    }
+    if (n_atoms > 0) {
+        if (half_list) {
+            LjHalfArgs p;
+            p.a = a;
+            p.atom_acc = reinterpret_cast<double*>(
+                w + align_up((size_t)(n_systems > 0 ? n_systems : 1) * 10 * sizeof(double)));
+            size_t n = (size_t)n_atoms * 4;
+            hipLaunchKernelGGL(clear_f64_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock),
+                               0, st, p.atom_acc, n);
+            dim3 grid((n_atoms + kBlock - 1) / kBlock), blk(kBlock);
+            const bool vir = virials != nullptr;
+            if (vir && shifts) hipLaunchKernelGGL((lj_half_kernel<true, true>), grid, blk, 0, st, p);
+            else if (vir) hipLaunchKernelGGL((lj_half_kernel<true, false>), grid, blk, 0, st, p);
+            else if (shifts) hipLaunchKernelGGL((lj_half_kernel<false, true>), grid, blk, 0, st, p);
+            else hipLaunchKernelGGL((lj_half_kernel<false, false>), grid, blk, 0, st, p);
+            hipLaunchKernelGGL(lj_half_finish_kernel, grid, blk, 0, st, p.atom_acc, batch_idx,
+                               atomic_energies, forces, a.sys_acc, n_atoms);
+        } else {
+            const bool vir = virials != nullptr;
+            const bool sys = a.sys_acc != nullptr;
+            switch (lanes_per_row(max_neighbors)) {
+                case 8: launch_full<8>(a, vir, shifts, sys, st); break;
+                case 16: launch_full<16>(a, vir, shifts, sys, st); break;
+                case 32: launch_full<32>(a, vir, shifts, sys, st); break;
+                default: launch_full<64>(a, vir, shifts, sys, st); break;
+            }
+        }
+    }
+    if (want_sys && n_systems > 0) {
+        int n = n_systems * 10;
+        hipLaunchKernelGGL(lj_sys_finish_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+                           a.sys_acc, system_energies, virials, n_systems);
+    }
+    NVAMD_LAUNCH_CHECK("lj launch");
+    return NVAMD_OK;
+}

@@ -1,0 +1,620 @@
+// Batched periodic cell-list neighbor build for gfx950.
+//
+// Reference interface: nvalchemiops.torch.neighbors.neighbor_list as called at
+// nvalchemi/neighbors.py:253-266 and nvalchemi/hooks/neighbor_list.py:328-343 (dense
+// (N,K) matrix + counts + (N,K,3) integer shifts written in place, counting past K as the
+// overflow signal), including the stale-slot masking the hook performs afterwards
+// (nvalchemi/hooks/neighbor_list.py:377-380).
+//
+// Pipeline (all on the caller's stream, no host synchronisation, no allocation):
+//   1 prepare   per system: cell, inverse, periodic flags; clear histogram and bounds
+//   2 bounds    fractional bounding box on non-periodic axes (skipped work for periodic ones)
+//   3 grid      per system: cells per axis (width >= cutoff), stencil radius, cell offsets
+//   4 bin       per atom: wrapped fractional coordinate -> cell, rank inside the cell
+//   5 scan      exclusive scan of the histogram (three small kernels)
+//   6 scatter   counting-sort the atoms into cell order: cell-local coordinates + wrap
+//   7 search    one workgroup per cell: stage the stencil's atoms in LDS, one wavefront per
+//               centre atom, 64 candidates per step, ballot + prefix-popcount compaction
+//               into the atom's row
+//
+// Which pairs are neighbors is decided in double on the original float32 positions
+// (geom.h).  The search classifies candidates with a float32 distance on cell-local
+// coordinates whose rounding error is bounded by a per-system tolerance; only candidates
+// inside that band around the cutoff are re-evaluated exactly, so the list is independent
+// of the order of float32 operations in the fast path.
+#include "common.h"
+#include "geom.h"
+#include "scan.h"
+
+namespace nvamd {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kTile = 1024;       // candidates staged in LDS at a time
+constexpr int kStencilBatch = kBlock; // stencil cells enumerated at a time (one per lane)
+constexpr int kCenterChunk = 256;   // centre atoms of a cell handled per pass
+constexpr int kMaxCellsPerAxis = 1024;
+constexpr int kMinCellCap = 8;    // a system may use at least this many cells
+constexpr int kMaxStencilRadius = 32;  // cells searched per axis and direction, at most
+
+struct NlSys {
+    double h[9];       // rows = lattice vectors (identity without a cell)
+    double hinv[9];    // frac = r . hinv
+    double width[3];   // perpendicular width of the cell along each lattice direction
+    double lo[3];      // lower end of the binned fractional interval
+    double ext[3];     // its length (1 on periodic axes)
+    double step[9];    // row d = (ext[d]/nc[d]) * h[d,:] : one cell step along axis d
+    float tol;         // relative half-width of the float32 uncertainty band on d^2
+    int nc[3];
+    int R[3];
+    int per[3];
+    int cell_offset;
+    int n_cells;
+    int atom_begin, atom_end;
+};
+
+struct NlHeader {
+    int total_cells;
+    int error;  // bit 0: a system's cell is degenerate or narrower than cutoff/kMaxStencilRadius
+    int pad[14];
+};
+
+struct NlWorkspace {
+    NlHeader* hdr;
+    NlSys* sys;
+    uint32_t* bounds;    // (B,6) order keys: min x,y,z then max x,y,z
+    int* cell_offset;    // (B+1)
+    int* atom_cell;      // (N)
+    int* atom_rank;      // (N)
+    int* cell_count;     // (C)
+    int* cell_start;     // (C+1)
+    int* block_sums;     // scan partials
+    float4* sorted_pos;  // (N) cell-local xyz + original index bits
+    int4* sorted_aux;    // (N) wrap integers
+    int max_cells;
+    int n_scan_blocks;
+};
+
+size_t max_cells_for(int n_atoms, int n_systems) {
+    return (size_t)n_atoms + (size_t)kMinCellCap * (size_t)n_systems + 1;
+}
+
+size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
+    size_t N = (size_t)(n_atoms > 0 ? n_atoms : 1), B = (size_t)(n_systems > 0 ? n_systems : 1);
+    size_t C = max_cells_for(n_atoms, n_systems);
+    size_t nsb = (size_t)scan::tiles_for(C);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        size_t o = off;
+        off += align_up(bytes);
+        return base ? base + o : nullptr;
+    };
+    char* p;
+    p = take(sizeof(NlHeader)); if (ws) ws->hdr = reinterpret_cast<NlHeader*>(p);
+    p = take(B * sizeof(NlSys)); if (ws) ws->sys = reinterpret_cast<NlSys*>(p);
+    p = take(B * 6 * sizeof(uint32_t)); if (ws) ws->bounds = reinterpret_cast<uint32_t*>(p);
+    p = take((B + 1) * sizeof(int)); if (ws) ws->cell_offset = reinterpret_cast<int*>(p);
+    p = take(N * sizeof(int)); if (ws) ws->atom_cell = reinterpret_cast<int*>(p);
+    p = take(N * sizeof(int)); if (ws) ws->atom_rank = reinterpret_cast<int*>(p);
+    p = take(C * sizeof(int)); if (ws) ws->cell_count = reinterpret_cast<int*>(p);
+    p = take((C + 1) * sizeof(int)); if (ws) ws->cell_start = reinterpret_cast<int*>(p);
+    p = take((nsb + 1) * sizeof(int)); if (ws) ws->block_sums = reinterpret_cast<int*>(p);
+    p = take(N * sizeof(float4)); if (ws) ws->sorted_pos = reinterpret_cast<float4*>(p);
+    p = take(N * sizeof(int4)); if (ws) ws->sorted_aux = reinterpret_cast<int4*>(p);
+    if (ws) {
+        ws->max_cells = (int)C;
+        ws->n_scan_blocks = (int)nsb;
+    }
+    return off;
+}
+
+struct NlArgs {
+    const float* pos;
+    const float* cell;
+    const uint8_t* pbc;
+    const int32_t* ptr;
+    const int32_t* bidx;
+    const uint8_t* rebuild;
+    int n_atoms, n_systems, K, half, tail_mode;
+    double rc, rc2, rcb;
+    int32_t* nm;
+    int32_t* nn;
+    int32_t* shifts;
+};
+
+__device__ __forceinline__ void inv3(const double* m, double* inv) {
+    double c00 = m[4] * m[8] - m[5] * m[7];
+    double c01 = m[5] * m[6] - m[3] * m[8];
+    double c02 = m[3] * m[7] - m[4] * m[6];
+    double det = m[0] * c00 + m[1] * c01 + m[2] * c02;
+    double id = 1.0 / det;
+    inv[0] = c00 * id;
+    inv[1] = (m[2] * m[7] - m[1] * m[8]) * id;
+    inv[2] = (m[1] * m[5] - m[2] * m[4]) * id;
+    inv[3] = c01 * id;
+    inv[4] = (m[0] * m[8] - m[2] * m[6]) * id;
+    inv[5] = (m[2] * m[3] - m[0] * m[5]) * id;
+    inv[6] = c02 * id;
+    inv[7] = (m[1] * m[6] - m[0] * m[7]) * id;
+    inv[8] = (m[0] * m[4] - m[1] * m[3]) * id;
+}
+
+__device__ __forceinline__ void frac_of(const NlSys& s, const float* __restrict__ r, double* f) {
+    double x = (double)r[0], y = (double)r[1], z = (double)r[2];
+    f[0] = x * s.hinv[0] + y * s.hinv[3] + z * s.hinv[6];
+    f[1] = x * s.hinv[1] + y * s.hinv[4] + z * s.hinv[7];
+    f[2] = x * s.hinv[2] + y * s.hinv[5] + z * s.hinv[8];
+}
+
+// ---- 1 prepare ------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspace ws) {
+    int t = blockIdx.x * kBlock + threadIdx.x;
+    if (t < ws.max_cells) ws.cell_count[t] = 0;
+    if (t == 0) ws.hdr->error = 0;
+    if (t >= a.n_systems) return;
+    NlSys s;
+    const bool has_cell = a.cell != nullptr;
+#pragma unroll
+    for (int k = 0; k < 9; ++k) s.h[k] = has_cell ? (double)a.cell[9 * (size_t)t + k] : ((k % 4 == 0) ? 1.0 : 0.0);
+    inv3(s.h, s.hinv);
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        double nx = s.hinv[d], ny = s.hinv[3 + d], nz = s.hinv[6 + d];
+        s.width[d] = 1.0 / sqrt(nx * nx + ny * ny + nz * nz);
+        s.per[d] = (has_cell && a.pbc) ? (a.pbc[3 * (size_t)t + d] != 0) : 0;
+        s.lo[d] = 0.0;
+        s.ext[d] = 1.0;
+        s.nc[d] = 1;
+        s.R[d] = 0;
+        ws.bounds[6 * (size_t)t + d] = 0xffffffffu;      // min key
+        ws.bounds[6 * (size_t)t + 3 + d] = 0u;           // max key
+    }
+#pragma unroll
+    for (int k = 0; k < 9; ++k) s.step[k] = s.h[k];
+    s.tol = 0.f;
+    s.cell_offset = 0;
+    s.n_cells = 1;
+    s.atom_begin = a.ptr[t];
+    s.atom_end = a.ptr[t + 1];
+    ws.sys[t] = s;
+}
+
+// ---- 2 bounds -------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void nl_bounds_kernel(NlArgs a, NlWorkspace ws) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.n_atoms) return;
+    int sidx = a.bidx[i];
+    const NlSys& s = ws.sys[sidx];
+    if (s.per[0] && s.per[1] && s.per[2]) return;
+    double f[3];
+    frac_of(s, a.pos + 3 * (size_t)i, f);
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        if (s.per[d]) continue;
+        float lo = __double2float_rd(f[d]), hi = __double2float_ru(f[d]);
+        atomicMin(ws.bounds + 6 * (size_t)sidx + d, float_order_key(lo));
+        atomicMax(ws.bounds + 6 * (size_t)sidx + 3 + d, float_order_key(hi));
+    }
+}
+
+// ---- 3 grid ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws) {
+    __shared__ int s_scan[1024];
+    __shared__ int s_carry;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < a.n_systems; base += 1024) {
+        int t = base + threadIdx.x;
+        int ncell = 0;
+        if (t < a.n_systems) {
+            NlSys s = ws.sys[t];
+            int n_at = s.atom_end - s.atom_begin;
+            for (int d = 0; d < 3; ++d) {
+                if (!s.per[d]) {
+                    uint32_t kmin = ws.bounds[6 * (size_t)t + d], kmax = ws.bounds[6 * (size_t)t + 3 + d];
+                    if (kmin <= kmax && n_at > 0) {
+                        double lo = (double)float_from_order_key(kmin), hi = (double)float_from_order_key(kmax);
+                        s.lo[d] = lo;
+                        s.ext[d] = hi - lo;
+                    }
+                    if (!(s.ext[d] > 1e-30)) s.ext[d] = 1e-30;
+                }
+                double span = s.ext[d] * s.width[d];
+                double q = floor(span / a.rcb);
+                int c = (q >= 1.0) ? (q > (double)kMaxCellsPerAxis ? kMaxCellsPerAxis : (int)q) : 1;
+                s.nc[d] = c;
+            }
+            int cap = n_at > kMinCellCap ? n_at : kMinCellCap;
+            while ((long long)s.nc[0] * s.nc[1] * s.nc[2] > (long long)cap) {
+                int m = 0;
+                if (s.nc[1] > s.nc[m]) m = 1;
+                if (s.nc[2] > s.nc[m]) m = 2;
+                if (s.nc[m] == 1) break;
+                s.nc[m] = (s.nc[m] + 1) / 2;
+            }
+            double reach = 0.0;  // largest cell-local coordinate the search can meet
+            for (int d = 0; d < 3; ++d) {
+                double cw = s.ext[d] * s.width[d] / s.nc[d];
+                int R;
+                if (!s.per[d] && s.nc[d] == 1) R = 0;
+                else {
+                    double r = ceil(a.rcb / cw);
+                    if (r >= 1.0 && r <= (double)kMaxStencilRadius) R = (int)r;
+                    else {
+                        R = (r > (double)kMaxStencilRadius) ? kMaxStencilRadius : 1;
+                        if (n_at > 0) atomicOr(&ws.hdr->error, 1);
+                    }
+                    if (!s.per[d] && R > s.nc[d] - 1) R = s.nc[d] - 1;
+                }
+                s.R[d] = R;
+                double sc = s.ext[d] / s.nc[d];
+                double len = 0.0;
+                for (int k = 0; k < 3; ++k) {
+                    s.step[3 * d + k] = sc * s.h[3 * d + k];
+                    len += s.step[3 * d + k] * s.step[3 * d + k];
+                }
+                reach += (R + 1) * sqrt(len);
+            }
+            s.tol = (float)(1.0e-6 * (reach / a.rc + 1.0));
+            s.n_cells = n_at > 0 ? s.nc[0] * s.nc[1] * s.nc[2] : 0;
+            ncell = s.n_cells;
+            ws.sys[t] = s;
+        }
+        // exclusive scan of ncell over the 1024 systems of this pass
+        s_scan[threadIdx.x] = ncell;
+        __syncthreads();
+        for (int o = 1; o < 1024; o <<= 1) {
+            int v = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0;
+            __syncthreads();
+            s_scan[threadIdx.x] += v;
+            __syncthreads();
+        }
+        int incl = s_scan[threadIdx.x];
+        int carry = s_carry;
+        if (t < a.n_systems) {
+            ws.sys[t].cell_offset = carry + incl - ncell;
+            ws.cell_offset[t] = carry + incl - ncell;
+        }
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = carry + incl;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        ws.cell_offset[a.n_systems] = s_carry;
+        ws.hdr->total_cells = s_carry;
+    }
+}
+
+// ---- 4 bin / 6 scatter ----------------------------------------------------------------------
+struct Binned {
+    int cell;      // global cell id
+    int w[3];      // wrap integers (periodic axes)
+    float u[3];    // cartesian offset from the cell's corner
+};
+
+__device__ __forceinline__ Binned bin_atom(const NlSys& s, const float* __restrict__ r) {
+    Binned b;
+    double f[3], g[3];
+    frac_of(s, r, f);
+    int c[3];
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        double fd = f[d];
+        int w = 0;
+        if (s.per[d]) {
+            double fl = floor(fd);
+            fl = fl > 2.0e9 ? 2.0e9 : (fl < -2.0e9 ? -2.0e9 : fl);
+            w = (int)fl;
+            fd -= fl;
+        }
+        b.w[d] = w;
+        double x = (fd - s.lo[d]) / s.ext[d] * (double)s.nc[d];
+        double fx = floor(x);
+        int ci = fx < 0.0 ? 0 : (fx > (double)(s.nc[d] - 1) ? s.nc[d] - 1 : (int)fx);
+        c[d] = ci;
+        g[d] = x - (double)ci;
+    }
+    b.cell = s.cell_offset + (c[0] * s.nc[1] + c[1]) * s.nc[2] + c[2];
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+        b.u[k] = (float)(g[0] * s.step[k] + g[1] * s.step[3 + k] + g[2] * s.step[6 + k]);
+    return b;
+}
+
+__global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.n_atoms) return;
+    const NlSys& s = ws.sys[a.bidx[i]];
+    Binned b = bin_atom(s, a.pos + 3 * (size_t)i);
+    ws.atom_cell[i] = b.cell;
+    ws.atom_rank[i] = atomicAdd(ws.cell_count + b.cell, 1);
+}
+
+__global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspace ws) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= a.n_atoms) return;
+    const NlSys& s = ws.sys[a.bidx[i]];
+    Binned b = bin_atom(s, a.pos + 3 * (size_t)i);
+    int slot = ws.cell_start[b.cell] + ws.atom_rank[i];
+    ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
+    ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
+}
+
+// ---- 7 search -------------------------------------------------------------------------------
+__device__ __forceinline__ int floordiv(int x, int n) {
+    int q = x / n, r = x - q * n;
+    return (r < 0) ? q - 1 : q;
+}
+
+__device__ __forceinline__ bool half_keep(int i, int j, int s0, int s1, int s2) {
+    if (i != j) return i < j;
+    if (s0 != 0) return s0 > 0;
+    if (s1 != 0) return s1 > 0;
+    return s2 > 0;
+}
+
+__global__ __launch_bounds__(kBlock) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
+    __shared__ float4 c_pos[kTile];          // cell-local xyz of a candidate + its atom index
+    __shared__ int4 c_aux[kTile];            // image of its cell minus its own wrap
+    __shared__ int st_start[kStencilBatch];
+    __shared__ int st_prefix[kStencilBatch + 1];
+    __shared__ int st_q[kStencilBatch][3];
+    __shared__ float st_off[kStencilBatch][3];
+    __shared__ int row_cnt[kCenterChunk];    // running row lengths of the centre atoms
+    __shared__ int s_wave[kWavesPerBlock];
+    __shared__ int s_sys;
+
+    const int total_cells = ws.hdr->total_cells;
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const float rc2f = (float)a.rc2;
+    // each XCD (consecutive workgroups go to the 8 XCDs round-robin) walks one contiguous
+    // eighth of the cells, so the stencil data it re-reads stays in its own L2
+    const int xcd = blockIdx.x % 8, slot0 = blockIdx.x / 8, stride = gridDim.x / 8;
+    const int per_xcd = (total_cells + 7) / 8;
+
+    for (int li = slot0; li < per_xcd; li += stride) {
+        // NOTE: every thread of the workgroup takes the same path through this loop body
+        const int c = xcd * per_xcd + li;
+        if (c >= total_cells) break;
+        // system of this cell: last s with cell_offset[s] <= c
+        if (threadIdx.x == 0) {
+            int lo = 0, hi = a.n_systems;  // invariant: offset[lo] <= c < offset[hi]
+            while (hi - lo > 1) {
+                int mid = (lo + hi) >> 1;
+                if (ws.cell_offset[mid] <= c) lo = mid; else hi = mid;
+            }
+            s_sys = lo;
+        }
+        __syncthreads();
+        const int sidx = s_sys;
+        __syncthreads();
+        if (a.rebuild && !a.rebuild[sidx]) continue;
+        const int n_center = ws.cell_count[c];
+        if (n_center == 0) continue;
+        const NlSys& S = ws.sys[sidx];
+        const int c_begin = ws.cell_start[c];
+        const int lc = c - S.cell_offset;
+        const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
+        const int per0 = S.per[0], per1 = S.per[1], per2 = S.per[2];
+        const int cz = lc % nc2, cy = (lc / nc2) % nc1, cx = lc / (nc2 * nc1);
+        const int R0 = S.R[0], R1 = S.R[1], R2 = S.R[2];
+        const int e1 = 2 * R1 + 1, e2 = 2 * R2 + 1;
+        const int n_stencil = (2 * R0 + 1) * e1 * e2;
+        const float tol = S.tol;
+        const float rc2_lo = rc2f * (1.0f - tol), rc2_hi = rc2f * (1.0f + tol);
+
+        for (int cc0 = 0; cc0 < n_center; cc0 += kCenterChunk) {
+            const int n_cc = (n_center - cc0) < kCenterChunk ? (n_center - cc0) : kCenterChunk;
+            for (int k = threadIdx.x; k < n_cc; k += kBlock) row_cnt[k] = 0;
+
+            for (int sb = 0; sb < n_stencil; sb += kStencilBatch) {
+                // ---- enumerate up to kStencilBatch stencil cells, one per lane
+                int my_count = 0;
+                {
+                    int si = sb + (int)threadIdx.x;
+                    int start = 0, q0 = 0, q1 = 0, q2 = 0;
+                    float o0 = 0.f, o1 = 0.f, o2 = 0.f;
+                    if (si < n_stencil) {
+                        int oz = si % e2 - R2, oy = (si / e2) % e1 - R1, ox = si / (e2 * e1) - R0;
+                        int gx = cx + ox, gy = cy + oy, gz = cz + oz;
+                        bool ok = true;
+                        if (per0) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
+                        if (per1) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
+                        if (per2) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
+                        if (ok) {
+                            int c2 = S.cell_offset + (gx * nc1 + gy) * nc2 + gz;
+                            start = ws.cell_start[c2];
+                            my_count = ws.cell_count[c2];
+                            double ddx = (double)ox, ddy = (double)oy, ddz = (double)oz;
+                            o0 = (float)(ddx * S.step[0] + ddy * S.step[3] + ddz * S.step[6]);
+                            o1 = (float)(ddx * S.step[1] + ddy * S.step[4] + ddz * S.step[7]);
+                            o2 = (float)(ddx * S.step[2] + ddy * S.step[5] + ddz * S.step[8]);
+                        }
+                    }
+                    st_start[threadIdx.x] = start;
+                    st_q[threadIdx.x][0] = q0; st_q[threadIdx.x][1] = q1; st_q[threadIdx.x][2] = q2;
+                    st_off[threadIdx.x][0] = o0; st_off[threadIdx.x][1] = o1; st_off[threadIdx.x][2] = o2;
+                }
+                int batch_total;
+                int ex = scan::block_exclusive(my_count, s_wave, batch_total);
+                st_prefix[threadIdx.x] = ex;
+                if (threadIdx.x == 0) st_prefix[kStencilBatch] = batch_total;
+                __syncthreads();
+
+                for (int t0 = 0; t0 < batch_total; t0 += kTile) {
+                    const int tile_n = (batch_total - t0) < kTile ? (batch_total - t0) : kTile;
+                    // ---- stage the tile: candidate -> stencil entry by binary search
+                    for (int k = threadIdx.x; k < tile_n; k += kBlock) {
+                        int flat = t0 + k;
+                        int lo = 0, hi = kStencilBatch;  // prefix[lo] <= flat < prefix[hi]
+                        while (hi - lo > 1) {
+                            int mid = (lo + hi) >> 1;
+                            if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
+                        }
+                        int slot = st_start[lo] + (flat - st_prefix[lo]);
+                        float4 p = ws.sorted_pos[slot];
+                        int4 w = ws.sorted_aux[slot];
+                        p.x += st_off[lo][0];
+                        p.y += st_off[lo][1];
+                        p.z += st_off[lo][2];
+                        c_pos[k] = p;
+                        c_aux[k] = make_int4(st_q[lo][0] - w.x, st_q[lo][1] - w.y, st_q[lo][2] - w.z, 0);
+                    }
+                    __syncthreads();
+
+                    // ---- each wave: its centre atoms against the tile, 64 candidates a step
+                    for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
+                        const float4 ci = ws.sorted_pos[c_begin + cc0 + ca];
+                        const int4 wa = ws.sorted_aux[c_begin + cc0 + ca];
+                        const float xi = ci.x, yi = ci.y, zi = ci.z;
+                        const int i_atom = __float_as_int(ci.w);
+                        int32_t* row = a.nm + (size_t)i_atom * a.K;
+                        int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
+                        int cnt = row_cnt[ca];
+                        for (int k0 = 0; k0 < tile_n; k0 += kWave) {
+                            int k = k0 + lane;
+                            bool in = false;
+                            int j = 0, s0 = 0, s1 = 0, s2 = 0;
+                            if (k < tile_n) {
+                                float4 p = c_pos[k];
+                                float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
+                                float d2 = dx * dx + dy * dy + dz * dz;
+                                if (d2 < rc2_hi) {
+                                    int4 w = c_aux[k];
+                                    j = __float_as_int(p.w);
+                                    s0 = w.x + wa.x; s1 = w.y + wa.y; s2 = w.z + wa.z;
+                                    in = true;
+                                    if (!(d2 < rc2_lo)) {
+                                        // inside the float32 uncertainty band: decide exactly
+                                        const float* pi = a.pos + 3 * (size_t)i_atom;
+                                        const float* pj = a.pos + 3 * (size_t)j;
+                                        double e0, e1d, e2d;
+                                        double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2],
+                                                                  s0, s1, s2, S.h, e0, e1d, e2d);
+                                        in = r2 < a.rc2;
+                                    }
+                                    if (j == i_atom && s0 == 0 && s1 == 0 && s2 == 0) in = false;
+                                    if (a.half && in) in = half_keep(i_atom, j, s0, s1, s2);
+                                }
+                            }
+                            unsigned long long m = __ballot(in);
+                            if (in) {
+                                int slot = cnt + __popcll(m & ((1ull << lane) - 1ull));
+                                if (slot < a.K) {
+                                    row[slot] = j;
+                                    if (srow) {
+                                        srow[3 * slot + 0] = s0;
+                                        srow[3 * slot + 1] = s1;
+                                        srow[3 * slot + 2] = s2;
+                                    }
+                                }
+                            }
+                            cnt += __popcll(m);
+                        }
+                        if (lane == 0) row_cnt[ca] = cnt;
+                    }
+                    __syncthreads();
+                }
+            }
+
+            // ---- counts, and padding over what the previous build left beyond them
+            for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
+                const int i_atom = __float_as_int(ws.sorted_pos[c_begin + cc0 + ca].w);
+                const int cnt = row_cnt[ca];
+                const int old_cnt = a.nn[i_atom];
+                int32_t* row = a.nm + (size_t)i_atom * a.K;
+                int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
+                const int hi_slot = a.tail_mode ? a.K : (old_cnt < a.K ? old_cnt : a.K);
+                for (int k = cnt + lane; k < hi_slot; k += kWave) {
+                    row[k] = a.n_atoms;
+                    if (srow) {
+                        srow[3 * k + 0] = 0;
+                        srow[3 * k + 1] = 0;
+                        srow[3 * k + 2] = 0;
+                    }
+                }
+                if (lane == 0) a.nn[i_atom] = cnt;
+            }
+            __syncthreads();
+        }
+    }
+}
+
+}  // namespace
+}  // namespace nvamd
+
+using namespace nvamd;
+
+NVAMD_EXPORT int32_t nvamd_nl_workspace_bytes(int32_t n_atoms, int32_t n_systems, size_t* bytes) {
+    if (!bytes || n_atoms < 0 || n_systems < 0)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl workspace: bad argument");
+    *bytes = carve(nullptr, nullptr, n_atoms, n_systems);
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, const uint8_t* pbc,
+                                    const int32_t* batch_ptr, const int32_t* batch_idx,
+                                    const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                                    double cutoff, int32_t max_neighbors, int32_t half_fill,
+                                    int32_t tail_mode, int32_t* neighbor_matrix, int32_t* num_neighbors,
+                                    int32_t* neighbor_matrix_shifts, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: negative size");
+    if (!(cutoff > 0.0)) return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: cutoff must be positive");
+    if (n_atoms == 0 || n_systems == 0) return NVAMD_OK;
+    if (!positions || !batch_ptr || !batch_idx || !num_neighbors || (max_neighbors > 0 && !neighbor_matrix))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: null buffer");
+    if ((cell == nullptr) != (pbc == nullptr))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: cell and pbc must be given together");
+    if (cell && !neighbor_matrix_shifts && max_neighbors > 0)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: periodic build needs neighbor_matrix_shifts");
+    size_t need = carve(nullptr, nullptr, n_atoms, n_systems);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "nl: workspace %zu < %zu bytes", workspace_bytes, need);
+    if (max_cells_for(n_atoms, n_systems) > 0x7fffffffull)
+        return fail(NVAMD_ERR_UNSUPPORTED, "nl: too many cells");
+
+    NlWorkspace ws;
+    carve(&ws, static_cast<char*>(workspace), n_atoms, n_systems);
+    NlArgs a;
+    a.pos = positions;
+    a.cell = cell;
+    a.pbc = pbc;
+    a.ptr = batch_ptr;
+    a.bidx = batch_idx;
+    a.rebuild = rebuild_flags;
+    a.n_atoms = n_atoms;
+    a.n_systems = n_systems;
+    a.K = max_neighbors;
+    a.half = half_fill ? 1 : 0;
+    a.tail_mode = tail_mode ? 1 : 0;
+    a.rc = cutoff;
+    a.rc2 = cutoff * cutoff;
+    a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
+    a.nm = neighbor_matrix;
+    a.nn = num_neighbors;
+    a.shifts = neighbor_matrix_shifts;
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    dim3 blk(kBlock);
+    auto blocks = [](size_t n) { return dim3((unsigned)((n + kBlock - 1) / kBlock)); };
+    size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
+    hipLaunchKernelGGL(nl_prepare_kernel, blocks(n_prep), blk, 0, st, a, ws);
+    hipLaunchKernelGGL(nl_bounds_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+    hipLaunchKernelGGL(nl_grid_kernel, dim3(1), dim3(1024), 0, st, a, ws);
+    hipLaunchKernelGGL(nl_bin_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+    scan::exclusive(scan::LoadArray{ws.cell_count}, &ws.hdr->total_cells, 0, ws.n_scan_blocks,
+                    ws.block_sums, ws.cell_start, st);
+    hipLaunchKernelGGL(nl_scatter_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+    // one workgroup per cell; the grid is a fixed size (the cell count lives on the device)
+    // and strides over the cells
+    unsigned n_search = 8u * 2048u;
+    size_t cells_bound = max_cells_for(n_atoms, n_systems);
+    if (cells_bound < n_search) n_search = (unsigned)((cells_bound + 7) / 8 * 8);
+    hipLaunchKernelGGL(nl_search_kernel, dim3(n_search), blk, 0, st, a, ws);
+    NVAMD_LAUNCH_CHECK("neighbor list launch");
+    return NVAMD_OK;
+}

@@ -1,0 +1,282 @@
+"""ctypes binding of ``libnvalchemi_amd.so`` (declared in ``include/nvalchemi_amd.h``).
+
+This module is the only place that touches the C ABI.  It hands raw device pointers,
+sizes and the current HIP stream to the library; tensors are checked here (device, dtype,
+contiguity, shape) because the kernels trust their arguments.  There is no CPU
+implementation behind these functions: a tensor that is not on a ROCm device, or a missing
+library, raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+import torch
+
+_HERE = Path(__file__).resolve().parent
+LIB_PATH = _HERE / "lib" / "libnvalchemi_amd.so"
+
+OK = 0
+_c = ctypes
+_vp = _c.c_void_p
+_i32 = _c.c_int32
+_f64 = _c.c_double
+
+_SIGNATURES = {
+    "nvamd_abi_version": (_i32, []),
+    "nvamd_last_error": (_c.c_char_p, []),
+    "nvamd_nl_workspace_bytes": (_i32, [_i32, _i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_nl_build": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32,
+                              _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_coo_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_nl_edge_ptr": (_i32, [_vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_nl_matrix_to_coo": (_i32, [_vp, _vp, _vp, _i32, _i32, _c.c_int64, _vp, _vp, _vp]),
+    "nvamd_lj_workspace_bytes": (_i32, [_i32, _i32, _i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_lj_energy_forces": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _f64, _f64,
+                                      _f64, _f64, _i32, _vp, _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_vv_position_update": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_vv_velocity_finalize": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_fire_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_fire_step": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
+    "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+class KernelLibraryError(RuntimeError):
+    """The HIP library is missing, or one of its entry points reported an error."""
+
+
+def library() -> ctypes.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise KernelLibraryError(
+                f"{LIB_PATH} not found: build it with `python nvalchemi-toolkit_amd/build.py` "
+                "(there is no fallback implementation)"
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != OK:
+        msg = library().nvamd_last_error().decode(errors="replace")
+        raise KernelLibraryError(f"{what} failed with code {rc}: {msg}")
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str, dtype: torch.dtype, shape: tuple | None = None) -> int:
+    """Validate a tensor the kernels will index blindly and return its device pointer."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if t.device.type != "cuda":
+        raise KernelLibraryError(
+            f"{name}: tensor is on {t.device}; the nvalchemi_amd kernels run on a ROCm device only"
+        )
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected dtype {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: tensor must be contiguous")
+    if shape is not None:
+        if t.dim() != len(shape) or any(e is not None and int(s) != int(e) for s, e in zip(t.shape, shape)):
+            raise ValueError(f"{name}: expected shape {shape}, got {tuple(t.shape)}")
+    return t.data_ptr()
+
+
+def _opt(t, name, dtype, shape=None) -> int | None:
+    return None if t is None else _dev(t, name, dtype, shape)
+
+
+def _as_u8(t: torch.Tensor | None) -> torch.Tensor | None:
+    """bool tensors are passed as bytes (same storage)."""
+    if t is None:
+        return None
+    if t.dtype == torch.bool:
+        return t.view(torch.uint8)
+    return t
+
+
+class _Workspaces:
+    """One growing scratch buffer per (device, purpose); kernels of one purpose run in
+    stream order, so they can share it."""
+
+    def __init__(self) -> None:
+        self._bufs: dict[tuple, torch.Tensor] = {}
+
+    def get(self, device: torch.device, purpose: str, nbytes: int) -> torch.Tensor:
+        key = (device.index, purpose)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+            self._bufs[key] = buf
+        return buf
+
+
+workspaces = _Workspaces()
+
+
+def _size(fn, *args) -> int:
+    out = ctypes.c_size_t(0)
+    _check(fn(*args, ctypes.byref(out)), fn.__name__)
+    return int(out.value)
+
+
+# --------------------------------------------------------------------------------------------
+# neighbor list
+# --------------------------------------------------------------------------------------------
+def nl_workspace_bytes(n_atoms: int, n_systems: int) -> int:
+    return _size(library().nvamd_nl_workspace_bytes, int(n_atoms), int(n_systems))
+
+
+def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, max_neighbors,
+             half_fill, tail_mode, neighbor_matrix, num_neighbors, neighbor_matrix_shifts,
+             workspace: torch.Tensor | None = None) -> None:
+    lib = library()
+    N = positions.shape[0]
+    B = batch_ptr.shape[0] - 1
+    K = int(max_neighbors)
+    p_pos = _dev(positions, "positions", torch.float32, (N, 3))
+    p_cell = _opt(cell, "cell", torch.float32, (B, 3, 3))
+    p_pbc = _opt(_as_u8(pbc), "pbc", torch.uint8, (B, 3))
+    p_ptr = _dev(batch_ptr, "batch_ptr", torch.int32, (B + 1,))
+    p_idx = _dev(batch_idx, "batch_idx", torch.int32, (N,))
+    p_flags = _opt(_as_u8(rebuild_flags), "rebuild_flags", torch.uint8, (B,))
+    p_nm = _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K))
+    p_nn = _dev(num_neighbors, "num_neighbors", torch.int32, (N,))
+    p_sh = _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3))
+    need = nl_workspace_bytes(N, B)
+    ws = workspace if workspace is not None else workspaces.get(positions.device, "nl", need)
+    if ws.device != positions.device or ws.numel() * ws.element_size() < need:
+        raise ValueError("neighbor-list workspace too small or on another device")
+    _check(lib.nvamd_nl_build(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,
+                              int(bool(half_fill)), int(tail_mode), p_nm, p_nn, p_sh, ws.data_ptr(),
+                              ws.numel() * ws.element_size(), _stream(positions.device)),
+           "nvamd_nl_build")
+
+
+def nl_edge_ptr(num_neighbors, max_neighbors, edge_ptr) -> None:
+    lib = library()
+    N = num_neighbors.shape[0]
+    need = _size(lib.nvamd_coo_workspace_bytes, N)
+    ws = workspaces.get(num_neighbors.device, "coo", need)
+    _check(lib.nvamd_nl_edge_ptr(_dev(num_neighbors, "num_neighbors", torch.int32, (N,)), N,
+                                 int(max_neighbors), _dev(edge_ptr, "edge_ptr", torch.int32, (N + 1,)),
+                                 ws.data_ptr(), ws.numel(), _stream(num_neighbors.device)),
+           "nvamd_nl_edge_ptr")
+
+
+def nl_matrix_to_coo(neighbor_matrix, neighbor_matrix_shifts, edge_ptr, neighbor_list,
+                     neighbor_list_shifts) -> None:
+    lib = library()
+    N, K = neighbor_matrix.shape
+    E = neighbor_list.shape[0]
+    _check(lib.nvamd_nl_matrix_to_coo(
+        _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+        _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+        _dev(edge_ptr, "edge_ptr", torch.int32, (N + 1,)), N, K, E,
+        _dev(neighbor_list, "neighbor_list", torch.int32, (E, 2)),
+        _opt(neighbor_list_shifts, "neighbor_list_shifts", torch.int32, (E, 3)),
+        _stream(neighbor_matrix.device)), "nvamd_nl_matrix_to_coo")
+
+
+# --------------------------------------------------------------------------------------------
+# Lennard-Jones
+# --------------------------------------------------------------------------------------------
+def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
+                     batch_idx, fill_value, epsilon, sigma, cutoff, switch_width, half_list,
+                     atomic_energies, forces, virials=None, system_energies=None) -> None:
+    lib = library()
+    N = positions.shape[0]
+    K = neighbor_matrix.shape[1]
+    B = cells.shape[0]
+    need = _size(lib.nvamd_lj_workspace_bytes, N, B, int(bool(half_list)))
+    ws = workspaces.get(positions.device, "lj", need)
+    _check(lib.nvamd_lj_energy_forces(
+        _dev(positions, "positions", torch.float32, (N, 3)),
+        _dev(cells, "cells", torch.float32, (B, 3, 3)),
+        _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+        _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+        _dev(num_neighbors, "num_neighbors", torch.int32, (N,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), float(switch_width),
+        int(bool(half_list)),
+        _dev(atomic_energies, "atomic_energies", torch.float32, (N,)),
+        _dev(forces, "forces", torch.float32, (N, 3)),
+        _opt(virials, "virials", torch.float32, (B, 9)),
+        _opt(system_energies, "system_energies", torch.float32, (B,)),
+        ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces")
+
+
+# --------------------------------------------------------------------------------------------
+# integrators
+# --------------------------------------------------------------------------------------------
+def vv_position_update(positions, velocities, forces, masses, dt, batch_idx, active=None) -> None:
+    N = positions.shape[0]
+    M = dt.shape[0]
+    _check(library().nvamd_vv_position_update(
+        _dev(positions, "positions", torch.float32, (N, 3)),
+        _dev(velocities, "velocities", torch.float32, (N, 3)),
+        _dev(forces, "forces", torch.float32, (N, 3)),
+        _dev(masses, "masses", torch.float32, (N,)),
+        _dev(dt, "dt", torch.float32, (M,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _opt(_as_u8(active), "active", torch.uint8, (M,)),
+        N, M, _stream(positions.device)), "nvamd_vv_position_update")
+
+
+def vv_velocity_finalize(velocities, forces_new, masses, dt, batch_idx, active=None) -> None:
+    N = velocities.shape[0]
+    M = dt.shape[0]
+    _check(library().nvamd_vv_velocity_finalize(
+        _dev(velocities, "velocities", torch.float32, (N, 3)),
+        _dev(forces_new, "forces_new", torch.float32, (N, 3)),
+        _dev(masses, "masses", torch.float32, (N,)),
+        _dev(dt, "dt", torch.float32, (M,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _opt(_as_u8(active), "active", torch.uint8, (M,)),
+        N, M, _stream(velocities.device)), "nvamd_vv_velocity_finalize")
+
+
+def fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_alpha, dt_min, dt_max,
+              maxstep, n_steps_positive, n_min, f_dec, f_inc, uphill_flag, vf, vv, ff, batch_idx,
+              compute_reductions=True, active=None) -> None:
+    lib = library()
+    N = positions.shape[0]
+    M = alpha.shape[0]
+    f32, i32 = torch.float32, torch.int32
+    need = _size(lib.nvamd_fire_workspace_bytes, M)
+    ws = workspaces.get(positions.device, "fire", need)
+    _check(lib.nvamd_fire_step(
+        _dev(positions, "positions", f32, (N, 3)), _dev(velocities, "velocities", f32, (N, 3)),
+        _dev(forces, "forces", f32, (N, 3)), _dev(masses, "masses", f32, (N,)),
+        _dev(alpha, "alpha", f32, (M,)), _dev(dt, "dt", f32, (M,)),
+        _dev(alpha_start, "alpha_start", f32, (M,)), _dev(f_alpha, "f_alpha", f32, (M,)),
+        _dev(dt_min, "dt_min", f32, (M,)), _dev(dt_max, "dt_max", f32, (M,)),
+        _dev(maxstep, "maxstep", f32, (M,)), _dev(n_steps_positive, "n_steps_positive", i32, (M,)),
+        _dev(n_min, "n_min", i32, (M,)), _dev(f_dec, "f_dec", f32, (M,)), _dev(f_inc, "f_inc", f32, (M,)),
+        _dev(uphill_flag, "uphill_flag", i32, (M,)), _dev(vf, "vf", f32, (M,)), _dev(vv, "vv", f32, (M,)),
+        _dev(ff, "ff", f32, (M,)), _dev(batch_idx, "batch_idx", i32, (N,)),
+        int(bool(compute_reductions)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
+        N, M, ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_fire_step")
+
+
+def segment_fmax(forces, batch_idx, fmax) -> None:
+    N = forces.shape[0]
+    M = fmax.shape[0]
+    _check(library().nvamd_segment_fmax(
+        _dev(forces, "forces", torch.float32, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        N, M, _dev(fmax, "fmax", torch.float32, (M,)), _stream(forces.device)), "nvamd_segment_fmax")
