@@ -1,0 +1,103 @@
+"""The neighbor functions the reference imports from its ops wheel, backed by the HIP
+library: ``neighbor_list`` (nvalchemi/neighbors.py:253-266,
+nvalchemi/hooks/neighbor_list.py:328-343), ``estimate_max_neighbors``
+(nvalchemi/neighbors.py:228) and ``get_neighbor_list_from_neighbor_matrix``
+(nvalchemi/neighbors.py:92-103).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+_METHODS = {None, "naive", "cell_list", "batch_naive", "batch_cell_list", "batch_cell_list_pair_centric",
+            "batch_cluster_tile", "cluster_tile", "naive_tile"}
+
+
+def ceil16(n: int) -> int:
+    return ((int(n) + 15) // 16) * 16
+
+
+def estimate_max_neighbors(cutoff: float, atomic_density: float = 0.2, safety_factor: float = 1.5) -> int:
+    """Row width guess: atoms in the cutoff sphere at ``atomic_density``, times a safety
+    factor, rounded up to 16.  Only the buffer width depends on it, never the list: callers
+    grow on overflow and trim on over-estimate."""
+    expected = atomic_density * (4.0 / 3.0) * math.pi * float(cutoff) ** 3
+    return max(16, ceil16(math.ceil(safety_factor * expected)))
+
+
+def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | None = None,
+                  pbc: torch.Tensor | None = None, max_neighbors: int | None = None,
+                  half_fill: bool = False, batch_ptr: torch.Tensor | None = None,
+                  batch_idx: torch.Tensor | None = None, neighbor_matrix: torch.Tensor | None = None,
+                  num_neighbors: torch.Tensor | None = None,
+                  neighbor_matrix_shifts: torch.Tensor | None = None,
+                  rebuild_flags: torch.Tensor | None = None, method: str | None = None,
+                  tail_mode: int = 1, **scratch) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+    """Build the dense neighbor list in place and return ``(neighbor_matrix, num_neighbors,
+    neighbor_matrix_shifts)``.
+
+    ``neighbor_matrix (N,K)`` int32 must arrive padded with ``N`` (or hold a previous
+    result), ``num_neighbors (N)`` int32 zeroed (or the previous counts); they are allocated
+    when ``None``.  ``num_neighbors`` keeps counting past ``K``: ``max >= K`` means overflow.
+    ``cell``/``pbc`` ``None`` means non-periodic.  ``rebuild_flags (B) bool``: systems with
+    ``False`` keep their rows.  ``method`` is accepted for compatibility (one cell-list
+    kernel serves every case); scratch keyword tensors of the reference's strategies are
+    ignored.  ``tail_mode=1`` rewrites the padding of every rebuilt row; ``0`` only clears
+    what the previous build left (persistent buffers that only this function writes).
+    """
+    if method not in _METHODS:
+        raise ValueError(f"unknown neighbor list method {method!r}")
+    if positions.dtype != torch.float32:
+        raise NotImplementedError("the HIP neighbor list takes float32 positions")
+    N = positions.shape[0]
+    dev = positions.device
+    if batch_ptr is None:
+        batch_ptr = torch.tensor([0, N], dtype=torch.int32, device=dev)
+    if batch_idx is None:
+        B = batch_ptr.shape[0] - 1
+        batch_idx = torch.repeat_interleave(torch.arange(B, dtype=torch.int32, device=dev),
+                                            (batch_ptr[1:] - batch_ptr[:-1]).to(torch.long), output_size=N)
+    B = batch_ptr.shape[0] - 1
+    if (cell is None) != (pbc is None):
+        if cell is None:
+            pbc = None
+        else:
+            pbc = torch.zeros(B, 3, dtype=torch.bool, device=dev)
+    if cell is not None:
+        cell = cell.to(torch.float32).reshape(B, 3, 3).contiguous()
+        pbc = pbc.reshape(B, 3).contiguous()
+    K = int(max_neighbors if max_neighbors is not None else
+            (neighbor_matrix.shape[1] if neighbor_matrix is not None else estimate_max_neighbors(cutoff)))
+    if neighbor_matrix is None:
+        neighbor_matrix = torch.full((N, K), N, dtype=torch.int32, device=dev)
+    if num_neighbors is None:
+        num_neighbors = torch.zeros(N, dtype=torch.int32, device=dev)
+    if neighbor_matrix_shifts is None and cell is not None:
+        neighbor_matrix_shifts = torch.zeros((N, K, 3), dtype=torch.int32, device=dev)
+    _lib.nl_build(positions.contiguous(), cell, pbc, batch_ptr.to(torch.int32).contiguous(),
+                  batch_idx.to(torch.int32).contiguous(), rebuild_flags, cutoff, K, half_fill, tail_mode,
+                  neighbor_matrix, num_neighbors, neighbor_matrix_shifts if cell is not None else None)
+    return neighbor_matrix, num_neighbors, neighbor_matrix_shifts
+
+
+def get_neighbor_list_from_neighbor_matrix(neighbor_matrix: torch.Tensor, num_neighbors: torch.Tensor,
+                                           neighbor_shift_matrix: torch.Tensor | None = None,
+                                           fill_value: int | None = None):
+    """Dense -> COO in row-major order.  Returns ``(edges (2,E) int32, edge_ptr (N+1) int32[,
+    shifts (E,3) int32])`` like the reference's helper (the caller transposes ``[0]``).
+    Reads back one integer (the edge count) to size the output."""
+    N, K = neighbor_matrix.shape
+    dev = neighbor_matrix.device
+    edge_ptr = torch.empty(N + 1, dtype=torch.int32, device=dev)
+    _lib.nl_edge_ptr(num_neighbors, K, edge_ptr)
+    E = int(edge_ptr[-1].item())
+    edges = torch.empty((E, 2), dtype=torch.int32, device=dev)
+    shifts = torch.empty((E, 3), dtype=torch.int32, device=dev) if neighbor_shift_matrix is not None else None
+    _lib.nl_matrix_to_coo(neighbor_matrix, neighbor_shift_matrix, edge_ptr, edges, shifts)
+    if shifts is None:
+        return edges.T, edge_ptr
+    return edges.T, edge_ptr, shifts

@@ -1,0 +1,69 @@
+"""Torch custom op and public wrapper for the FIRE step.
+
+Same schema and mutation set as ``nvalchemi::_fire_step_op`` and the same public
+``fire_step`` signature (nvalchemi/dynamics/_ops/fire.py:79-140,245-362).  Per system, with
+the reductions ``vf = sum F.v``, ``vv = sum v.v``, ``ff = sum F.F`` taken at entry:
+
+    vf > 0 : v <- (1-alpha) v + alpha sqrt(vv/ff) F        (alpha as stored)
+             n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max) ; alpha *= f_alpha
+    else   : v <- 0 ; n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
+    then   : v += dt F/m ; dr = dt v ; |dr| > maxstep -> dr *= maxstep/|dr| ; r += dr
+
+All atoms of a system see the same pre-update scalars.  Only the vanilla branch exists:
+``uphill_flag`` entries are ignored by the kernel (the ``FIRE`` class refuses ``uphill``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ... import _lib
+
+__all__ = ["fire_step"]
+
+
+@torch.library.custom_op(
+    "nvalchemi_amd::_fire_step_op",
+    mutates_args={"positions", "velocities", "alpha", "dt", "n_steps_positive", "vf", "vv", "ff"},
+)
+def _fire_step_op(positions: torch.Tensor, velocities: torch.Tensor, forces: torch.Tensor,
+                  masses: torch.Tensor, alpha: torch.Tensor, dt: torch.Tensor, alpha_start: torch.Tensor,
+                  f_alpha: torch.Tensor, dt_min: torch.Tensor, dt_max: torch.Tensor, maxstep: torch.Tensor,
+                  n_steps_positive: torch.Tensor, n_min: torch.Tensor, f_dec: torch.Tensor,
+                  f_inc: torch.Tensor, uphill_flag: torch.Tensor, vf: torch.Tensor, vv: torch.Tensor,
+                  ff: torch.Tensor, batch_idx: torch.Tensor, compute_reductions: bool = True) -> None:
+    _lib.fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_alpha, dt_min, dt_max,
+                   maxstep, n_steps_positive, n_min, f_dec, f_inc, uphill_flag, vf, vv, ff, batch_idx,
+                   compute_reductions)
+
+
+@_fire_step_op.register_fake
+def _(positions, velocities, forces, masses, alpha, dt, alpha_start, f_alpha, dt_min, dt_max, maxstep,
+      n_steps_positive, n_min, f_dec, f_inc, uphill_flag, vf, vv, ff, batch_idx,
+      compute_reductions=True) -> None:
+    pass
+
+
+def fire_step(positions: torch.Tensor, velocities: torch.Tensor, forces: torch.Tensor,
+              masses: torch.Tensor, alpha: torch.Tensor, dt: torch.Tensor, n_steps_positive: torch.Tensor,
+              alpha_start: torch.Tensor, f_alpha: torch.Tensor, dt_min: torch.Tensor, dt_max: torch.Tensor,
+              maxstep: torch.Tensor, n_min: torch.Tensor, f_dec: torch.Tensor, f_inc: torch.Tensor,
+              uphill_flag: torch.Tensor, *, vf: torch.Tensor | None = None, vv: torch.Tensor | None = None,
+              ff: torch.Tensor | None = None, batch_idx: torch.Tensor | None = None,
+              compute_reductions: bool = True, active: torch.Tensor | None = None) -> None:
+    """Full FIRE step; mutates positions, velocities, alpha, dt, n_steps_positive (and the
+    scratch ``vf``/``vv``/``ff``, allocated when ``None``).  ``active [M] bool`` (extension):
+    systems with ``False`` are left untouched."""
+    M = alpha.shape[0]
+    dtype, device = positions.dtype, positions.device
+    if vf is None:
+        vf = torch.zeros(M, dtype=dtype, device=device)
+    if vv is None:
+        vv = torch.zeros(M, dtype=dtype, device=device)
+    if ff is None:
+        ff = torch.zeros(M, dtype=dtype, device=device)
+    if batch_idx is None:
+        batch_idx = torch.zeros(positions.shape[0], dtype=torch.int32, device=device)
+    _lib.fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_alpha, dt_min, dt_max,
+                   maxstep, n_steps_positive, n_min, f_dec, f_inc, uphill_flag, vf, vv, ff, batch_idx,
+                   compute_reductions, active)

@@ -1,0 +1,366 @@
+"""The dynamics step contract.
+
+Mirror of nvalchemi/dynamics/base.py for the single-process path: ``DynamicsStage``
+(:120-157), ``_ConvergenceCriterion`` (:180-349), ``ConvergenceHook`` (:2215-2501),
+``BaseDynamics.step/compute/run`` (:1815-1955).  One step is
+
+    BEFORE_STEP -> BEFORE_PRE_UPDATE -> pre_update -> AFTER_PRE_UPDATE -> BEFORE_COMPUTE ->
+    compute (= model(batch), outputs copied into the batch's existing energy/forces/stress)
+    -> AFTER_COMPUTE -> BEFORE_POST_UPDATE -> post_update -> AFTER_POST_UPDATE -> AFTER_STEP
+    -> convergence check (-> ON_CONVERGE) -> step_count += 1
+
+The first step integrates with whatever ``batch.forces`` holds: ``run`` does not prime
+forces.  Systems with ``status >= exit_status`` keep positions, velocities and cell through
+a step; integrators that set ``_honors_active_mask`` get the mask (``self._active_mask``)
+and skip those systems inside their kernels, everything else is saved and restored around
+the update as the reference does.
+"""
+
+from __future__ import annotations
+
+from collections import OrderedDict
+from enum import Enum
+from typing import Any, Callable, Literal
+
+import torch
+from pydantic import BaseModel, ConfigDict
+
+from .. import _lib
+from ..hooks._context import DynamicsContext
+from ..hooks._registry import HookRegistryMixin
+from ..models.base import BaseModelMixin
+
+
+class DynamicsStage(Enum):
+    BEFORE_STEP = 0
+    BEFORE_PRE_UPDATE = 1
+    AFTER_PRE_UPDATE = 2
+    BEFORE_COMPUTE = 3
+    AFTER_COMPUTE = 4
+    BEFORE_POST_UPDATE = 5
+    AFTER_POST_UPDATE = 6
+    AFTER_STEP = 7
+    ON_CONVERGE = 8
+
+
+class _ConvergenceCriterion(BaseModel):
+    """One criterion on a batch key: optional reduction inside each entry (``reduce_op`` over
+    ``reduce_dims``), node-level values reduced per graph with max, then ``<= threshold``."""
+
+    model_config = ConfigDict(arbitrary_types_allowed=True)
+
+    key: str
+    threshold: float
+    reduce_dims: int | list[int] = -1
+    reduce_op: Literal["min", "max", "norm", "mean", "sum"] | None = None
+    custom_op: Callable[[torch.Tensor], torch.Tensor] | None = None
+
+    def _reduce_within_entry(self, target: torch.Tensor) -> torch.Tensor:
+        if self.reduce_op is None:
+            return target
+        if self.reduce_op == "min":
+            return torch.amin(target, self.reduce_dims)
+        if self.reduce_op == "max":
+            return torch.amax(target, self.reduce_dims)
+        if self.reduce_op == "norm":
+            return torch.linalg.vector_norm(target, dim=self.reduce_dims)
+        if self.reduce_op == "mean":
+            return torch.mean(target, dim=self.reduce_dims)
+        if self.reduce_op == "sum":
+            return torch.sum(target, dim=self.reduce_dims)
+        raise ValueError(f"Unknown reduce_op: {self.reduce_op!r}")
+
+    @staticmethod
+    def _scatter_reduce_to_graph(values: torch.Tensor, batch_idx: torch.Tensor, num_graphs: int) -> torch.Tensor:
+        out = torch.full((num_graphs,), float("-inf"), dtype=values.dtype, device=values.device)
+        out.scatter_reduce_(0, batch_idx.to(torch.long), values, reduce="amax", include_self=False)
+        return out
+
+    def _is_force_norm(self, target: torch.Tensor, batch) -> bool:
+        return (self.reduce_op == "norm" and self.reduce_dims in (-1, 1) and target.dim() == 2
+                and target.shape[1] == 3 and target.dtype == torch.float32 and target.is_cuda
+                and target.shape[0] == batch.num_nodes and batch.num_nodes != batch.num_graphs)
+
+    def __call__(self, batch) -> torch.Tensor:
+        target = getattr(batch, self.key, None)
+        if target is None:
+            raise KeyError("Key for convergence check not found;"
+                           f" expected={self.key!r}, available={list(batch.keys())}")
+        if self.custom_op is not None:
+            return self.custom_op(target)
+        if self._is_force_norm(target, batch):
+            # per-system max of the atomic force norms in one pass
+            fmax = torch.empty(batch.num_graphs, dtype=torch.float32, device=target.device)
+            _lib.segment_fmax(target.contiguous(), batch.batch_idx, fmax)
+            return fmax <= self.threshold
+        target = self._reduce_within_entry(target)
+        is_node_level = target.shape[0] == batch.num_nodes and batch.num_nodes != batch.num_graphs
+        if is_node_level:
+            if target.dim() > 1:
+                target = target.view(target.shape[0], -1).amax(dim=-1)
+            reduced = self._scatter_reduce_to_graph(target, batch.batch_idx, batch.num_graphs)
+        else:
+            reduced = target.squeeze(-1) if target.dim() == 2 else target
+        return reduced <= self.threshold
+
+
+class ConvergenceHook:
+    """AND of one or more criteria; optionally migrates ``batch.status`` of converged systems
+    from ``source_status`` to ``target_status``."""
+
+    def __init__(self, criteria=None, source_status: int | None = None, target_status: int | None = None,
+                 frequency: int = 1) -> None:
+        self.frequency = frequency
+        self.stage = DynamicsStage.AFTER_STEP
+        self.source_status = source_status
+        self.target_status = target_status
+        if criteria is None:
+            self.criteria = [_ConvergenceCriterion(key="forces", threshold=0.05, reduce_op="norm", reduce_dims=-1)]
+        elif isinstance(criteria, _ConvergenceCriterion):
+            self.criteria = [criteria]
+        elif isinstance(criteria, dict):
+            self.criteria = [_ConvergenceCriterion(**criteria)]
+        elif isinstance(criteria, (list, tuple)):
+            normalized = []
+            for item in criteria:
+                if isinstance(item, dict):
+                    normalized.append(_ConvergenceCriterion(**item))
+                elif isinstance(item, _ConvergenceCriterion):
+                    normalized.append(item)
+                else:
+                    raise TypeError("Each criterion must be a dict or _ConvergenceCriterion, "
+                                    f"got {type(item).__name__}")
+            self.criteria = normalized
+        else:
+            raise TypeError("criteria must be a dict, _ConvergenceCriterion, or list thereof, "
+                            f"got {type(criteria).__name__}")
+
+    @classmethod
+    def from_fmax(cls, threshold: float = 0.05, source_status: int | None = None,
+                  target_status: int | None = None, frequency: int = 1) -> "ConvergenceHook":
+        return cls.from_forces(threshold=threshold, frequency=frequency, source_status=source_status,
+                               target_status=target_status)
+
+    @classmethod
+    def from_forces(cls, threshold: float, frequency: int = 1, source_status: int | None = None,
+                    target_status: int | None = None) -> "ConvergenceHook":
+        return cls(criteria=[{"key": "forces", "threshold": threshold, "reduce_op": "norm", "reduce_dims": -1}],
+                   frequency=frequency, source_status=source_status, target_status=target_status)
+
+    @property
+    def num_criteria(self) -> int:
+        return len(self.criteria)
+
+    def converged_mask(self, batch) -> torch.Tensor:
+        """Boolean ``(B,)`` mask (no host synchronisation)."""
+        mask = self.criteria[0](batch)
+        for c in self.criteria[1:]:
+            mask = mask & c(batch)
+        return mask
+
+    def evaluate(self, batch) -> torch.Tensor | None:
+        """Indices of systems that satisfy every criterion, or ``None``."""
+        mask = self.converged_mask(batch)
+        idx = torch.where(mask)[0]
+        return idx if idx.numel() > 0 else None
+
+    def __call__(self, ctx: DynamicsContext, stage: Enum) -> None:
+        batch = ctx.batch
+        if self.source_status is None or self.target_status is None:
+            return
+        if not hasattr(batch, "status") or batch.status is None:
+            return
+        mask = self.converged_mask(batch)
+        flat = batch.status.view(-1)
+        migrate = mask & (flat[: mask.shape[0]] == self.source_status)
+        flat[: mask.shape[0]] = torch.where(migrate, torch.full_like(flat[: mask.shape[0]], self.target_status),
+                                            flat[: mask.shape[0]])
+
+
+class BaseDynamics(HookRegistryMixin):
+    """Coordinates a model with an integrator over a ``Batch``.
+
+    Subclasses override ``pre_update`` / ``post_update`` (and ``_init_state`` for per-system
+    state) and declare ``__needs_keys__`` / ``__provides_keys__``.
+    """
+
+    _stage_type = DynamicsStage
+    __needs_keys__: set[str] = set()
+    __provides_keys__: set[str] = set()
+    _mutable_fields: tuple[str, ...] = ("positions", "velocities", "cell")
+    _honors_active_mask: bool = False
+    _OUTPUT_KEY_TO_BATCH_ATTR: dict[str, str] = {"energy": "energy", "forces": "forces", "stress": "stress"}
+
+    def __init__(self, model: BaseModelMixin, hooks: list | None = None, convergence_hook: Any = None,
+                 n_steps: int | None = None, exit_status: int = 1, **kwargs: Any) -> None:
+        if not isinstance(model, BaseModelMixin):
+            raise TypeError(f"Expected a `BaseModelMixin` instance, got {type(model).__name__}."
+                            " Please wrap your model with a `BaseModelMixin` subclass.")
+        self.model = model
+        self.step_count = 0
+        if isinstance(convergence_hook, dict):
+            convergence_hook = ConvergenceHook(**convergence_hook)
+        self.convergence_hook = convergence_hook
+        self.n_steps = n_steps
+        self.exit_status = exit_status
+        self.model_config = model.model_config
+        self.current_hook_stage: DynamicsStage | None = None
+        self.sampler = None
+        self.global_rank = 0
+        self._init_hooks(hooks)
+        self._last_converged: torch.Tensor | None = None
+        self._last_outputs: OrderedDict | None = None
+        self._active_mask: torch.Tensor | None = None
+
+    # ---- hooks ---------------------------------------------------------------------------------
+    def _call_hooks(self, stage: DynamicsStage, batch) -> None:
+        self.current_hook_stage = stage
+        super()._call_hooks(stage, batch)
+
+    def _build_context(self, batch) -> DynamicsContext:
+        mask = None
+        if self._last_converged is not None:
+            mask = torch.zeros(batch.num_graphs, dtype=torch.bool, device=batch.positions.device)
+            mask[self._last_converged] = True
+        return DynamicsContext(batch=batch, step_count=self.step_count, model=self.model,
+                               converged_mask=mask, global_rank=self.global_rank, workflow=self)
+
+    def _open_hooks(self) -> None:
+        seen: set[int] = set()
+        for hook in self.hooks:
+            if id(hook) not in seen and hasattr(hook, "__enter__"):
+                seen.add(id(hook))
+                hook.__enter__()
+
+    def _close_hooks(self) -> None:
+        seen: set[int] = set()
+        for hook in self.hooks:
+            if id(hook) in seen:
+                continue
+            seen.add(id(hook))
+            if hasattr(hook, "__exit__"):
+                hook.__exit__(None, None, None)
+            elif hasattr(hook, "close"):
+                hook.close()
+
+    # ---- state ---------------------------------------------------------------------------------
+    def _init_state(self, batch) -> None:
+        """Allocate per-system integrator state (``self._state``); default: none."""
+
+    def _ensure_state_initialized(self, batch) -> None:
+        if not getattr(self, "_state_ready", False):
+            self._init_state(batch)
+            self._state_ready = True
+
+    def pre_update(self, batch) -> None:
+        """First half of the integration step (no-op here)."""
+
+    def post_update(self, batch) -> None:
+        """Second half of the integration step (no-op here)."""
+
+    # ---- model evaluation ----------------------------------------------------------------------
+    def _check_convergence(self, batch) -> torch.Tensor | None:
+        if self.convergence_hook is None:
+            return None
+        return self.convergence_hook.evaluate(batch)
+
+    def _validate_model_outputs(self, outputs) -> None:
+        for key in self.__needs_keys__:
+            if outputs.get(key) is None:
+                raise RuntimeError(f"{type(self).__name__} requires '{key}' from the model, but the model "
+                                   f"returned only {list(outputs.keys())}.")
+
+    def compute(self, batch) -> OrderedDict:
+        """``model(batch)``, validated against ``__needs_keys__``; known outputs are copied
+        into the batch tensors that already exist (``copy_(value.view(target.shape))``)."""
+        self._last_outputs = None
+        outputs = self.model(batch)
+        self._validate_model_outputs(outputs)
+        detached: OrderedDict = OrderedDict()
+        for key, value in outputs.items():
+            detached[key] = value.detach() if isinstance(value, torch.Tensor) else value
+        del outputs
+        for out_key, batch_attr in self._OUTPUT_KEY_TO_BATCH_ATTR.items():
+            value = detached.get(out_key)
+            if value is not None:
+                target = getattr(batch, batch_attr, None)
+                if target is not None:
+                    target.copy_(value.view(target.shape))
+        pos = getattr(batch, "positions", None)
+        if isinstance(pos, torch.Tensor) and pos.requires_grad:
+            pos.requires_grad_(False)
+        self._last_outputs = detached
+        return detached
+
+    # ---- the step ------------------------------------------------------------------------------
+    def step(self, batch):
+        self._ensure_state_initialized(batch)
+        self._call_hooks(DynamicsStage.BEFORE_STEP, batch)
+
+        active_mask: torch.Tensor | None = None
+        status = getattr(batch, "status", None)
+        if status is not None:
+            flat = status.squeeze(-1) if status.dim() == 2 else status
+            active_mask = flat[: batch.num_graphs] < self.exit_status
+        self._active_mask = active_mask
+
+        saved: dict[str, torch.Tensor] = {}
+        node_mask = sys_mask = None
+        if active_mask is not None and not self._honors_active_mask:
+            node_mask = torch.repeat_interleave(active_mask, batch.num_nodes_per_graph.to(torch.long),
+                                                output_size=batch.num_nodes)
+            sys_mask = ~active_mask
+            for field in self._mutable_fields:
+                val = getattr(batch, field, None)
+                if val is None:
+                    continue
+                if val.shape[0] == batch.num_nodes:
+                    saved[field] = val[~node_mask].clone()
+                elif val.shape[0] == batch.num_graphs:
+                    saved[field] = val[sys_mask].clone()
+
+        self._call_hooks(DynamicsStage.BEFORE_PRE_UPDATE, batch)
+        self.pre_update(batch)
+        self._call_hooks(DynamicsStage.AFTER_PRE_UPDATE, batch)
+        self._call_hooks(DynamicsStage.BEFORE_COMPUTE, batch)
+        self.compute(batch)
+        self._call_hooks(DynamicsStage.AFTER_COMPUTE, batch)
+        self._call_hooks(DynamicsStage.BEFORE_POST_UPDATE, batch)
+        self.post_update(batch)
+        self._call_hooks(DynamicsStage.AFTER_POST_UPDATE, batch)
+        if saved:
+            with torch.no_grad():
+                for field, sv in saved.items():
+                    val = getattr(batch, field)
+                    if val.shape[0] == batch.num_nodes:
+                        val[~node_mask] = sv
+                    else:
+                        val[sys_mask] = sv
+
+        self._call_hooks(DynamicsStage.AFTER_STEP, batch)
+        converged = self._check_convergence(batch)
+        self._last_converged = converged
+        if converged is not None:
+            self._call_hooks(DynamicsStage.ON_CONVERGE, batch)
+        self.step_count += 1
+        return batch, converged
+
+    def run(self, batch, n_steps: int | None = None):
+        resolved = n_steps if n_steps is not None else self.n_steps
+        if resolved is None:
+            raise ValueError("No step count provided. Either pass `n_steps` to run() or set it at "
+                             f"construction time via `{type(self).__name__}(..., n_steps=N)`.")
+        self._open_hooks()
+        try:
+            for _ in range(resolved):
+                batch, converged = self.step(batch)
+                if self.sampler is None and converged is not None and converged.numel() == batch.num_graphs:
+                    break
+        finally:
+            self._close_hooks()
+        return batch
+
+    def __repr__(self) -> str:
+        return (f"{type(self).__name__}(model={type(self.model).__name__}, n_steps={self.n_steps}, "
+                f"step_count={self.step_count}, convergence_hook={self.convergence_hook!r}, "
+                f"hooks={len(self.hooks)})")

@@ -1,0 +1,166 @@
+"""``NeighborListHook``: rebuild the neighbor list before each model evaluation.
+
+Mirror of nvalchemi/hooks/neighbor_list.py:112-760 for what callers see: constructor
+``(config, skin, max_neighbors, stage, method)``, the persistent result buffers
+``_neighbor_matrix`` / ``_num_neighbors`` / ``_neighbor_matrix_shifts`` (read by other
+wrappers, nvalchemi/models/pipeline.py:185-196), the K policy (start from the estimate or
+the override; without PBC cap at ceil16(max atoms per system); after the first build grow
+to ceil16(1.5*actual) on overflow and re-run, or trim to ceil16(2*actual) when
+over-estimated, never below the override; :401-486), and the published batch keys.
+
+Differences in mechanism, not in results: there are no staging copies (the kernels read the
+batch tensors directly), and the padding of rows is maintained by the build kernel itself
+instead of a masked fill over the whole ``(N,K)`` buffers after every build (:377-380).
+With ``skin > 0`` the list is searched out to ``cutoff + skin`` as the reference does, but it
+is rebuilt on every call (the displacement test that skips rebuilds is not implemented).
+"""
+
+from __future__ import annotations
+
+from enum import Enum
+
+import torch
+
+from .._neighbor_ops import ceil16, estimate_max_neighbors, neighbor_list
+from ..models.base import NeighborConfig, NeighborListFormat
+from ..neighbors import _write_neighbor_data_to_batch
+from ._context import HookContext
+
+
+class NeighborListHook:
+    """Compute and cache neighbor lists at ``DynamicsStage.BEFORE_COMPUTE``.
+
+    Parameters
+    ----------
+    config : NeighborConfig
+        Cutoff, format (MATRIX or COO) and half-list flag of the model.
+    skin : float
+        Extra search radius; see the module note.
+    max_neighbors : int | None
+        Row width K for the matrix; estimated from the cutoff when ``None``.  Acts as a
+        floor when the hook trims an over-estimate.
+    stage : Enum | None
+        Stage the hook fires at (assigned at registration when ``None``).
+    method : str | None
+        Accepted for compatibility with the reference's strategy names.
+    """
+
+    def __init__(self, config: NeighborConfig, skin: float = 0.0, max_neighbors: int | None = None,
+                 stage: Enum | None = None, method: str | None = None) -> None:
+        self.config = config
+        self.skin = skin
+        self.stage = stage
+        self.method = method
+        self._max_neighbors_override = max_neighbors
+        self.frequency = 1
+        self._neighbor_list_flag = config.format == NeighborListFormat.COO
+
+        self._neighbor_matrix: torch.Tensor | None = None
+        self._num_neighbors: torch.Tensor | None = None
+        self._neighbor_matrix_shifts: torch.Tensor | None = None
+        self._max_neighbors: int = 0
+        self._alloc_N: int | None = None
+        self._alloc_B: int | None = None
+        self._alloc_periodic: bool | None = None
+        self._neighbor_list_method: str | None = None
+        self._actual_max_k: torch.Tensor | None = None
+        self._first_build: bool = True
+
+    def __call__(self, ctx: HookContext, stage: Enum) -> None:
+        self._rebuild(ctx.batch)
+
+    # ------------------------------------------------------------------
+    def _rebuild(self, batch) -> None:
+        positions = batch.positions
+        N = batch.num_nodes
+        B = batch.num_graphs
+        pbc = getattr(batch, "pbc", None)
+        cell = getattr(batch, "cell", None)
+        if cell is None:
+            pbc = None
+        periodic = pbc is not None
+
+        if (self._neighbor_matrix is None or self._neighbor_matrix.shape[0] != N
+                or self._alloc_periodic != periodic or self._neighbor_matrix.device != positions.device):
+            self._alloc_output_tensors(N, batch, pbc)
+            self._alloc_periodic = periodic
+        if self._alloc_N != N or self._alloc_B != B:
+            self._neighbor_list_method = self._select_neighbor_list_method(N, B)
+            self._alloc_N = N
+            self._alloc_B = B
+
+        cutoff = self.config.cutoff + self.skin
+        self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
+
+        if self._first_build:
+            # the one host synchronisation: validate K against the actual maximum
+            self._first_build = False
+            self._actual_max_k = self._num_neighbors.max() if N > 0 else None
+            if self._check_and_resize_k(N, positions.device, pbc):
+                self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
+                # the grown K must be accepted: one spare slot per row
+                while N > 0 and int(self._num_neighbors.max()) >= self._max_neighbors:
+                    self._max_neighbors = ceil16(int(int(self._num_neighbors.max()) * 1.5))
+                    self._realloc_k(N, positions.device, pbc)
+                    self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
+
+        _write_neighbor_data_to_batch(
+            batch=batch, neighbor_matrix=self._neighbor_matrix, num_neighbors=self._num_neighbors,
+            neighbor_matrix_shifts=self._neighbor_matrix_shifts,
+            format=NeighborListFormat.COO if self._neighbor_list_flag else NeighborListFormat.MATRIX,
+            cutoff=self.config.cutoff)
+
+    def _build(self, batch, cutoff, cell, pbc, rebuild_flags) -> None:
+        neighbor_list(positions=batch.positions, cutoff=cutoff, cell=cell, pbc=pbc,
+                      max_neighbors=self._max_neighbors, half_fill=self.config.half_list,
+                      batch_ptr=batch.batch_ptr, batch_idx=batch.batch_idx,
+                      neighbor_matrix=self._neighbor_matrix, num_neighbors=self._num_neighbors,
+                      neighbor_matrix_shifts=self._neighbor_matrix_shifts, rebuild_flags=rebuild_flags,
+                      method=self._neighbor_list_method, tail_mode=0)
+
+    # ------------------------------------------------------------------
+    def _alloc_output_tensors(self, N: int, batch, pbc: torch.Tensor | None) -> None:
+        """(Re)allocate the result buffers for atom count *N* and reset the K check."""
+        max_nbrs = self._max_neighbors_override
+        if max_nbrs is None:
+            max_nbrs = estimate_max_neighbors(cutoff=self.config.cutoff + self.skin)
+        if pbc is None and batch.max_num_nodes > 0:
+            max_nbrs = min(max_nbrs, ceil16(batch.max_num_nodes))
+        self._max_neighbors = int(max_nbrs)
+        self._realloc_k(N, batch.device, pbc)
+        self._first_build = True
+        self._actual_max_k = None
+
+    def _realloc_k(self, N: int, device: torch.device, pbc: torch.Tensor | None) -> None:
+        K = self._max_neighbors
+        self._neighbor_matrix = torch.full((N, K), N, dtype=torch.int32, device=device)
+        self._num_neighbors = torch.zeros(N, dtype=torch.int32, device=device)
+        self._neighbor_matrix_shifts = (
+            torch.zeros(N, K, 3, dtype=torch.int32, device=device) if pbc is not None else None)
+
+    def _check_and_resize_k(self, N: int, device: torch.device, pbc: torch.Tensor | None) -> bool:
+        """Compare K with the actual maximum (host sync).  Returns ``True`` if K grew and the
+        build must be re-run; an over-estimate is trimmed in place."""
+        if self._actual_max_k is None:
+            return False
+        actual = int(self._actual_max_k.item())
+        if actual >= self._max_neighbors:
+            self._max_neighbors = ceil16(int(actual * 1.5))
+            self._realloc_k(N, device, pbc)
+            return True
+        if 0 < actual < 0.5 * self._max_neighbors:
+            new_k = ceil16(int(actual * 2))
+            if self._max_neighbors_override is not None:
+                new_k = max(new_k, self._max_neighbors_override)
+            if new_k < self._max_neighbors:
+                self._max_neighbors = new_k
+                self._neighbor_matrix = self._neighbor_matrix[:, :new_k].contiguous()
+                if self._neighbor_matrix_shifts is not None:
+                    self._neighbor_matrix_shifts = self._neighbor_matrix_shifts[:, :new_k].contiguous()
+        return False
+
+    def _select_neighbor_list_method(self, N: int, B: int) -> str:
+        """Name of the strategy, as the reference would report it; one kernel serves both."""
+        if self.method is not None:
+            return self.method
+        return "cell_list" if N // max(B, 1) >= 2000 else "naive"

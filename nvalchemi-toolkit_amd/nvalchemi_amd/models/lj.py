@@ -1,0 +1,147 @@
+"""``LennardJonesModelWrapper``: the LJ potential as a model for the dynamics engine.
+
+Mirror of nvalchemi/models/lj.py:82-488: same constructor, the same ``ModelConfig``
+(outputs energy/forces/stress, active energy+forces, MATRIX neighbor format), the same
+``adapt_input`` errors (``KeyError`` for a missing input, ``TypeError`` for a non-batch),
+outputs ``energy (B,1)`` / ``forces (N,3)`` / optional ``stress (B,3,3) = -W/|det cell|``.
+The per-system energy (fp64 sum of float32 atomic energies) and the per-system virial come
+out of the same kernel launch instead of separate scatter passes.
+"""
+
+from __future__ import annotations
+
+from collections import OrderedDict
+from typing import Any
+
+import torch
+from torch import nn
+
+from ..data import AtomicData, Batch
+from ._ops.lj import lj_energy_forces_system_batch
+from .base import BaseModelMixin, ModelConfig, NeighborConfig, NeighborListFormat
+
+__all__ = ["LennardJonesModelWrapper"]
+
+
+class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
+    """Lennard-Jones potential ``u(r) = 4 eps [(sigma/r)^12 - (sigma/r)^6]``, plain
+    truncation at ``cutoff``.
+
+    Parameters
+    ----------
+    epsilon, sigma, cutoff : float
+        Well depth, zero-crossing distance, cutoff radius.
+    switch_width : float
+        Must be ``0.0``: the C2 switching function is not implemented.
+    half_list : bool
+        ``True`` if the neighbor matrix holds each pair once.
+    """
+
+    def __init__(self, epsilon: float, sigma: float, cutoff: float, switch_width: float = 0.0,
+                 half_list: bool = False) -> None:
+        super().__init__()
+        if switch_width != 0.0:
+            raise NotImplementedError("switch_width > 0 (C2 switching) is not implemented")
+        self.epsilon = epsilon
+        self.sigma = sigma
+        self.cutoff = cutoff
+        self.switch_width = switch_width
+        self.half_list = half_list
+        self.model_config = ModelConfig(
+            outputs=frozenset({"energy", "forces", "stress"}),
+            active_outputs={"energy", "forces"},
+            autograd_outputs=frozenset(),
+            autograd_inputs=frozenset({"positions"}),
+            required_inputs=frozenset(),
+            optional_inputs=frozenset(),
+            supports_pbc=True,
+            needs_pbc=False,
+            neighbor_config=NeighborConfig(cutoff=self.cutoff, format=NeighborListFormat.MATRIX,
+                                           half_list=self.half_list),
+        )
+        self._eye_cells: torch.Tensor | None = None
+
+    @property
+    def embedding_shapes(self) -> dict[str, tuple[int, ...]]:
+        return {}
+
+    def compute_embeddings(self, data, **kwargs):
+        raise NotImplementedError("LennardJonesModelWrapper does not produce embeddings.")
+
+    def export_model(self, path, as_state_dict: bool = False) -> None:
+        raise NotImplementedError
+
+    # ------------------------------------------------------------------
+    def adapt_input(self, data: AtomicData | Batch, **kwargs: Any) -> dict[str, Any]:
+        """Collect the kernel inputs from *data* (no gradients are enabled: forces are
+        analytic)."""
+        input_dict: dict[str, Any] = {}
+        for key in self.input_data():
+            value = getattr(data, key, None)
+            if value is None:
+                raise KeyError(f"'{key}' required but not found in input data.")
+            input_dict[key] = value
+        if not isinstance(data, Batch):
+            raise TypeError("LennardJonesModelWrapper requires a Batch input; got "
+                            f"{type(data).__name__}.  Use Batch.from_data_list([data]) to wrap it.")
+        input_dict["batch_idx"] = data.batch_idx.to(torch.int32)
+        input_dict["ptr"] = data.batch_ptr.to(torch.int32)
+        input_dict["num_graphs"] = data.num_graphs
+        input_dict["fill_value"] = data.num_nodes
+        input_dict["cells"] = getattr(data, "cell", None)
+        input_dict["neighbor_matrix_shifts"] = getattr(data, "neighbor_matrix_shifts", None)
+        return input_dict
+
+    def adapt_output(self, model_output: Any, data: AtomicData | Batch) -> OrderedDict:
+        output: OrderedDict = OrderedDict()
+        output["energy"] = model_output["energy"]
+        if "forces" in self.model_config.active_outputs:
+            output["forces"] = model_output["forces"]
+        if "stress" in self.model_config.active_outputs:
+            if "virial" in model_output:
+                if not hasattr(data, "cell") or data.cell is None:
+                    raise ValueError("stress output requires cell for volume computation")
+                volume = torch.det(data.cell).abs().view(-1, 1, 1)
+                output["stress"] = -model_output["virial"] / volume
+            elif "stress" in model_output:
+                output["stress"] = model_output["stress"]
+            else:
+                raise RuntimeError("'stress' is in active_outputs but missing from model output")
+        return output
+
+    def output_data(self) -> set[str]:
+        keys = {"energy"}
+        if "forces" in self.model_config.active_outputs:
+            keys.add("forces")
+        if "stress" in self.model_config.active_outputs:
+            keys.add("stress")
+        return keys
+
+    # ------------------------------------------------------------------
+    def forward(self, data: AtomicData | Batch, **kwargs: Any) -> OrderedDict:
+        """``OrderedDict`` with ``energy (B,1)``, ``forces (N,3)`` and optionally
+        ``stress (B,3,3)``."""
+        inp = self.adapt_input(data, **kwargs)
+        positions = inp["positions"]
+        B = inp["num_graphs"]
+        cells = inp.get("cells")
+        shifts = inp.get("neighbor_matrix_shifts")
+        if cells is None:
+            if (self._eye_cells is None or self._eye_cells.shape[0] != B
+                    or self._eye_cells.device != positions.device):
+                self._eye_cells = torch.eye(3, dtype=positions.dtype, device=positions.device) \
+                    .unsqueeze(0).expand(B, 3, 3).contiguous()
+            cells = self._eye_cells
+            shifts = None
+        else:
+            cells = cells.contiguous()
+        compute_stress = "stress" in self.model_config.active_outputs
+        _, forces, sys_e, virials = lj_energy_forces_system_batch(
+            positions.contiguous(), cells, inp["neighbor_matrix"].contiguous(),
+            None if shifts is None else shifts.contiguous(), inp["num_neighbors"].contiguous(),
+            inp["batch_idx"].contiguous(), inp["fill_value"], self.epsilon, self.sigma, self.cutoff,
+            self.switch_width, self.half_list, compute_virial=compute_stress)
+        model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
+        if virials is not None:
+            model_output["virial"] = virials.view(B, 3, 3)
+        return self.adapt_output(model_output, data)

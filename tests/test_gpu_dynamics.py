@@ -1,0 +1,248 @@
+"""GPU end-to-end parity: the package's Batch / hooks / model / dynamics stack against step
+loops driven by the CPU oracle on the same seeded inputs.
+
+Tolerance: 1e-5 relative / 1e-6 absolute on positions, velocities, forces and energies over
+the whole trajectory (the figure the task states for this path); neighbor data bit-exact as
+canonical (i, j, shift) sets.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _reference_loop import fire as ref_fire
+from _reference_loop import nve as ref_nve
+from _systems import fcc_boxes, molecules_batch, periodic_batch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def make_batch(P, Z, M, C, pb, ptr, V=None):
+    from nvalchemi_amd.data import AtomicData, Batch
+
+    data = []
+    for s in range(len(ptr) - 1):
+        a0, a1 = int(ptr[s]), int(ptr[s + 1])
+        kw = dict(atomic_masses=torch.from_numpy(M[a0:a1]), forces=torch.zeros(a1 - a0, 3),
+                  energy=torch.zeros(1, 1))
+        if V is not None:
+            kw["velocities"] = torch.from_numpy(V[a0:a1])
+        if C is not None:
+            kw["cell"] = torch.from_numpy(C[s])
+            kw["pbc"] = torch.from_numpy(pb[s])
+        data.append(AtomicData(torch.from_numpy(P[a0:a1]), torch.from_numpy(Z[a0:a1]), **kw))
+    return Batch.from_data_list(data, device=DEV)
+
+
+def close(got, ref, what):
+    got = got.detach().cpu().numpy().astype(np.float64).reshape(ref.shape)
+    ref = ref.astype(np.float64)
+    err = np.abs(got - ref)
+    tol = ATOL + RTOL * np.abs(ref)
+    assert (err <= tol).all(), (what, float(err.max()), float((err / tol).max()))
+
+
+def test_config1_molecules_100_step_nve_trajectory():
+    from nvalchemi_amd.dynamics import NVE
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, Z, M, ptr = molecules_batch(seed=0)
+    V = np.zeros_like(P)
+    batch = make_batch(P, Z, M, None, None, ptr)
+    model = LennardJonesModelWrapper(epsilon=0.01, sigma=2.5, cutoff=5.0)
+    dyn = NVE(model, dt=0.5, hooks=model.make_neighbor_hooks())
+    checks = []
+
+    def record(step, p, v, f, e):
+        if step in (0, 1, 9, 49, 99):
+            checks.append((step, p.copy(), v.copy(), f.copy(), e.copy()))
+
+    ref_nve(P, V, M, None, None, ptr, 5.0, 0.01, 2.5, 0.5, 100, K=32, record=record)
+    it = iter(checks)
+    nxt = next(it)
+    for step in range(100):
+        dyn.step(batch)
+        if nxt is not None and step == nxt[0]:
+            close(batch.positions, nxt[1], f"positions@{step}")
+            close(batch.velocities, nxt[2], f"velocities@{step}")
+            close(batch.forces, nxt[3], f"forces@{step}")
+            close(batch.energy, nxt[4], f"energy@{step}")
+            nxt = next(it, None)
+    assert dyn.step_count == 100 and nxt is None
+
+
+def test_fcc_boxes_nve_trajectory_and_energy_conservation():
+    from nvalchemi_amd.dynamics import NVE
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=0, n_boxes=3, reps=3, a=3.6)
+    N = len(P)
+    rng = np.random.default_rng(1)
+    M = np.full(N, 63.546, dtype=np.float32)
+    V = rng.normal(0, 0.02, (N, 3)).astype(np.float32)
+    Z = np.full(N, 29, dtype=np.int64)
+    sig = (3.6 / np.sqrt(2)) / 2 ** (1 / 6)
+    rc = 5.0  # below half the 10.8 A box
+    batch = make_batch(P, Z, M, C, pb, ptr, V)
+    model = LennardJonesModelWrapper(epsilon=0.01, sigma=float(sig), cutoff=rc)
+    dyn = NVE(model, dt=1.0, hooks=model.make_neighbor_hooks())
+    dyn.run(batch, n_steps=100)
+    rP, rV, rF, rE = ref_nve(P, V, M, C, pb, ptr, rc, 0.01, float(sig), 1.0, 100, K=96)
+    close(batch.positions, rP, "positions")
+    close(batch.velocities, rV, "velocities")
+    close(batch.forces, rF, "forces")
+    close(batch.energy, rE, "energy")
+    # neighbor data on the batch is the oracle's, as a set
+    ref = oracle.nl_brute(rP, C, pb, ptr, rc)
+    got = oracle.matrix_to_edges(batch.neighbor_matrix.cpu().numpy(), batch.num_neighbors.cpu().numpy(),
+                                 batch.neighbor_matrix_shifts.cpu().numpy())
+    assert np.array_equal(got, ref)
+
+
+def test_fire_relaxation_matches_oracle_and_reaches_the_minimum():
+    from nvalchemi_amd.dynamics import FIRE, ConvergenceHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=3, n_boxes=2, reps=3, a=1.5496, jitter=0.03)  # nn distance ~ 1.096 sigma
+    N = len(P)
+    M = np.ones(N, dtype=np.float32)
+    Z = np.full(N, 18, dtype=np.int64)
+    batch = make_batch(P, Z, M, C, pb, ptr)
+    model = LennardJonesModelWrapper(epsilon=1.0, sigma=1.0, cutoff=2.2)
+    dyn = FIRE(model, dt=0.005, hooks=model.make_neighbor_hooks(),
+               convergence_hook=ConvergenceHook.from_fmax(1e-3))
+    n = 60
+    for _ in range(n):
+        dyn.step(batch)
+    rP, rV, rF, rE, st, _ = ref_fire(P, np.zeros_like(P), M, C, pb, ptr, 2.2, 1.0, 1.0, 0.005, n, K=96)
+    close(batch.positions, rP, "positions")
+    close(batch.forces, rF, "forces")
+    close(batch.energy, rE, "energy")
+    assert np.array_equal(dyn._state.n_steps_positive.cpu().numpy(), st["n_steps_positive"])
+    assert np.allclose(dyn._state.dt.cpu().numpy(), st["dt"], rtol=1e-6)
+    # and it goes downhill
+    e0 = ref_fire(P, np.zeros_like(P), M, C, pb, ptr, 2.2, 1.0, 1.0, 0.005, 1, K=96)[3]
+    assert np.all(batch.energy.cpu().numpy().ravel() < e0)
+
+
+def test_status_mask_freezes_converged_systems_like_the_oracle_loop():
+    from nvalchemi_amd.dynamics import FIRE, ConvergenceHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    from _systems import ptr_from_counts
+
+    parts = [fcc_boxes(seed=100 + s, n_boxes=1, reps=reps, a=1.5496, jitter=jit)
+             for s, (reps, jit) in enumerate([(2, 0.005), (3, 0.05), (2, 0.02), (3, 0.01), (2, 0.08), (2, 0.002)])]
+    P = np.concatenate([p[0] for p in parts])
+    C = np.concatenate([p[1] for p in parts])
+    pb = np.concatenate([p[2] for p in parts])
+    ptr = ptr_from_counts([len(p[0]) for p in parts])
+    N = len(P)
+    M = np.ones(N, dtype=np.float32)
+    Z = np.full(N, 18, dtype=np.int64)
+    batch = make_batch(P, Z, M, C, pb, ptr)
+    batch.status = torch.zeros(len(ptr) - 1, 1, dtype=torch.long, device=DEV)
+    model = LennardJonesModelWrapper(epsilon=1.0, sigma=1.0, cutoff=2.2)
+    tol = 1.0
+    hook = ConvergenceHook.from_fmax(tol, source_status=0, target_status=1)
+    dyn = FIRE(model, dt=0.005, hooks=model.make_neighbor_hooks() + [hook])
+    n = 40
+    for _ in range(n):
+        dyn.step(batch)
+    rP, rV, rF, rE, st, status = ref_fire(P, np.zeros_like(P), M, C, pb, ptr, 2.2, 1.0, 1.0, 0.005, n, K=96,
+                                          fmax_tol=tol)
+    assert np.array_equal(batch.status.cpu().numpy().ravel(), status)
+    assert 0 < status.sum() < len(status), "the case must exercise both frozen and active systems"
+    close(batch.positions, rP, "positions")
+    close(batch.velocities, rV, "velocities")
+
+
+def test_compute_neighbors_matrix_and_coo_and_hook_k_policy():
+    from nvalchemi_amd.hooks import HookContext, NeighborListHook
+    from nvalchemi_amd.models import NeighborConfig, NeighborListFormat
+    from nvalchemi_amd.neighbors import compute_neighbors
+
+    P, C, pb, ptr = periodic_batch(23, 4, 50, 200, 0.6)
+    N = len(P)
+    Z = np.ones(N, dtype=np.int64)
+    M = np.ones(N, dtype=np.float32)
+    ref = oracle.nl_brute(P, C, pb, ptr, 2.5)
+    counts = np.bincount(ref[:, 0], minlength=N)
+
+    batch = make_batch(P, Z, M, C, pb, ptr)
+    compute_neighbors(batch, cutoff=2.5)  # estimate K=32 overflows at this density: the retry loop runs
+    assert batch._neighbor_list_cutoff == 2.5
+    K = batch.neighbor_matrix.shape[1]
+    assert K > counts.max()
+    got = oracle.matrix_to_edges(batch.neighbor_matrix.cpu().numpy(), batch.num_neighbors.cpu().numpy(),
+                                 batch.neighbor_matrix_shifts.cpu().numpy())
+    assert np.array_equal(got, ref)
+
+    batch2 = make_batch(P, Z, M, C, pb, ptr)
+    compute_neighbors(batch2, config=NeighborConfig(cutoff=2.5, format=NeighborListFormat.COO))
+    nl = batch2.neighbor_list.cpu().numpy()
+    sh = batch2.neighbor_list_shifts.cpu().numpy()
+    assert nl.shape == (len(ref), 2) and sh.shape == (len(ref), 3) and batch2.neighbor_list.dtype == torch.int32
+    assert np.array_equal(oracle.canonical_edges(np.concatenate([nl, sh], 1)), ref)
+    assert np.all(np.diff(nl[:, 0]) >= 0), "row-major: sources ascending"
+    assert np.array_equal(batch2.edge_ptr.cpu().numpy(), np.concatenate([[0], np.cumsum(counts)]))
+    bi = oracle.batch_idx_from_ptr(ptr)
+    assert np.array_equal(batch2.num_edges_per_graph.cpu().numpy(), np.bincount(bi[ref[:, 0]], minlength=4))
+    with pytest.raises(ValueError):
+        compute_neighbors(batch2)
+
+    # hook: grows from the estimate, leaves a spare slot, results identical; second call reuses buffers
+    hook = NeighborListHook(NeighborConfig(cutoff=2.5, format=NeighborListFormat.MATRIX))
+    batch3 = make_batch(P, Z, M, C, pb, ptr)
+    hook(HookContext(batch=batch3), None)
+    assert hook._max_neighbors % 16 == 0 and hook._max_neighbors > counts.max()
+    buf = hook._neighbor_matrix
+    hook(HookContext(batch=batch3), None)
+    assert hook._neighbor_matrix is buf and batch3.neighbor_matrix is buf
+    got = oracle.matrix_to_edges(buf.cpu().numpy(), hook._num_neighbors.cpu().numpy(),
+                                 hook._neighbor_matrix_shifts.cpu().numpy())
+    assert np.array_equal(got, ref)
+    # over-estimate is trimmed to ceil16(2*actual), never below the override
+    hook2 = NeighborListHook(NeighborConfig(cutoff=2.5, format=NeighborListFormat.MATRIX), max_neighbors=512)
+    hook2(HookContext(batch=batch3), None)
+    assert hook2._max_neighbors == 512
+    hook3 = NeighborListHook(NeighborConfig(cutoff=1.2, format=NeighborListFormat.MATRIX))
+    hook3._max_neighbors_override = None
+    b4 = make_batch(P, Z, M, C, pb, ptr)
+    hook3(HookContext(batch=b4), None)
+    actual = int(b4.num_neighbors.max())
+    assert hook3._max_neighbors in (16, ((2 * actual + 15) // 16) * 16)
+
+
+def test_non_periodic_batch_has_no_shift_key_and_lj_stress():
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+    from nvalchemi_amd.neighbors import compute_neighbors
+
+    P, Z, M, ptr = molecules_batch(seed=2)
+    batch = make_batch(P, Z, M, None, None, ptr)
+    compute_neighbors(batch, cutoff=5.0)
+    assert getattr(batch, "neighbor_matrix_shifts", None) is None
+    assert batch.neighbor_matrix.shape[1] == 32  # ceil16(max atoms per system)
+    model = LennardJonesModelWrapper(0.01, 2.5, 5.0)
+    out = model(batch)
+    assert list(out.keys()) == ["energy", "forces"] and out["energy"].shape == (len(ptr) - 1, 1)
+
+    Pp, C, pb, ptrp = fcc_boxes(seed=1, n_boxes=2, reps=3, a=0.95 * np.sqrt(2.0), jitter=0.02)
+    b = make_batch(Pp, np.ones(len(Pp), dtype=np.int64), np.ones(len(Pp), dtype=np.float32), C, pb, ptrp)
+    m2 = LennardJonesModelWrapper(1.0, 1.0, 1.3)
+    m2.model_config.active_outputs = {"energy", "forces", "stress"}
+    compute_neighbors(b, config=m2.model_config.neighbor_config)
+    out = m2(b)
+    bi = oracle.batch_idx_from_ptr(ptrp)
+    ref = oracle.lj_matrix(Pp, C, b.neighbor_matrix.cpu().numpy(), b.neighbor_matrix_shifts.cpu().numpy(),
+                           b.num_neighbors.cpu().numpy(), bi, len(Pp), 1.0, 1.0, 1.3, virial=True)
+    vol = np.abs(np.linalg.det(C.astype(np.float64)))[:, None, None]
+    exp = -ref["virials"].reshape(-1, 3, 3) / vol
+    got = out["stress"].cpu().numpy()
+    assert np.allclose(got, exp, rtol=1e-5, atol=1e-5 * np.abs(exp).max())
+    assert np.all(np.diagonal(got, axis1=1, axis2=2) < 0)  # compressed: negative (tensile-positive convention)
+    with pytest.raises(KeyError):  # a bare AtomicData carries no neighbor keys
+        m2(b.get_data(0))
