@@ -169,6 +169,8 @@ __device__ __forceinline__ bool wave_segmented_max(int seg, float& v) {
 }
 
 // ---- FIRE -----------------------------------------------------------------------------------
+constexpr float kFireVmax = 3.0e38f;
+
 struct FireScratch {
     double* acc;   // (M,3): sum F.v, sum v.v, sum F.F
     float* mix_a;  // (M) factor on v
@@ -280,10 +282,16 @@ __global__ __launch_bounds__(kBlock) void fire_update_kernel(
         float vm = (ma * vel[b + a]) + (mb * f);
         float acc = f / m;
         v[a] = vm + (h * acc);
+        v[a] = fminf(fmaxf(v[a], -kFireVmax), kFireVmax);  // keep dr finite
         dr[a] = h * v[a];
     }
-    float n2 = (dr[0] * dr[0] + dr[1] * dr[1]) + dr[2] * dr[2];
-    float nrm = sqrtf(n2);
+    // |dr| without overflow: scale by the largest component first
+    float big = fmaxf(fmaxf(fabsf(dr[0]), fabsf(dr[1])), fabsf(dr[2]));
+    float nrm = 0.0f;
+    if (big > 0.0f) {
+        float a0 = dr[0] / big, a1 = dr[1] / big, a2 = dr[2] / big;
+        nrm = big * sqrtf((a0 * a0 + a1 * a1) + a2 * a2);
+    }
     if (nrm > ms) {
         float sc = ms / nrm;
 #pragma unroll

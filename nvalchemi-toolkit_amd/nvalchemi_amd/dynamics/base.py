@@ -274,7 +274,12 @@ class BaseDynamics(HookRegistryMixin):
         """``model(batch)``, validated against ``__needs_keys__``; known outputs are copied
         into the batch tensors that already exist (``copy_(value.view(target.shape))``)."""
         self._last_outputs = None
-        outputs = self.model(batch)
+        if getattr(self.model, "accepts_output_buffers", False):
+            # the model writes straight into the batch's result tensors: no second pass over them
+            buffers = {k: getattr(batch, attr, None) for k, attr in self._OUTPUT_KEY_TO_BATCH_ATTR.items()}
+            outputs = self.model(batch, out=buffers)
+        else:
+            outputs = self.model(batch)
         self._validate_model_outputs(outputs)
         detached: OrderedDict = OrderedDict()
         for key, value in outputs.items():
@@ -284,7 +289,8 @@ class BaseDynamics(HookRegistryMixin):
             value = detached.get(out_key)
             if value is not None:
                 target = getattr(batch, batch_attr, None)
-                if target is not None:
+                if target is not None and not (value.data_ptr() == target.data_ptr()
+                                               and value.numel() == target.numel()):
                     target.copy_(value.view(target.shape))
         pos = getattr(batch, "positions", None)
         if isinstance(pos, torch.Tensor) and pos.requires_grad:

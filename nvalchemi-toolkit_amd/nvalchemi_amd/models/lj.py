@@ -61,6 +61,10 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
         )
         self._eye_cells: torch.Tensor | None = None
 
+    #: ``forward(batch, out={"forces": ..., "energy": ...})`` writes into the given tensors
+    #: (used by the dynamics engine to fill the batch without a copy pass)
+    accepts_output_buffers = True
+
     @property
     def embedding_shapes(self) -> dict[str, tuple[int, ...]]:
         return {}
@@ -118,9 +122,10 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
         return keys
 
     # ------------------------------------------------------------------
-    def forward(self, data: AtomicData | Batch, **kwargs: Any) -> OrderedDict:
+    def forward(self, data: AtomicData | Batch, out: dict | None = None, **kwargs: Any) -> OrderedDict:
         """``OrderedDict`` with ``energy (B,1)``, ``forces (N,3)`` and optionally
-        ``stress (B,3,3)``."""
+        ``stress (B,3,3)``.  Results are fresh tensors unless ``out`` supplies float32
+        contiguous ``forces (N,3)`` / ``energy (B,1)`` tensors to fill."""
         inp = self.adapt_input(data, **kwargs)
         positions = inp["positions"]
         B = inp["num_graphs"]
@@ -136,11 +141,21 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
         else:
             cells = cells.contiguous()
         compute_stress = "stress" in self.model_config.active_outputs
+        N = positions.shape[0]
+        bufs = {}
+        if out:
+            f_out, e_out = out.get("forces"), out.get("energy")
+            if (isinstance(f_out, torch.Tensor) and f_out.shape == (N, 3) and f_out.dtype == positions.dtype
+                    and f_out.is_contiguous() and f_out.device == positions.device):
+                bufs["forces"] = f_out
+            if (isinstance(e_out, torch.Tensor) and e_out.numel() == B and e_out.dtype == positions.dtype
+                    and e_out.is_contiguous() and e_out.device == positions.device):
+                bufs["system_energies"] = e_out.view(B)
         _, forces, sys_e, virials = lj_energy_forces_system_batch(
             positions.contiguous(), cells, inp["neighbor_matrix"].contiguous(),
             None if shifts is None else shifts.contiguous(), inp["num_neighbors"].contiguous(),
             inp["batch_idx"].contiguous(), inp["fill_value"], self.epsilon, self.sigma, self.cutoff,
-            self.switch_width, self.half_list, compute_virial=compute_stress)
+            self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs)
         model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
         if virials is not None:
             model_output["virial"] = virials.view(B, 3, 3)

@@ -61,6 +61,7 @@
 #endif
 
 #define ORC_API __attribute__((visibility("default")))
+#define ORC_VMAX 3.0e38f
 
 /* ------------------------------------------------------------------------------------------
  * per-system geometry
@@ -452,7 +453,8 @@ ORC_API void orc_vv_post(float* vel, const float* forces, const float* masses, c
  *   P > 0 : v <- (1-alpha) v + alpha sqrt(vv/ff) F   with the STORED alpha;
  *           n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max), alpha *= f_alpha
  *   else  : v <- 0 ; n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
- *   MD    : v += dt F/m ; dr = dt v ; |dr| > maxstep -> dr *= maxstep/|dr| ; r += dr
+ *   MD    : v += dt F/m (clamped to +-3e38) ; dr = dt v ; |dr| > maxstep -> dr *= maxstep/|dr| ;
+ *           r += dr   (|dr| is evaluated scaled by its largest component, so it cannot overflow)
  * Every atom of a system uses the same pre-update scalars.  vf/vv/ff outputs are the
  * float32-rounded reductions.
  * ---------------------------------------------------------------------------------------- */
@@ -510,10 +512,16 @@ ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const fl
             float vm = (mixa[s] * vel[3 * i + a]) + (mixb[s] * f);
             float acc1 = f / m;
             v[a] = vm + (h * acc1);
+            v[a] = fminf(fmaxf(v[a], -ORC_VMAX), ORC_VMAX); /* keep dr finite */
             dr[a] = h * v[a];
         }
-        float n2 = (dr[0] * dr[0] + dr[1] * dr[1]) + dr[2] * dr[2];
-        float nrm = sqrtf(n2);
+        /* |dr| without overflow: scale by the largest component first */
+        float big = fmaxf(fmaxf(fabsf(dr[0]), fabsf(dr[1])), fabsf(dr[2]));
+        float nrm = 0.0f;
+        if (big > 0.0f) {
+            float a0 = dr[0] / big, a1 = dr[1] / big, a2 = dr[2] / big;
+            nrm = big * sqrtf((a0 * a0 + a1 * a1) + a2 * a2);
+        }
         if (nrm > ms) {
             float sc = ms / nrm;
             for (int a = 0; a < 3; ++a) dr[a] = dr[a] * sc;

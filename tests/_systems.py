@@ -70,3 +70,16 @@ def fcc_boxes(seed=0, n_boxes=4, reps=5, a=3.6, jitter=0.05):
     C = np.broadcast_to(np.eye(3) * reps * a, (n_boxes, 3, 3))
     pb = np.ones((n_boxes, 3), dtype=bool)
     return P.astype(np.float32), C.astype(np.float32).copy(), pb, ptr_from_counts([n] * n_boxes)
+
+
+def sheared_fcc_boxes(seed=0, n_boxes=3, reps=3, a=1.5496, jitter=0.03, shear=0.25):
+    """FCC boxes deformed by a random shear per box: triclinic cells without overlapping atoms."""
+    rng = np.random.default_rng(seed)
+    P, C, pb, ptr = fcc_boxes(seed=seed, n_boxes=n_boxes, reps=reps, a=a, jitter=jitter)
+    P = P.astype(np.float64)
+    C = C.astype(np.float64)
+    for s in range(n_boxes):
+        D = np.eye(3) + np.tril(rng.uniform(-shear, shear, (3, 3)), -1)
+        P[ptr[s]:ptr[s + 1]] = P[ptr[s]:ptr[s + 1]] @ D
+        C[s] = C[s] @ D
+    return P.astype(np.float32), C.astype(np.float32), pb, ptr

@@ -95,8 +95,8 @@ def test_fcc_boxes_nve_trajectory_and_energy_conservation():
     close(batch.velocities, rV, "velocities")
     close(batch.forces, rF, "forces")
     close(batch.energy, rE, "energy")
-    # neighbor data on the batch is the oracle's, as a set
-    ref = oracle.nl_brute(rP, C, pb, ptr, rc)
+    # neighbor data on the batch is the oracle's, as a set (for the device's own final positions)
+    ref = oracle.nl_brute(batch.positions.cpu().numpy(), C, pb, ptr, rc)
     got = oracle.matrix_to_edges(batch.neighbor_matrix.cpu().numpy(), batch.num_neighbors.cpu().numpy(),
                                  batch.neighbor_matrix_shifts.cpu().numpy())
     assert np.array_equal(got, ref)
