@@ -31,9 +31,11 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kTile = 1024;       // candidates staged in LDS at a time
-constexpr int kStencilBatch = kBlock; // stencil cells enumerated at a time (one per lane)
-constexpr int kCenterChunk = 256;   // centre atoms of a cell handled per pass
+constexpr int kTile = 768;        // candidates staged in LDS at a time
+constexpr int kStencilBatch = 64; // stencil cells enumerated at a time (one per lane of a wave)
+constexpr int kCenterChunk = 64;  // centre atoms of a cell handled per pass
+constexpr int kHitCap = 256;      // per-wave list of accepted candidates before it is written out
+constexpr int kPackOverflow = 1 << 30;
 constexpr int kMaxCellsPerAxis = 1024;
 constexpr int kMinCellCap = 8;    // a system may use at least this many cells
 constexpr int kMaxStencilRadius = 32;  // cells searched per axis and direction, at most
@@ -54,6 +56,16 @@ struct NlSys {
     int atom_begin, atom_end;
 };
 
+// What the search kernel needs per system, in 32-bit words (read through scalar loads).
+struct NlSearchSys {
+    float step[9];  // cell step vectors, row d = one cell along axis d
+    float tol;      // relative half-width of the float32 uncertainty band on d^2
+    int nc[3];
+    int R[3];
+    int per[3];
+    int cell_offset;
+};
+
 struct NlHeader {
     int total_cells;
     int error;  // bit 0: a system's cell is degenerate or narrower than cutoff/kMaxStencilRadius
@@ -64,7 +76,9 @@ struct NlWorkspace {
     NlHeader* hdr;
     NlSys* sys;
     uint32_t* bounds;    // (B,6) order keys: min x,y,z then max x,y,z
+    NlSearchSys* ssys;   // (B)
     int* cell_offset;    // (B+1)
+    int* cell_sys;       // (C) system of each non-empty cell
     int* atom_cell;      // (N)
     int* atom_rank;      // (N)
     int* cell_count;     // (C)
@@ -94,7 +108,9 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
     p = take(sizeof(NlHeader)); if (ws) ws->hdr = reinterpret_cast<NlHeader*>(p);
     p = take(B * sizeof(NlSys)); if (ws) ws->sys = reinterpret_cast<NlSys*>(p);
     p = take(B * 6 * sizeof(uint32_t)); if (ws) ws->bounds = reinterpret_cast<uint32_t*>(p);
+    p = take(B * sizeof(NlSearchSys)); if (ws) ws->ssys = reinterpret_cast<NlSearchSys*>(p);
     p = take((B + 1) * sizeof(int)); if (ws) ws->cell_offset = reinterpret_cast<int*>(p);
+    p = take(C * sizeof(int)); if (ws) ws->cell_sys = reinterpret_cast<int*>(p);
     p = take(N * sizeof(int)); if (ws) ws->atom_cell = reinterpret_cast<int*>(p);
     p = take(N * sizeof(int)); if (ws) ws->atom_rank = reinterpret_cast<int*>(p);
     p = take(C * sizeof(int)); if (ws) ws->cell_count = reinterpret_cast<int*>(p);
@@ -256,7 +272,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
                 }
                 reach += (R + 1) * sqrt(len);
             }
-            s.tol = (float)(1.0e-6 * (reach / a.rc + 1.0));
+            s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
             s.n_cells = n_at > 0 ? s.nc[0] * s.nc[1] * s.nc[2] : 0;
             ncell = s.n_cells;
             ws.sys[t] = s;
@@ -273,8 +289,20 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
         int incl = s_scan[threadIdx.x];
         int carry = s_carry;
         if (t < a.n_systems) {
-            ws.sys[t].cell_offset = carry + incl - ncell;
-            ws.cell_offset[t] = carry + incl - ncell;
+            const int off = carry + incl - ncell;
+            ws.sys[t].cell_offset = off;
+            ws.cell_offset[t] = off;
+            const NlSys& s = ws.sys[t];
+            NlSearchSys q;
+            for (int k = 0; k < 9; ++k) q.step[k] = (float)s.step[k];
+            q.tol = s.tol;
+            for (int d = 0; d < 3; ++d) {
+                q.nc[d] = s.nc[d];
+                q.R[d] = s.R[d];
+                q.per[d] = s.per[d];
+            }
+            q.cell_offset = off;
+            ws.ssys[t] = q;
         }
         __syncthreads();
         if (threadIdx.x == 1023) s_carry = carry + incl;
@@ -329,6 +357,7 @@ __global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws
     Binned b = bin_atom(s, a.pos + 3 * (size_t)i);
     ws.atom_cell[i] = b.cell;
     ws.atom_rank[i] = atomicAdd(ws.cell_count + b.cell, 1);
+    ws.cell_sys[b.cell] = a.bidx[i];
 }
 
 __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspace ws) {
@@ -354,20 +383,32 @@ __device__ __forceinline__ bool half_keep(int i, int j, int s0, int s1, int s2) 
     return s2 > 0;
 }
 
-__global__ __launch_bounds__(kBlock) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
-    __shared__ float4 c_pos[kTile];          // cell-local xyz of a candidate + its atom index
-    __shared__ int4 c_aux[kTile];            // image of its cell minus its own wrap
+__device__ __forceinline__ int pack_shift(int x, int y, int z) {
+    // three signed 10-bit fields; anything wider is flagged and recovered from global memory
+    if ((unsigned)(x + 512) > 1023u || (unsigned)(y + 512) > 1023u || (unsigned)(z + 512) > 1023u)
+        return kPackOverflow;
+    return (x + 512) | ((y + 512) << 10) | ((z + 512) << 20);
+}
+
+__device__ __forceinline__ float uniform_f(float v) {
+    return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+
+__global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
+    __shared__ float4 c_pos[kTile];           // cell-local xyz of a candidate + its atom index
+    __shared__ int c_pk[kTile];               // packed (image of its cell - its own wrap)
+    __shared__ float4 ca_pos[kCenterChunk];   // centre atoms of this pass: local xyz + atom index
+    __shared__ int4 ca_w[kCenterChunk];       // their wrap integers
+    __shared__ int row_cnt[kCenterChunk];     // running row lengths
     __shared__ int st_start[kStencilBatch];
     __shared__ int st_prefix[kStencilBatch + 1];
     __shared__ int st_q[kStencilBatch][3];
     __shared__ float st_off[kStencilBatch][3];
-    __shared__ int row_cnt[kCenterChunk];    // running row lengths of the centre atoms
-    __shared__ int s_wave[kWavesPerBlock];
-    __shared__ int s_sys;
+    __shared__ unsigned short hits[kWavesPerBlock][kHitCap];
 
     const int total_cells = ws.hdr->total_cells;
     const int lane = lane_id();
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
     const float rc2f = (float)a.rc2;
     // each XCD (consecutive workgroups go to the 8 XCDs round-robin) walks one contiguous
     // eighth of the cells, so the stencil data it re-reads stays in its own L2
@@ -378,70 +419,65 @@ __global__ __launch_bounds__(kBlock) void nl_search_kernel(NlArgs a, NlWorkspace
         // NOTE: every thread of the workgroup takes the same path through this loop body
         const int c = xcd * per_xcd + li;
         if (c >= total_cells) break;
-        // system of this cell: last s with cell_offset[s] <= c
-        if (threadIdx.x == 0) {
-            int lo = 0, hi = a.n_systems;  // invariant: offset[lo] <= c < offset[hi]
-            while (hi - lo > 1) {
-                int mid = (lo + hi) >> 1;
-                if (ws.cell_offset[mid] <= c) lo = mid; else hi = mid;
-            }
-            s_sys = lo;
-        }
-        __syncthreads();
-        const int sidx = s_sys;
-        __syncthreads();
-        if (a.rebuild && !a.rebuild[sidx]) continue;
-        const int n_center = ws.cell_count[c];
-        if (n_center == 0) continue;
-        const NlSys& S = ws.sys[sidx];
         const int c_begin = ws.cell_start[c];
+        const int n_center = ws.cell_start[c + 1] - c_begin;
+        if (n_center == 0) continue;
+        const int sidx = __builtin_amdgcn_readfirstlane(ws.cell_sys[c]);
+        if (a.rebuild && !a.rebuild[sidx]) continue;
+        const NlSearchSys S = ws.ssys[sidx];
         const int lc = c - S.cell_offset;
         const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
-        const int per0 = S.per[0], per1 = S.per[1], per2 = S.per[2];
         const int cz = lc % nc2, cy = (lc / nc2) % nc1, cx = lc / (nc2 * nc1);
         const int R0 = S.R[0], R1 = S.R[1], R2 = S.R[2];
         const int e1 = 2 * R1 + 1, e2 = 2 * R2 + 1;
         const int n_stencil = (2 * R0 + 1) * e1 * e2;
-        const float tol = S.tol;
-        const float rc2_lo = rc2f * (1.0f - tol), rc2_hi = rc2f * (1.0f + tol);
+        const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
 
         for (int cc0 = 0; cc0 < n_center; cc0 += kCenterChunk) {
             const int n_cc = (n_center - cc0) < kCenterChunk ? (n_center - cc0) : kCenterChunk;
-            for (int k = threadIdx.x; k < n_cc; k += kBlock) row_cnt[k] = 0;
+            if ((int)threadIdx.x < n_cc) {
+                ca_pos[threadIdx.x] = ws.sorted_pos[c_begin + cc0 + threadIdx.x];
+                ca_w[threadIdx.x] = ws.sorted_aux[c_begin + cc0 + threadIdx.x];
+                row_cnt[threadIdx.x] = 0;
+            }
 
             for (int sb = 0; sb < n_stencil; sb += kStencilBatch) {
-                // ---- enumerate up to kStencilBatch stencil cells, one per lane
-                int my_count = 0;
-                {
-                    int si = sb + (int)threadIdx.x;
-                    int start = 0, q0 = 0, q1 = 0, q2 = 0;
+                // ---- wave 0 enumerates up to 64 stencil cells, one per lane, and scans their sizes
+                if (wave == 0) {
+                    const int si = sb + lane;
+                    int start = 0, count = 0, q0 = 0, q1 = 0, q2 = 0;
                     float o0 = 0.f, o1 = 0.f, o2 = 0.f;
                     if (si < n_stencil) {
                         int oz = si % e2 - R2, oy = (si / e2) % e1 - R1, ox = si / (e2 * e1) - R0;
                         int gx = cx + ox, gy = cy + oy, gz = cz + oz;
                         bool ok = true;
-                        if (per0) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
-                        if (per1) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
-                        if (per2) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
+                        if (S.per[0]) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
+                        if (S.per[1]) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
+                        if (S.per[2]) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
                         if (ok) {
                             int c2 = S.cell_offset + (gx * nc1 + gy) * nc2 + gz;
                             start = ws.cell_start[c2];
-                            my_count = ws.cell_count[c2];
-                            double ddx = (double)ox, ddy = (double)oy, ddz = (double)oz;
-                            o0 = (float)(ddx * S.step[0] + ddy * S.step[3] + ddz * S.step[6]);
-                            o1 = (float)(ddx * S.step[1] + ddy * S.step[4] + ddz * S.step[7]);
-                            o2 = (float)(ddx * S.step[2] + ddy * S.step[5] + ddz * S.step[8]);
+                            count = ws.cell_start[c2 + 1] - start;
+                            float fx = (float)ox, fy = (float)oy, fz = (float)oz;
+                            o0 = fx * S.step[0] + fy * S.step[3] + fz * S.step[6];
+                            o1 = fx * S.step[1] + fy * S.step[4] + fz * S.step[7];
+                            o2 = fx * S.step[2] + fy * S.step[5] + fz * S.step[8];
                         }
                     }
-                    st_start[threadIdx.x] = start;
-                    st_q[threadIdx.x][0] = q0; st_q[threadIdx.x][1] = q1; st_q[threadIdx.x][2] = q2;
-                    st_off[threadIdx.x][0] = o0; st_off[threadIdx.x][1] = o1; st_off[threadIdx.x][2] = o2;
+                    int incl = count;
+#pragma unroll
+                    for (int o = 1; o < kWave; o <<= 1) {
+                        int up = __shfl_up(incl, o, kWave);
+                        if (lane >= o) incl += up;
+                    }
+                    st_start[lane] = start;
+                    st_prefix[lane] = incl - count;
+                    if (lane == kWave - 1) st_prefix[kStencilBatch] = incl;
+                    st_q[lane][0] = q0; st_q[lane][1] = q1; st_q[lane][2] = q2;
+                    st_off[lane][0] = o0; st_off[lane][1] = o1; st_off[lane][2] = o2;
                 }
-                int batch_total;
-                int ex = scan::block_exclusive(my_count, s_wave, batch_total);
-                st_prefix[threadIdx.x] = ex;
-                if (threadIdx.x == 0) st_prefix[kStencilBatch] = batch_total;
                 __syncthreads();
+                const int batch_total = st_prefix[kStencilBatch];
 
                 for (int t0 = 0; t0 < batch_total; t0 += kTile) {
                     const int tile_n = (batch_total - t0) < kTile ? (batch_total - t0) : kTile;
@@ -449,7 +485,8 @@ __global__ __launch_bounds__(kBlock) void nl_search_kernel(NlArgs a, NlWorkspace
                     for (int k = threadIdx.x; k < tile_n; k += kBlock) {
                         int flat = t0 + k;
                         int lo = 0, hi = kStencilBatch;  // prefix[lo] <= flat < prefix[hi]
-                        while (hi - lo > 1) {
+#pragma unroll
+                        for (int it = 0; it < 6; ++it) {
                             int mid = (lo + hi) >> 1;
                             if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
                         }
@@ -460,48 +497,49 @@ __global__ __launch_bounds__(kBlock) void nl_search_kernel(NlArgs a, NlWorkspace
                         p.y += st_off[lo][1];
                         p.z += st_off[lo][2];
                         c_pos[k] = p;
-                        c_aux[k] = make_int4(st_q[lo][0] - w.x, st_q[lo][1] - w.y, st_q[lo][2] - w.z, 0);
+                        c_pk[k] = pack_shift(st_q[lo][0] - w.x, st_q[lo][1] - w.y, st_q[lo][2] - w.z);
                     }
                     __syncthreads();
 
                     // ---- each wave: its centre atoms against the tile, 64 candidates a step
                     for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
-                        const float4 ci = ws.sorted_pos[c_begin + cc0 + ca];
-                        const int4 wa = ws.sorted_aux[c_begin + cc0 + ca];
-                        const float xi = ci.x, yi = ci.y, zi = ci.z;
-                        const int i_atom = __float_as_int(ci.w);
+                        const float4 ci = ca_pos[ca];
+                        const int4 wa = ca_w[ca];
+                        const float xi = uniform_f(ci.x), yi = uniform_f(ci.y), zi = uniform_f(ci.z);
+                        const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ci.w));
+                        const int wi0 = __builtin_amdgcn_readfirstlane(wa.x);
+                        const int wi1 = __builtin_amdgcn_readfirstlane(wa.y);
+                        const int wi2 = __builtin_amdgcn_readfirstlane(wa.z);
+                        const int self_pk = pack_shift(-wi0, -wi1, -wi2);  // shift 0 <=> q - w_j == -w_i
                         int32_t* row = a.nm + (size_t)i_atom * a.K;
                         int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
-                        int cnt = row_cnt[ca];
-                        for (int k0 = 0; k0 < tile_n; k0 += kWave) {
-                            int k = k0 + lane;
-                            bool in = false;
-                            int j = 0, s0 = 0, s1 = 0, s2 = 0;
-                            if (k < tile_n) {
-                                float4 p = c_pos[k];
-                                float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
-                                float d2 = dx * dx + dy * dy + dz * dz;
-                                if (d2 < rc2_hi) {
-                                    int4 w = c_aux[k];
-                                    j = __float_as_int(p.w);
-                                    s0 = w.x + wa.x; s1 = w.y + wa.y; s2 = w.z + wa.z;
-                                    in = true;
-                                    if (!(d2 < rc2_lo)) {
-                                        // inside the float32 uncertainty band: decide exactly
-                                        const float* pi = a.pos + 3 * (size_t)i_atom;
-                                        const float* pj = a.pos + 3 * (size_t)j;
-                                        double e0, e1d, e2d;
-                                        double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2],
-                                                                  s0, s1, s2, S.h, e0, e1d, e2d);
-                                        in = r2 < a.rc2;
+                        int base = __builtin_amdgcn_readfirstlane(row_cnt[ca]);  // entries found before this tile
+                        int nh = 0;                                               // entries in the hit list
+                        unsigned short* my_hits = hits[wave];
+
+                        auto flush = [&]() {
+                            for (int l = lane; l < nh; l += kWave) {
+                                const int k = my_hits[l];
+                                const int j = __float_as_int(c_pos[k].w);
+                                int pk = c_pk[k];
+                                int s0, s1, s2;
+                                if (pk & kPackOverflow) {
+                                    // wide shift: recover it from the sorted arrays
+                                    int flat = t0 + k, lo = 0, hi = kStencilBatch;
+                                    for (int it = 0; it < 6; ++it) {
+                                        int mid = (lo + hi) >> 1;
+                                        if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
                                     }
-                                    if (j == i_atom && s0 == 0 && s1 == 0 && s2 == 0) in = false;
-                                    if (a.half && in) in = half_keep(i_atom, j, s0, s1, s2);
+                                    int4 w = ws.sorted_aux[st_start[lo] + (flat - st_prefix[lo])];
+                                    s0 = st_q[lo][0] - w.x + wi0;
+                                    s1 = st_q[lo][1] - w.y + wi1;
+                                    s2 = st_q[lo][2] - w.z + wi2;
+                                } else {
+                                    s0 = (pk & 1023) - 512 + wi0;
+                                    s1 = ((pk >> 10) & 1023) - 512 + wi1;
+                                    s2 = ((pk >> 20) & 1023) - 512 + wi2;
                                 }
-                            }
-                            unsigned long long m = __ballot(in);
-                            if (in) {
-                                int slot = cnt + __popcll(m & ((1ull << lane) - 1ull));
+                                const int slot = base + l;
                                 if (slot < a.K) {
                                     row[slot] = j;
                                     if (srow) {
@@ -511,18 +549,90 @@ __global__ __launch_bounds__(kBlock) void nl_search_kernel(NlArgs a, NlWorkspace
                                     }
                                 }
                             }
-                            cnt += __popcll(m);
+                            base += nh;
+                            nh = 0;
+                        };
+
+                        for (int k0 = 0; k0 < tile_n; k0 += kWave) {
+                            const int k = k0 + lane;
+                            const int kk = k < tile_n ? k : tile_n - 1;
+                            const float4 p = c_pos[kk];
+                            const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
+                            const float d2 = dx * dx + dy * dy + dz * dz;
+                            const int j = __float_as_int(p.w);
+                            bool in = (k < tile_n) && (d2 < rc2_hi);
+                            const bool special = in && (!(d2 < rc2_lo) || j == i_atom);
+                            if (__builtin_amdgcn_ballot_w64(special)) {
+                                if (special) {
+                                    int pk = c_pk[kk];
+                                    if (j == i_atom && pk == self_pk && !(pk & kPackOverflow)) in = false;
+                                    if (in && !(d2 < rc2_lo)) {
+                                        // inside the float32 uncertainty band: decide exactly
+                                        int s0, s1, s2;
+                                        if (pk & kPackOverflow) {
+                                            int flat = t0 + kk, lo = 0, hi = kStencilBatch;
+                                            for (int it = 0; it < 6; ++it) {
+                                                int mid = (lo + hi) >> 1;
+                                                if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
+                                            }
+                                            int4 w = ws.sorted_aux[st_start[lo] + (flat - st_prefix[lo])];
+                                            s0 = st_q[lo][0] - w.x + wi0;
+                                            s1 = st_q[lo][1] - w.y + wi1;
+                                            s2 = st_q[lo][2] - w.z + wi2;
+                                        } else {
+                                            s0 = (pk & 1023) - 512 + wi0;
+                                            s1 = ((pk >> 10) & 1023) - 512 + wi1;
+                                            s2 = ((pk >> 20) & 1023) - 512 + wi2;
+                                        }
+                                        const float* pi = a.pos + 3 * (size_t)i_atom;
+                                        const float* pj = a.pos + 3 * (size_t)j;
+                                        double e0, e1d, e2d;
+                                        double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0,
+                                                                  s1, s2, ws.sys[sidx].h, e0, e1d, e2d);
+                                        in = r2 < a.rc2;
+                                        if (j == i_atom && s0 == 0 && s1 == 0 && s2 == 0) in = false;
+                                    }
+                                }
+                            }
+                            if (a.half) {
+                                if (j == i_atom) {
+                                    // self image: keep the lexicographically positive shift
+                                    int pk = c_pk[kk];
+                                    int s0 = (pk & 1023) - 512 + wi0, s1 = ((pk >> 10) & 1023) - 512 + wi1,
+                                        s2 = ((pk >> 20) & 1023) - 512 + wi2;
+                                    if (pk & kPackOverflow) {
+                                        int flat = t0 + kk, lo = 0, hi = kStencilBatch;
+                                        for (int it = 0; it < 6; ++it) {
+                                            int mid = (lo + hi) >> 1;
+                                            if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
+                                        }
+                                        int4 w = ws.sorted_aux[st_start[lo] + (flat - st_prefix[lo])];
+                                        s0 = st_q[lo][0] - w.x + wi0;
+                                        s1 = st_q[lo][1] - w.y + wi1;
+                                        s2 = st_q[lo][2] - w.z + wi2;
+                                    }
+                                    in = in && half_keep(i_atom, j, s0, s1, s2);
+                                } else {
+                                    in = in && (i_atom < j);
+                                }
+                            }
+                            const unsigned long long m = __builtin_amdgcn_ballot_w64(in);
+                            if (in) my_hits[nh + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0))] = (unsigned short)k;
+                            nh += __popcll(m);
+                            if (nh > kHitCap - kWave) flush();
                         }
-                        if (lane == 0) row_cnt[ca] = cnt;
+                        flush();
+                        if (lane == 0) row_cnt[ca] = base;
                     }
                     __syncthreads();
                 }
+                __syncthreads();  // everyone has read this batch's totals before wave 0 rewrites them
             }
 
             // ---- counts, and padding over what the previous build left beyond them
             for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
-                const int i_atom = __float_as_int(ws.sorted_pos[c_begin + cc0 + ca].w);
-                const int cnt = row_cnt[ca];
+                const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ca_pos[ca].w));
+                const int cnt = __builtin_amdgcn_readfirstlane(row_cnt[ca]);
                 const int old_cnt = a.nn[i_atom];
                 int32_t* row = a.nm + (size_t)i_atom * a.K;
                 int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
