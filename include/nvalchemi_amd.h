@@ -102,7 +102,7 @@ int32_t nvamd_nl_matrix_to_coo(const int32_t* neighbor_matrix,
  *   virials (B,9) f32 or NULL: W = -sum r_ij (x) F_ij, row-major, overwritten.
  *   system_energies (B) f32 or NULL: fp64 sum of the float32 atomic energies, overwritten.
  *   switch_width must be 0 (the C2 switching function is not implemented).
- *   workspace: nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list).
+ *   workspace: nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list); always required.
  * ---------------------------------------------------------------------------------------- */
 int32_t nvamd_lj_workspace_bytes(int32_t n_atoms, int32_t n_systems, int32_t half_list,
                                  size_t* bytes);

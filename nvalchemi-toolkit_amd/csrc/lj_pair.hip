@@ -35,6 +35,10 @@ struct LjArgs {
     float* forces;
     double* sys_acc;  // (B, 1 + 9): energy then virial, fp64, zeroed before the launch
     unsigned n_blocks;
+    int rows_per_block;
+    const int32_t* sys_first;  // (B) first atom of each non-empty system
+    const int32_t* sys_last;   // (B) one past its last atom
+    int lds_atoms;             // stage positions in LDS when the systems of a run have at most this many atoms
 };
 
 template <int LPR>
@@ -44,24 +48,34 @@ __device__ __forceinline__ double group_sum(double v) {
     return v;
 }
 
-template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS>
-__global__ __launch_bounds__(kBlock) void lj_matrix_kernel(LjArgs a) {
-    constexpr int G = kBlock / LPR;  // rows per workgroup
-    __shared__ int s_sys[G];
-    __shared__ double s_val[G][VIRIAL ? 7 : 1];
+constexpr int kSysSlots = 8;      // consecutive systems a workgroup accumulates in LDS
+constexpr int kLdsAtoms = 4096;   // positions of this many consecutive atoms fit the LDS stage
+constexpr int kBlockFull = 512;   // workgroup size of the full-list kernel
 
-    unsigned lb = xcd_contiguous_block(blockIdx.x, a.n_blocks);
-    if (lb >= a.n_blocks) return;
+// first/last atom of every non-empty system, from the non-decreasing batch_idx
+__global__ __launch_bounds__(kBlock) void lj_sys_range_kernel(const int32_t* __restrict__ bidx, int n_atoms,
+                                                              int32_t* __restrict__ first,
+                                                              int32_t* __restrict__ last) {
+    int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_atoms) return;
+    int s = bidx[i];
+    if (i == 0 || bidx[i - 1] != s) first[s] = i;
+    if (i == n_atoms - 1 || bidx[i + 1] != s) last[s] = i + 1;
+}
+
+// One pass over the rows [row0, row_end).  LDS_POS: neighbor positions come from the LDS stage
+// (atoms [span0, span0 + span_n)), otherwise from global memory.
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC>
+__device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, int sys_base,
+                                        const float* __restrict__ s_pos, int span0, int span_n,
+                                        double (*s_acc)[VIRIAL ? 7 : 1]) {
+    constexpr int G = kBlockFull / LPR;
     const int g = threadIdx.x / LPR;
     const int sub = threadIdx.x % LPR;
-    const int i = (int)(lb * G) + g;
-    const bool row_ok = i < a.n_atoms;
-
-    double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
-    double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;  // xx xy xz yy yz zz
-    int sys = -1 - g;
-    if (row_ok) {
-        sys = a.bidx[i];
+    for (int i = row0 + g; i < row_end; i += G) {
+        double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
+        double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;  // xx xy xz yy yz zz
+        const int sys = a.bidx[i];
         int cnt = a.nn[i];
         cnt = cnt < a.K ? cnt : a.K;
         const float* pi = a.pos + 3 * (size_t)i;
@@ -77,95 +91,174 @@ __global__ __launch_bounds__(kBlock) void lj_matrix_kernel(LjArgs a) {
         }
         const int32_t* row = a.nm + (size_t)i * a.K;
         const int32_t* srow = SHIFTS ? a.shifts + (size_t)i * a.K * 3 : nullptr;
-        for (int k = sub; k < cnt; k += LPR) {
-            int j = row[k];
-            if (j < 0 || j >= a.fill) continue;
-            int s0 = 0, s1 = 0, s2 = 0;
-            if (SHIFTS) {
-                s0 = srow[3 * k + 0];
-                s1 = srow[3 * k + 1];
-                s2 = srow[3 * k + 2];
+        // UNROLL row entries per lane are in flight at once: first every index and shift of the
+        // chunk, then every neighbor position, then the arithmetic (the loop is latency bound
+        // otherwise: two dependent trips to memory per entry)
+        constexpr int UNROLL = 4;
+        for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
+            int jj[UNROLL], s0[UNROLL], s1[UNROLL], s2[UNROLL];
+            float xj[UNROLL], yj[UNROLL], zj[UNROLL];
+            if (VEC) {
+                // each lane owns four consecutive entries: one 16-byte load of indices and three
+                // of shifts, so a row is read as contiguous 256 + 768 byte runs (K % 4 == 0)
+                const int kb = k0 + UNROLL * sub;
+                const int kq = kb <= a.K - 4 ? kb : a.K - 4;
+                const int4 j4 = *reinterpret_cast<const int4*>(row + kq);
+                jj[0] = j4.x; jj[1] = j4.y; jj[2] = j4.z; jj[3] = j4.w;
+                if (SHIFTS) {
+                    const int4* sp = reinterpret_cast<const int4*>(srow + 3 * kq);
+                    const int4 sa = sp[0], sb = sp[1], sc = sp[2];
+                    s0[0] = sa.x; s1[0] = sa.y; s2[0] = sa.z;
+                    s0[1] = sa.w; s1[1] = sb.x; s2[1] = sb.y;
+                    s0[2] = sb.z; s1[2] = sb.w; s2[2] = sc.x;
+                    s0[3] = sc.y; s1[3] = sc.z; s2[3] = sc.w;
+                } else {
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) s0[u] = s1[u] = s2[u] = 0;
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+                    if (kb + u >= cnt) jj[u] = -1;
+            } else {
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                // clamped, unconditional loads (slot cnt-1 exists): nothing to wait for in between
+                const int k = k0 + u * LPR + sub;
+                const int kq = k < cnt ? k : cnt - 1;
+                jj[u] = row[kq];
+                s0[u] = s1[u] = s2[u] = 0;
+                if (SHIFTS) {
+                    s0[u] = srow[3 * kq + 0];
+                    s1[u] = srow[3 * kq + 1];
+                    s2[u] = srow[3 * kq + 2];
+                }
+                if (k >= cnt) jj[u] = -1;
             }
-            const float* pj = a.pos + 3 * (size_t)j;
-            double d0, d1, d2;
-            double r2 = pair_d2_exact(xi, yi, zi, pj[0], pj[1], pj[2], s0, s1, s2, h, d0, d1, d2);
-            if (!(r2 < a.rc2)) continue;
-            double ir2 = 1.0 / r2;
-            double q2 = a.sig2 * ir2;
-            double q6 = q2 * q2 * q2;
-            double q12 = q6 * q6;
-            e += 0.5 * (a.c4eps * (q12 - q6));
-            double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
-            fx += gg * d0;
-            fy += gg * d1;
-            fz += gg * d2;
-            if (VIRIAL) {
-                double hg = -0.5 * gg;
-                w0 += hg * d0 * d0;
-                w1 += hg * d0 * d1;
-                w2 += hg * d0 * d2;
-                w3 += hg * d1 * d1;
-                w4 += hg * d1 * d2;
-                w5 += hg * d2 * d2;
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const bool ok = jj[u] >= 0 && jj[u] < a.fill;
+                const int j = ok ? jj[u] : i;
+                if (!ok) jj[u] = -1;
+                const unsigned rel = (unsigned)(j - span0);
+                if (LDS_POS && rel < (unsigned)span_n) {
+                    xj[u] = s_pos[3 * rel + 0];
+                    yj[u] = s_pos[3 * rel + 1];
+                    zj[u] = s_pos[3 * rel + 2];
+                } else {
+                    const float* pj = a.pos + 3 * (size_t)j;
+                    xj[u] = pj[0];
+                    yj[u] = pj[1];
+                    zj[u] = pj[2];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                double d0, d1, d2;
+                double r2 = pair_d2_exact(xi, yi, zi, xj[u], yj[u], zj[u], s0[u], s1[u], s2[u], h, d0, d1, d2);
+                if (jj[u] < 0 || !(r2 < a.rc2)) continue;
+                double ir2 = 1.0 / r2;
+                double q2 = a.sig2 * ir2;
+                double q6 = q2 * q2 * q2;
+                double q12 = q6 * q6;
+                e += 0.5 * (a.c4eps * (q12 - q6));
+                double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
+                fx += gg * d0;
+                fy += gg * d1;
+                fz += gg * d2;
+                if (VIRIAL) {
+                    double hg = -0.5 * gg;
+                    w0 += hg * d0 * d0;
+                    w1 += hg * d0 * d1;
+                    w2 += hg * d0 * d2;
+                    w3 += hg * d1 * d1;
+                    w4 += hg * d1 * d2;
+                    w5 += hg * d2 * d2;
+                }
             }
         }
-    }
-    e = group_sum<LPR>(e);
-    fx = group_sum<LPR>(fx);
-    fy = group_sum<LPR>(fy);
-    fz = group_sum<LPR>(fz);
-    if (VIRIAL) {
-        w0 = group_sum<LPR>(w0);
-        w1 = group_sum<LPR>(w1);
-        w2 = group_sum<LPR>(w2);
-        w3 = group_sum<LPR>(w3);
-        w4 = group_sum<LPR>(w4);
-        w5 = group_sum<LPR>(w5);
-    }
-    if (sub == 0) {
-        float ef = (float)e;
-        if (row_ok) {
+        e = group_sum<LPR>(e);
+        fx = group_sum<LPR>(fx);
+        fy = group_sum<LPR>(fy);
+        fz = group_sum<LPR>(fz);
+        if (VIRIAL) {
+            w0 = group_sum<LPR>(w0);
+            w1 = group_sum<LPR>(w1);
+            w2 = group_sum<LPR>(w2);
+            w3 = group_sum<LPR>(w3);
+            w4 = group_sum<LPR>(w4);
+            w5 = group_sum<LPR>(w5);
+        }
+        if (sub == 0) {
+            const float ef = (float)e;
             a.e_atom[i] = ef;
             float* fo = a.forces + 3 * (size_t)i;
             fo[0] = (float)fx;
             fo[1] = (float)fy;
             fo[2] = (float)fz;
-        }
-        if (SYS) {
-            s_sys[g] = sys;
-            s_val[g][0] = (double)ef;  // the reference sums the rounded atomic energies
-            if (VIRIAL) {
-                s_val[g][1] = w0; s_val[g][2] = w1; s_val[g][3] = w2;
-                s_val[g][4] = w3; s_val[g][5] = w4; s_val[g][6] = w5;
+            if (SYS) {
+                // the reference sums the float32-rounded atomic energies in double
+                const int slot = sys - sys_base;
+                if (slot >= 0 && slot < kSysSlots) {
+                    atomicAdd(&s_acc[slot][0], (double)ef);
+                    if (VIRIAL) {
+                        atomicAdd(&s_acc[slot][1], w0); atomicAdd(&s_acc[slot][2], w1);
+                        atomicAdd(&s_acc[slot][3], w2); atomicAdd(&s_acc[slot][4], w3);
+                        atomicAdd(&s_acc[slot][5], w4); atomicAdd(&s_acc[slot][6], w5);
+                    }
+                } else {
+                    double* out = a.sys_acc + 10 * (size_t)sys;
+                    atomic_add_f64(out + 0, (double)ef);
+                    if (VIRIAL) {
+                        atomic_add_f64(out + 1, w0); atomic_add_f64(out + 2, w1);
+                        atomic_add_f64(out + 3, w2); atomic_add_f64(out + 5, w3);
+                        atomic_add_f64(out + 6, w4); atomic_add_f64(out + 9, w5);
+                    }
+                }
             }
         }
     }
+}
+
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool VEC>
+__global__ __launch_bounds__(kBlockFull) void lj_matrix_kernel(LjArgs a) {
+    constexpr int NV = VIRIAL ? 7 : 1;
+    __shared__ double s_acc[kSysSlots][NV];
+    __shared__ float s_pos[3 * kLdsAtoms];
+
+    // a workgroup owns rows_per_block consecutive rows; workgroups are numbered so that each
+    // XCD walks one contiguous eighth of the atoms
+    const unsigned lb = xcd_contiguous_block(blockIdx.x, a.n_blocks);
+    if (lb >= a.n_blocks) return;
+    const int row0 = (int)lb * a.rows_per_block;
+    const int row_end = (row0 + a.rows_per_block) < a.n_atoms ? (row0 + a.rows_per_block) : a.n_atoms;
+    if (row0 >= row_end) return;
+    const int sys_lo = a.bidx[row0];
+    if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
+
+    // neighbors live in the systems of these rows: stage their positions in LDS when they fit
+    // (atom order carries no spatial locality, so gathers through the caches move a whole line
+    // per 12 useful bytes)
+    const int span0 = a.sys_first[sys_lo];
+    const int span_n = a.sys_last[a.bidx[row_end - 1]] - span0;
+    const bool staged = span_n > 0 && span_n <= a.lds_atoms;
+    if (staged) {
+        const float* src = a.pos + 3 * (size_t)span0;
+        for (int t = threadIdx.x; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
+    }
+    __syncthreads();
+    if (staged) lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC>(a, row0, row_end, sys_lo, s_pos, span0, span_n, s_acc);
+    else lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC>(a, row0, row_end, sys_lo, s_pos, 0, 0, s_acc);
+
     if (SYS) {
         __syncthreads();
-        // rows of one system are consecutive: the first row of each run adds the run up
-        if (threadIdx.x < G) {
-            int t = threadIdx.x;
-            int s = s_sys[t];
-            bool head = s >= 0 && (t == 0 || s_sys[t - 1] != s);
-            if (head) {
-                constexpr int NV = VIRIAL ? 7 : 1;
-                double acc[NV];
-#pragma unroll
-                for (int k = 0; k < NV; ++k) acc[k] = 0.0;
-                for (int u = t; u < G && s_sys[u] == s; ++u) {
-#pragma unroll
-                    for (int k = 0; k < NV; ++k) acc[k] += s_val[u][k];
-                }
-                double* out = a.sys_acc + 10 * (size_t)s;
-                atomic_add_f64(out + 0, acc[0]);
-                if (VIRIAL) {
-                    atomic_add_f64(out + 1, acc[1]);
-                    atomic_add_f64(out + 2, acc[2]);
-                    atomic_add_f64(out + 3, acc[3]);
-                    atomic_add_f64(out + 5, acc[4]);
-                    atomic_add_f64(out + 6, acc[5]);
-                    atomic_add_f64(out + 9, acc[6]);
-                }
+        if (threadIdx.x < kSysSlots * NV) {
+            const int slot = threadIdx.x / NV, k = threadIdx.x % NV;
+            const double v = s_acc[slot][k];
+            if (v != 0.0 && sys_lo + slot < a.n_systems) {
+                // k: 0 energy, 1..6 the upper triangle xx xy xz yy yz zz of the virial
+                const int where = (k == 0) ? 0 : (k <= 3 ? k : (k <= 5 ? k + 1 : 9));
+                atomic_add_f64(a.sys_acc + 10 * (size_t)(sys_lo + slot) + where, v);
             }
         }
     }
@@ -271,15 +364,28 @@ __global__ __launch_bounds__(kBlock) void lj_sys_finish_kernel(const double* __r
 
 template <int LPR>
 void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_t st) {
-    constexpr int G = kBlock / LPR;
+    constexpr int G = kBlockFull / LPR;
     LjArgs b = a;
-    b.n_blocks = (unsigned)((a.n_atoms + G - 1) / G);
+    // a workgroup owns a run of consecutive rows: long enough to amortise the staging of its
+    // systems' positions and to keep per-system sums in LDS, short enough to fill the chip
+    static int forced_rows = [] {
+        const char* e = getenv("NVAMD_LJ_ROWS_PER_BLOCK");
+        return e ? atoi(e) : 0;
+    }();
+    int rows = forced_rows > 0 ? forced_rows : 512;
+    while (forced_rows <= 0 && rows > 4 * G && (a.n_atoms + rows - 1) / rows < 256 * 6) rows /= 2;
+    rows = (rows + G - 1) / G * G;
+    b.rows_per_block = rows;
+    b.n_blocks = (unsigned)((a.n_atoms + rows - 1) / rows);
     unsigned per = (b.n_blocks + 7) / 8;
-    dim3 grid(per * 8), blk(kBlock);
-#define NVAMD_LJ_CASE(V, S, Y)                                                          \
-    if (virial == V && shifts == S && sys == Y) {                                       \
-        hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y>), grid, blk, 0, st, b);      \
-        return;                                                                         \
+    dim3 grid(per * 8), blk(kBlockFull);
+    // 16-byte row loads need aligned rows: K a multiple of 4 and aligned base pointers
+    const bool vec = a.K >= 4 && a.K % 4 == 0 && aligned16(a.nm) && (!a.shifts || aligned16(a.shifts));
+#define NVAMD_LJ_CASE(V, S, Y)                                                                 \
+    if (virial == V && shifts == S && sys == Y) {                                              \
+        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true>), grid, blk, 0, st, b); \
+        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false>), grid, blk, 0, st, b);    \
+        return;                                                                                \
     }
     NVAMD_LJ_CASE(false, false, false)
     NVAMD_LJ_CASE(false, false, true)
@@ -296,8 +402,8 @@ int lanes_per_row(int K) {
         return e ? atoi(e) : 0;
     }();
     if (forced == 8 || forced == 16 || forced == 32 || forced == 64) return forced;
-    if (K <= 16) return 8;
-    if (K <= 256) return 16;
+    if (K <= 192) return 8;
+    if (K <= 512) return 16;
     return 32;
 }
 
@@ -311,6 +417,7 @@ NVAMD_EXPORT int32_t nvamd_lj_workspace_bytes(int32_t n_atoms, int32_t n_systems
     if (!bytes || n_atoms < 0 || n_systems < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj workspace: bad argument");
     size_t b = align_up((size_t)(n_systems > 0 ? n_systems : 1) * 10 * sizeof(double));
+    b += 2 * align_up((size_t)(n_systems > 0 ? n_systems : 1) * sizeof(int32_t));
     if (half_list) b += align_up((size_t)(n_atoms > 0 ? n_atoms : 1) * 4 * sizeof(double));
     *bytes = b;
     return NVAMD_OK;
@@ -339,7 +446,7 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
     size_t need = 0;
     nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list, &need);
     const bool want_sys = (virials != nullptr) || (system_energies != nullptr);
-    if ((want_sys || half_list) && (!workspace || workspace_bytes < need))
+    if (!workspace || workspace_bytes < need)
         return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "lj: workspace %zu < %zu bytes", workspace_bytes, need);
 
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -362,8 +469,17 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
     a.forces = forces;
     a.sys_acc = nullptr;
     a.n_blocks = 0;
+    a.rows_per_block = 0;
+    a.sys_first = nullptr;
+    a.sys_last = nullptr;
+    a.lds_atoms = getenv("NVAMD_LJ_NO_LDS") ? 0 : kLdsAtoms;
     const bool shifts = neighbor_matrix_shifts != nullptr;
     char* w = static_cast<char*>(workspace);
+    const size_t nsys = (size_t)(n_systems > 0 ? n_systems : 1);
+    int32_t* sys_first = reinterpret_cast<int32_t*>(w + align_up(nsys * 10 * sizeof(double)));
+    int32_t* sys_last = reinterpret_cast<int32_t*>(w + align_up(nsys * 10 * sizeof(double)) +
+                                                   align_up(nsys * sizeof(int32_t)));
+    char* w_half = w + align_up(nsys * 10 * sizeof(double)) + 2 * align_up(nsys * sizeof(int32_t));
     if (want_sys && n_systems > 0) {
         a.sys_acc = reinterpret_cast<double*>(w);
         size_t n = (size_t)n_systems * 10;
@@ -374,8 +490,7 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
         if (half_list) {
             LjHalfArgs p;
             p.a = a;
-            p.atom_acc = reinterpret_cast<double*>(
-                w + align_up((size_t)(n_systems > 0 ? n_systems : 1) * 10 * sizeof(double)));
+            p.atom_acc = reinterpret_cast<double*>(w_half);
             size_t n = (size_t)n_atoms * 4;
             hipLaunchKernelGGL(clear_f64_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock),
                                0, st, p.atom_acc, n);
@@ -390,6 +505,10 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
         } else {
             const bool vir = virials != nullptr;
             const bool sys = a.sys_acc != nullptr;
+            hipLaunchKernelGGL(lj_sys_range_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+                               batch_idx, n_atoms, sys_first, sys_last);
+            a.sys_first = sys_first;
+            a.sys_last = sys_last;
             switch (lanes_per_row(max_neighbors)) {
                 case 8: launch_full<8>(a, vir, shifts, sys, st); break;
                 case 16: launch_full<16>(a, vir, shifts, sys, st); break;

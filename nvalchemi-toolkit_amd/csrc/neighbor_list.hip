@@ -394,6 +394,38 @@ __device__ __forceinline__ float uniform_f(float v) {
     return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
 }
 
+// Shift of candidate k relative to the centre atom: packed fast path, or (wide shifts) recovered
+// from the sorted arrays through the stencil tables of the current batch.
+struct ShiftSource {
+    const int* c_pk;
+    const int* st_prefix;
+    const int* st_start;
+    const int (*st_q)[3];
+    const int4* sorted_aux;
+    int t0;
+};
+
+__device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, int wi0, int wi1, int wi2,
+                                                int& s0, int& s1, int& s2) {
+    const int pk = src.c_pk[k];
+    if (pk & kPackOverflow) {
+        int flat = src.t0 + k, lo = 0, hi = kStencilBatch;
+        for (int it = 0; it < 6; ++it) {
+            int mid = (lo + hi) >> 1;
+            if (src.st_prefix[mid] <= flat) lo = mid; else hi = mid;
+        }
+        int4 w = src.sorted_aux[src.st_start[lo] + (flat - src.st_prefix[lo])];
+        s0 = src.st_q[lo][0] - w.x + wi0;
+        s1 = src.st_q[lo][1] - w.y + wi1;
+        s2 = src.st_q[lo][2] - w.z + wi2;
+    } else {
+        s0 = (pk & 1023) - 512 + wi0;
+        s1 = ((pk >> 10) & 1023) - 512 + wi1;
+        s2 = ((pk >> 20) & 1023) - 512 + wi2;
+    }
+}
+
+template <bool HALF>
 __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
     __shared__ float4 c_pos[kTile];           // cell-local xyz of a candidate + its atom index
     __shared__ int c_pk[kTile];               // packed (image of its cell - its own wrap)
@@ -431,6 +463,7 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
         const int R0 = S.R[0], R1 = S.R[1], R2 = S.R[2];
         const int e1 = 2 * R1 + 1, e2 = 2 * R2 + 1;
         const int n_stencil = (2 * R0 + 1) * e1 * e2;
+        const int e_self = (R0 * e1 + R1) * e2 + R2;  // the stencil entry that is the centre cell itself
         const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
 
         for (int cc0 = 0; cc0 < n_center; cc0 += kCenterChunk) {
@@ -478,28 +511,41 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                 }
                 __syncthreads();
                 const int batch_total = st_prefix[kStencilBatch];
+                const int n_entries = (n_stencil - sb) < kStencilBatch ? (n_stencil - sb) : kStencilBatch;
+                // where the centre cell's own atoms sit in the flattened batch (-1: not in this batch)
+                const int self_flat0 = (e_self >= sb && e_self < sb + kStencilBatch) ? st_prefix[e_self - sb] + cc0 : -1;
 
                 for (int t0 = 0; t0 < batch_total; t0 += kTile) {
                     const int tile_n = (batch_total - t0) < kTile ? (batch_total - t0) : kTile;
-                    // ---- stage the tile: candidate -> stencil entry by binary search
-                    for (int k = threadIdx.x; k < tile_n; k += kBlock) {
-                        int flat = t0 + k;
-                        int lo = 0, hi = kStencilBatch;  // prefix[lo] <= flat < prefix[hi]
-#pragma unroll
-                        for (int it = 0; it < 6; ++it) {
-                            int mid = (lo + hi) >> 1;
-                            if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
+                    const int tile_pad = (tile_n + kWave - 1) & ~(kWave - 1);
+                    // ---- stage the tile: each wave copies whole stencil cells (contiguous in the
+                    //      sorted arrays) and shifts them by the cell's offset
+                    for (int e = wave; e < n_entries; e += kWavesPerBlock) {
+                        const int p0 = st_prefix[e], p1 = st_prefix[e + 1];
+                        const int lo_flat = p0 > t0 ? p0 : t0;
+                        const int hi_flat = p1 < t0 + tile_n ? p1 : t0 + tile_n;
+                        if (lo_flat >= hi_flat) continue;
+                        const int src0 = st_start[e] - p0;
+                        const float o0 = st_off[e][0], o1 = st_off[e][1], o2 = st_off[e][2];
+                        const int q0 = st_q[e][0], q1 = st_q[e][1], q2 = st_q[e][2];
+                        for (int flat = lo_flat + lane; flat < hi_flat; flat += kWave) {
+                            float4 p = ws.sorted_pos[src0 + flat];
+                            int4 w = ws.sorted_aux[src0 + flat];
+                            p.x += o0;
+                            p.y += o1;
+                            p.z += o2;
+                            c_pos[flat - t0] = p;
+                            c_pk[flat - t0] = pack_shift(q0 - w.x, q1 - w.y, q2 - w.z);
                         }
-                        int slot = st_start[lo] + (flat - st_prefix[lo]);
-                        float4 p = ws.sorted_pos[slot];
-                        int4 w = ws.sorted_aux[slot];
-                        p.x += st_off[lo][0];
-                        p.y += st_off[lo][1];
-                        p.z += st_off[lo][2];
-                        c_pos[k] = p;
-                        c_pk[k] = pack_shift(st_q[lo][0] - w.x, st_q[lo][1] - w.y, st_q[lo][2] - w.z);
                     }
+                    // padding up to a multiple of 64: candidates that no centre atom can reach
+                    if ((int)threadIdx.x < tile_pad - tile_n)
+                        c_pos[tile_n + threadIdx.x] = make_float4(3.0e38f, 0.f, 0.f, __int_as_float(-1));
                     __syncthreads();
+
+                    // the usual case, one batch and one tile: rows are finished right here
+                    const bool last_tile = (n_stencil <= kStencilBatch) && (batch_total <= kTile);
+                    const ShiftSource shifts{c_pk, st_prefix, st_start, st_q, ws.sorted_aux, t0};
 
                     // ---- each wave: its centre atoms against the tile, 64 candidates a step
                     for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
@@ -510,35 +556,21 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                         const int wi0 = __builtin_amdgcn_readfirstlane(wa.x);
                         const int wi1 = __builtin_amdgcn_readfirstlane(wa.y);
                         const int wi2 = __builtin_amdgcn_readfirstlane(wa.z);
-                        const int self_pk = pack_shift(-wi0, -wi1, -wi2);  // shift 0 <=> q - w_j == -w_i
+                        const int old_cnt = last_tile ? a.nn[i_atom] : 0;  // needed only at the end: load early
                         int32_t* row = a.nm + (size_t)i_atom * a.K;
                         int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
-                        int base = __builtin_amdgcn_readfirstlane(row_cnt[ca]);  // entries found before this tile
+                        int base = __builtin_amdgcn_readfirstlane(row_cnt[ca]);  // found before this tile
                         int nh = 0;                                               // entries in the hit list
                         unsigned short* my_hits = hits[wave];
+                        // the centre atom meets itself (shift 0) at exactly one tile slot
+                        const int k_self = (self_flat0 >= 0) ? self_flat0 + ca - t0 : -1;
 
                         auto flush = [&]() {
                             for (int l = lane; l < nh; l += kWave) {
                                 const int k = my_hits[l];
                                 const int j = __float_as_int(c_pos[k].w);
-                                int pk = c_pk[k];
                                 int s0, s1, s2;
-                                if (pk & kPackOverflow) {
-                                    // wide shift: recover it from the sorted arrays
-                                    int flat = t0 + k, lo = 0, hi = kStencilBatch;
-                                    for (int it = 0; it < 6; ++it) {
-                                        int mid = (lo + hi) >> 1;
-                                        if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
-                                    }
-                                    int4 w = ws.sorted_aux[st_start[lo] + (flat - st_prefix[lo])];
-                                    s0 = st_q[lo][0] - w.x + wi0;
-                                    s1 = st_q[lo][1] - w.y + wi1;
-                                    s2 = st_q[lo][2] - w.z + wi2;
-                                } else {
-                                    s0 = (pk & 1023) - 512 + wi0;
-                                    s1 = ((pk >> 10) & 1023) - 512 + wi1;
-                                    s2 = ((pk >> 20) & 1023) - 512 + wi2;
-                                }
+                                candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
                                 const int slot = base + l;
                                 if (slot < a.K) {
                                     row[slot] = j;
@@ -553,99 +585,89 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                             nh = 0;
                         };
 
-                        for (int k0 = 0; k0 < tile_n; k0 += kWave) {
+                        for (int k0 = 0; k0 < tile_pad; k0 += kWave) {
                             const int k = k0 + lane;
-                            const int kk = k < tile_n ? k : tile_n - 1;
-                            const float4 p = c_pos[kk];
+                            const float4 p = c_pos[k];
                             const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
                             const float d2 = dx * dx + dy * dy + dz * dz;
-                            const int j = __float_as_int(p.w);
-                            bool in = (k < tile_n) && (d2 < rc2_hi);
-                            const bool special = in && (!(d2 < rc2_lo) || j == i_atom);
-                            if (__builtin_amdgcn_ballot_w64(special)) {
-                                if (special) {
-                                    int pk = c_pk[kk];
-                                    if (j == i_atom && pk == self_pk && !(pk & kPackOverflow)) in = false;
-                                    if (in && !(d2 < rc2_lo)) {
-                                        // inside the float32 uncertainty band: decide exactly
-                                        int s0, s1, s2;
-                                        if (pk & kPackOverflow) {
-                                            int flat = t0 + kk, lo = 0, hi = kStencilBatch;
-                                            for (int it = 0; it < 6; ++it) {
-                                                int mid = (lo + hi) >> 1;
-                                                if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
-                                            }
-                                            int4 w = ws.sorted_aux[st_start[lo] + (flat - st_prefix[lo])];
-                                            s0 = st_q[lo][0] - w.x + wi0;
-                                            s1 = st_q[lo][1] - w.y + wi1;
-                                            s2 = st_q[lo][2] - w.z + wi2;
-                                        } else {
-                                            s0 = (pk & 1023) - 512 + wi0;
-                                            s1 = ((pk >> 10) & 1023) - 512 + wi1;
-                                            s2 = ((pk >> 20) & 1023) - 512 + wi2;
-                                        }
-                                        const float* pi = a.pos + 3 * (size_t)i_atom;
-                                        const float* pj = a.pos + 3 * (size_t)j;
-                                        double e0, e1d, e2d;
-                                        double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0,
-                                                                  s1, s2, ws.sys[sidx].h, e0, e1d, e2d);
-                                        in = r2 < a.rc2;
-                                        if (j == i_atom && s0 == 0 && s1 == 0 && s2 == 0) in = false;
-                                    }
+                            bool in = (d2 < rc2_hi) && (k != k_self);
+                            const bool band = in && !(d2 < rc2_lo);
+                            if (__builtin_amdgcn_ballot_w64(band)) {
+                                if (band) {
+                                    // inside the float32 uncertainty band: decide exactly
+                                    const int j = __float_as_int(p.w);
+                                    int s0, s1, s2;
+                                    candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
+                                    const float* pi = a.pos + 3 * (size_t)i_atom;
+                                    const float* pj = a.pos + 3 * (size_t)j;
+                                    double e0, e1d, e2d;
+                                    double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1, s2,
+                                                              ws.sys[sidx].h, e0, e1d, e2d);
+                                    in = r2 < a.rc2;
                                 }
                             }
-                            if (a.half) {
+                            if (HALF) {
+                                const int j = __float_as_int(p.w);
                                 if (j == i_atom) {
-                                    // self image: keep the lexicographically positive shift
-                                    int pk = c_pk[kk];
-                                    int s0 = (pk & 1023) - 512 + wi0, s1 = ((pk >> 10) & 1023) - 512 + wi1,
-                                        s2 = ((pk >> 20) & 1023) - 512 + wi2;
-                                    if (pk & kPackOverflow) {
-                                        int flat = t0 + kk, lo = 0, hi = kStencilBatch;
-                                        for (int it = 0; it < 6; ++it) {
-                                            int mid = (lo + hi) >> 1;
-                                            if (st_prefix[mid] <= flat) lo = mid; else hi = mid;
-                                        }
-                                        int4 w = ws.sorted_aux[st_start[lo] + (flat - st_prefix[lo])];
-                                        s0 = st_q[lo][0] - w.x + wi0;
-                                        s1 = st_q[lo][1] - w.y + wi1;
-                                        s2 = st_q[lo][2] - w.z + wi2;
+                                    if (in) {  // a periodic image of the centre atom: keep the positive shift
+                                        int s0, s1, s2;
+                                        candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
+                                        in = half_keep(i_atom, j, s0, s1, s2);
                                     }
-                                    in = in && half_keep(i_atom, j, s0, s1, s2);
                                 } else {
                                     in = in && (i_atom < j);
                                 }
                             }
                             const unsigned long long m = __builtin_amdgcn_ballot_w64(in);
-                            if (in) my_hits[nh + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0))] = (unsigned short)k;
+                            if (in) {
+                                const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                             __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                my_hits[nh + before] = (unsigned short)k;
+                            }
                             nh += __popcll(m);
                             if (nh > kHitCap - kWave) flush();
                         }
                         flush();
-                        if (lane == 0) row_cnt[ca] = base;
+                        if (last_tile) {
+                            // ---- count, and padding over what the previous build left beyond it
+                            const int hi_slot = a.tail_mode ? a.K : (old_cnt < a.K ? old_cnt : a.K);
+                            for (int k = base + lane; k < hi_slot; k += kWave) {
+                                row[k] = a.n_atoms;
+                                if (srow) {
+                                    srow[3 * k + 0] = 0;
+                                    srow[3 * k + 1] = 0;
+                                    srow[3 * k + 2] = 0;
+                                }
+                            }
+                            if (lane == 0) a.nn[i_atom] = base;
+                        } else if (lane == 0) {
+                            row_cnt[ca] = base;
+                        }
                     }
                     __syncthreads();
                 }
-                __syncthreads();  // everyone has read this batch's totals before wave 0 rewrites them
+                __syncthreads();  // everyone has read this batch's tables before wave 0 rewrites them
             }
 
-            // ---- counts, and padding over what the previous build left beyond them
-            for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
-                const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ca_pos[ca].w));
-                const int cnt = __builtin_amdgcn_readfirstlane(row_cnt[ca]);
-                const int old_cnt = a.nn[i_atom];
-                int32_t* row = a.nm + (size_t)i_atom * a.K;
-                int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
-                const int hi_slot = a.tail_mode ? a.K : (old_cnt < a.K ? old_cnt : a.K);
-                for (int k = cnt + lane; k < hi_slot; k += kWave) {
-                    row[k] = a.n_atoms;
-                    if (srow) {
-                        srow[3 * k + 0] = 0;
-                        srow[3 * k + 1] = 0;
-                        srow[3 * k + 2] = 0;
+            if (n_stencil > kStencilBatch || st_prefix[kStencilBatch] > kTile) {
+                // several batches or tiles: counts were carried in LDS, finish the rows now
+                for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
+                    const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ca_pos[ca].w));
+                    const int cnt = __builtin_amdgcn_readfirstlane(row_cnt[ca]);
+                    const int old_cnt = a.nn[i_atom];
+                    int32_t* row = a.nm + (size_t)i_atom * a.K;
+                    int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
+                    const int hi_slot = a.tail_mode ? a.K : (old_cnt < a.K ? old_cnt : a.K);
+                    for (int k = cnt + lane; k < hi_slot; k += kWave) {
+                        row[k] = a.n_atoms;
+                        if (srow) {
+                            srow[3 * k + 0] = 0;
+                            srow[3 * k + 1] = 0;
+                            srow[3 * k + 2] = 0;
+                        }
                     }
+                    if (lane == 0) a.nn[i_atom] = cnt;
                 }
-                if (lane == 0) a.nn[i_atom] = cnt;
             }
             __syncthreads();
         }
@@ -724,7 +746,8 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     unsigned n_search = 8u * 2048u;
     size_t cells_bound = max_cells_for(n_atoms, n_systems);
     if (cells_bound < n_search) n_search = (unsigned)((cells_bound + 7) / 8 * 8);
-    hipLaunchKernelGGL(nl_search_kernel, dim3(n_search), blk, 0, st, a, ws);
+    if (a.half) hipLaunchKernelGGL(nl_search_kernel<true>, dim3(n_search), blk, 0, st, a, ws);
+    else hipLaunchKernelGGL(nl_search_kernel<false>, dim3(n_search), blk, 0, st, a, ws);
     NVAMD_LAUNCH_CHECK("neighbor list launch");
     return NVAMD_OK;
 }
