@@ -133,6 +133,7 @@ struct NlArgs {
     const int32_t* bidx;
     const uint8_t* rebuild;
     int n_atoms, n_systems, K, half, tail_mode;
+    int dbg;  // experiment switches (0 in production)
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -565,35 +566,57 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                         // the centre atom meets itself (shift 0) at exactly one tile slot
                         const int k_self = (self_flat0 >= 0) ? self_flat0 + ca - t0 : -1;
 
+                        // The centre atom always "finds" itself (distance 0, shift 0) at tile slot
+                        // k_self; that entry is dropped when the hit list is written out, which keeps
+                        // the test out of the per-candidate loop.
                         auto flush = [&]() {
-                            for (int l = lane; l < nh; l += kWave) {
-                                const int k = my_hits[l];
-                                const int j = __float_as_int(c_pos[k].w);
-                                int s0, s1, s2;
-                                candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
-                                const int slot = base + l;
-                                if (slot < a.K) {
-                                    row[slot] = j;
-                                    if (srow) {
-                                        srow[3 * slot + 0] = s0;
-                                        srow[3 * slot + 1] = s1;
-                                        srow[3 * slot + 2] = s2;
+                            int removed = 0;  // 1 once the self entry has been passed
+                            for (int l0 = 0; l0 < nh; l0 += kWave) {
+                                const int l = l0 + lane;
+                                const bool live = l < nh;
+                                const int k = live ? my_hits[l] : -2;
+                                const unsigned long long ms = __builtin_amdgcn_ballot_w64(live && k == k_self);
+                                const int self_l = ms ? l0 + (int)__builtin_ctzll(ms) : 0x7fffffff;
+                                if (live && k != k_self && !(a.dbg & 2)) {
+                                    const int j = __float_as_int(c_pos[k].w);
+                                    int s0, s1, s2;
+                                    candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
+                                    const int slot = base + l - removed - (l > self_l ? 1 : 0);
+                                    if (slot < a.K) {
+                                        row[slot] = j;
+                                        if (srow) {
+                                            srow[3 * slot + 0] = s0;
+                                            srow[3 * slot + 1] = s1;
+                                            srow[3 * slot + 2] = s2;
+                                        }
                                     }
                                 }
+                                if (ms) removed = 1;
                             }
-                            base += nh;
+                            base += nh - removed;
                             nh = 0;
                         };
 
-                        for (int k0 = 0; k0 < tile_pad; k0 += kWave) {
+                        const char* lds_addr = reinterpret_cast<const char*>(c_pos) + lane * sizeof(float4);
+                        for (int k0 = (a.dbg & 4) ? tile_pad : 0; k0 < tile_pad; k0 += kWave, lds_addr += kWave * sizeof(float4)) {
                             const int k = k0 + lane;
-                            const float4 p = c_pos[k];
+                            const float4 p = *reinterpret_cast<const float4*>(lds_addr);
                             const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
                             const float d2 = dx * dx + dy * dy + dz * dz;
-                            bool in = (d2 < rc2_hi) && (k != k_self);
-                            const bool band = in && !(d2 < rc2_lo);
-                            if (__builtin_amdgcn_ballot_w64(band)) {
-                                if (band) {
+                            const unsigned long long m_hi = __builtin_amdgcn_ballot_w64(d2 < rc2_hi);
+                            const unsigned long long m_lo = __builtin_amdgcn_ballot_w64(d2 < rc2_lo);
+                            unsigned long long m;
+                            if (!HALF && m_hi == m_lo) {
+                                // the usual step: nobody is inside the uncertainty band
+                                m = m_lo;
+                                if (d2 < rc2_lo && !(a.dbg & 1)) {
+                                    const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                                 __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                    my_hits[nh + before] = (unsigned short)k;
+                                }
+                            } else {
+                                bool in = d2 < rc2_hi;
+                                if (in && !(d2 < rc2_lo) && k != k_self) {
                                     // inside the float32 uncertainty band: decide exactly
                                     const int j = __float_as_int(p.w);
                                     int s0, s1, s2;
@@ -605,24 +628,22 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                                                               ws.sys[sidx].h, e0, e1d, e2d);
                                     in = r2 < a.rc2;
                                 }
-                            }
-                            if (HALF) {
-                                const int j = __float_as_int(p.w);
-                                if (j == i_atom) {
-                                    if (in) {  // a periodic image of the centre atom: keep the positive shift
+                                if (HALF && in && k != k_self) {
+                                    const int j = __float_as_int(p.w);
+                                    if (j == i_atom) {  // a periodic image of the centre atom: keep the positive shift
                                         int s0, s1, s2;
                                         candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
                                         in = half_keep(i_atom, j, s0, s1, s2);
+                                    } else {
+                                        in = i_atom < j;
                                     }
-                                } else {
-                                    in = in && (i_atom < j);
                                 }
-                            }
-                            const unsigned long long m = __builtin_amdgcn_ballot_w64(in);
-                            if (in) {
-                                const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
-                                                                             __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-                                my_hits[nh + before] = (unsigned short)k;
+                                m = __builtin_amdgcn_ballot_w64(in);
+                                if (in) {
+                                    const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                                 __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                    my_hits[nh + before] = (unsigned short)k;
+                                }
                             }
                             nh += __popcll(m);
                             if (nh > kHitCap - kWave) flush();
@@ -723,6 +744,7 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     a.K = max_neighbors;
     a.half = half_fill ? 1 : 0;
     a.tail_mode = tail_mode ? 1 : 0;
+    { static int d = [] { const char* e = getenv("NVAMD_NL_DBG"); return e ? atoi(e) : 0; }(); a.dbg = d; }
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
