@@ -31,11 +31,13 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kTile = 768;        // candidates staged in LDS at a time
+constexpr int kTile = 960;        // candidates staged in LDS at a time
 constexpr int kStencilBatch = 64; // stencil cells enumerated at a time (one per lane of a wave)
-constexpr int kCenterChunk = 64;  // centre atoms of a cell handled per pass
-constexpr int kHitCap = 256;      // per-wave list of accepted candidates before it is written out
+constexpr int kCenterChunk = 96;  // centre atoms of a run of cells handled per pass
+constexpr int kMaxRun = 4;        // a workgroup's unit of work: up to this many cells in a row along z
+constexpr int kHitCap = 320;      // per-wave list of accepted candidates before it is written out
 constexpr int kPackOverflow = 1 << 30;
+static_assert(kMaxRun <= 4, "a centre atom's place in its run is kept in two bits");
 constexpr int kMaxCellsPerAxis = 1024;
 constexpr int kMinCellCap = 8;    // a system may use at least this many cells
 constexpr int kMaxStencilRadius = 32;  // cells searched per axis and direction, at most
@@ -53,6 +55,8 @@ struct NlSys {
     int per[3];
     int cell_offset;
     int n_cells;
+    int zr;            // cells per run along axis 2 (the search's unit of work)
+    int n_units;       // runs in this system
     int atom_begin, atom_end;
 };
 
@@ -64,12 +68,14 @@ struct NlSearchSys {
     int R[3];
     int per[3];
     int cell_offset;
+    int zr;
 };
 
 struct NlHeader {
     int total_cells;
     int error;  // bit 0: a system's cell is degenerate or narrower than cutoff/kMaxStencilRadius
-    int pad[14];
+    int total_units;
+    int pad[13];
 };
 
 struct NlWorkspace {
@@ -78,8 +84,8 @@ struct NlWorkspace {
     uint32_t* bounds;    // (B,6) order keys: min x,y,z then max x,y,z
     NlSearchSys* ssys;   // (B)
     int* cell_offset;    // (B+1)
-    int* cell_sys;       // (C) system of each non-empty cell
-    int* atom_cell;      // (N)
+    int* unit_offset;    // (B+1) first unit of each system
+    int2* units;         // (C) per unit of search work: first cell of the run, system
     int* atom_rank;      // (N)
     int* cell_count;     // (C)
     int* cell_start;     // (C+1)
@@ -110,8 +116,8 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
     p = take(B * 6 * sizeof(uint32_t)); if (ws) ws->bounds = reinterpret_cast<uint32_t*>(p);
     p = take(B * sizeof(NlSearchSys)); if (ws) ws->ssys = reinterpret_cast<NlSearchSys*>(p);
     p = take((B + 1) * sizeof(int)); if (ws) ws->cell_offset = reinterpret_cast<int*>(p);
-    p = take(C * sizeof(int)); if (ws) ws->cell_sys = reinterpret_cast<int*>(p);
-    p = take(N * sizeof(int)); if (ws) ws->atom_cell = reinterpret_cast<int*>(p);
+    p = take((B + 1) * sizeof(int)); if (ws) ws->unit_offset = reinterpret_cast<int*>(p);
+    p = take(C * sizeof(int2)); if (ws) ws->units = reinterpret_cast<int2*>(p);
     p = take(N * sizeof(int)); if (ws) ws->atom_rank = reinterpret_cast<int*>(p);
     p = take(C * sizeof(int)); if (ws) ws->cell_count = reinterpret_cast<int*>(p);
     p = take((C + 1) * sizeof(int)); if (ws) ws->cell_start = reinterpret_cast<int*>(p);
@@ -133,7 +139,6 @@ struct NlArgs {
     const int32_t* bidx;
     const uint8_t* rebuild;
     int n_atoms, n_systems, K, half, tail_mode;
-    int dbg;  // experiment switches (0 in production)
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -217,13 +222,15 @@ __global__ __launch_bounds__(kBlock) void nl_bounds_kernel(NlArgs a, NlWorkspace
 
 // ---- 3 grid ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws) {
-    __shared__ int s_scan[1024];
-    __shared__ int s_carry;
+    // low word: cells, high word: search units (both totals stay below 2^31, so the packed
+    // sums never carry into each other)
+    __shared__ unsigned long long s_scan[1024];
+    __shared__ unsigned long long s_carry;
     if (threadIdx.x == 0) s_carry = 0;
     __syncthreads();
     for (int base = 0; base < a.n_systems; base += 1024) {
         int t = base + threadIdx.x;
-        int ncell = 0;
+        int ncell = 0, nunit = 0;
         if (t < a.n_systems) {
             NlSys s = ws.sys[t];
             int n_at = s.atom_end - s.atom_begin;
@@ -250,7 +257,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
                 if (s.nc[m] == 1) break;
                 s.nc[m] = (s.nc[m] + 1) / 2;
             }
-            double reach = 0.0;  // largest cell-local coordinate the search can meet
+            double len[3];
             for (int d = 0; d < 3; ++d) {
                 double cw = s.ext[d] * s.width[d] / s.nc[d];
                 int R;
@@ -266,33 +273,57 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
                 }
                 s.R[d] = R;
                 double sc = s.ext[d] / s.nc[d];
-                double len = 0.0;
+                double l2 = 0.0;
                 for (int k = 0; k < 3; ++k) {
                     s.step[3 * d + k] = sc * s.h[3 * d + k];
-                    len += s.step[3 * d + k] * s.step[3 * d + k];
+                    l2 += s.step[3 * d + k] * s.step[3 * d + k];
                 }
-                reach += (R + 1) * sqrt(len);
+                len[d] = sqrt(l2);
             }
-            s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
             s.n_cells = n_at > 0 ? s.nc[0] * s.nc[1] * s.nc[2] : 0;
+            // Run length along axis 2: as long as the run's whole stencil is expected to fit one
+            // batch of stencil cells and one LDS tile, and its centre atoms one pass.
+            int zr = 1;
+            if (s.n_cells > 0) {
+                const double per_cell = 1.2 * (double)n_at / (double)s.n_cells;
+                const int e01 = (2 * s.R[0] + 1) * (2 * s.R[1] + 1);
+                for (int cand = 2; cand <= kMaxRun && cand <= s.nc[2]; ++cand) {
+                    const int entries = (cand + 2 * s.R[2]) * e01;
+                    if (entries > kStencilBatch) break;
+                    if (entries * per_cell + kWave > (double)kTile) break;
+                    if (cand * per_cell > (double)kCenterChunk) break;
+                    zr = cand;
+                }
+                const int runs = (s.nc[2] + zr - 1) / zr;
+                zr = (s.nc[2] + runs - 1) / runs;  // same number of runs, evened out
+            }
+            s.zr = zr;
+            s.n_units = s.n_cells > 0 ? s.nc[0] * s.nc[1] * ((s.nc[2] + zr - 1) / zr) : 0;
+            // largest cell-local coordinate the search can meet
+            const double reach = (s.R[0] + 1) * len[0] + (s.R[1] + 1) * len[1] + (s.R[2] + zr) * len[2];
+            s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
             ncell = s.n_cells;
+            nunit = s.n_units;
             ws.sys[t] = s;
         }
-        // exclusive scan of ncell over the 1024 systems of this pass
-        s_scan[threadIdx.x] = ncell;
+        // exclusive scan of both counts over the 1024 systems of this pass
+        const unsigned long long mine = (unsigned long long)(unsigned)ncell | ((unsigned long long)(unsigned)nunit << 32);
+        s_scan[threadIdx.x] = mine;
         __syncthreads();
         for (int o = 1; o < 1024; o <<= 1) {
-            int v = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0;
+            unsigned long long v = (int)threadIdx.x >= o ? s_scan[threadIdx.x - o] : 0ull;
             __syncthreads();
             s_scan[threadIdx.x] += v;
             __syncthreads();
         }
-        int incl = s_scan[threadIdx.x];
-        int carry = s_carry;
+        const unsigned long long incl = s_scan[threadIdx.x];
+        const unsigned long long carry = s_carry;
         if (t < a.n_systems) {
-            const int off = carry + incl - ncell;
+            const unsigned long long excl = carry + incl - mine;
+            const int off = (int)(unsigned)(excl & 0xffffffffull);
             ws.sys[t].cell_offset = off;
             ws.cell_offset[t] = off;
+            ws.unit_offset[t] = (int)(unsigned)(excl >> 32);
             const NlSys& s = ws.sys[t];
             NlSearchSys q;
             for (int k = 0; k < 9; ++k) q.step[k] = (float)s.step[k];
@@ -303,6 +334,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
                 q.per[d] = s.per[d];
             }
             q.cell_offset = off;
+            q.zr = s.zr;
             ws.ssys[t] = q;
         }
         __syncthreads();
@@ -310,8 +342,11 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        ws.cell_offset[a.n_systems] = s_carry;
-        ws.hdr->total_cells = s_carry;
+        const unsigned long long tot = s_carry;
+        ws.cell_offset[a.n_systems] = (int)(unsigned)(tot & 0xffffffffull);
+        ws.unit_offset[a.n_systems] = (int)(unsigned)(tot >> 32);
+        ws.hdr->total_cells = (int)(unsigned)(tot & 0xffffffffull);
+        ws.hdr->total_units = (int)(unsigned)(tot >> 32);
     }
 }
 
@@ -351,14 +386,26 @@ __device__ __forceinline__ Binned bin_atom(const NlSys& s, const float* __restri
     return b;
 }
 
+// Launched over max(atoms, cell bound) threads: thread t bins atom t and describes search unit t.
 __global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws) {
     int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < ws.hdr->total_units) {
+        // the system that owns unit i: the last one whose first unit is <= i
+        int lo = 0, hi = a.n_systems;
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (ws.unit_offset[mid] <= i) lo = mid; else hi = mid;
+        }
+        const NlSearchSys& q = ws.ssys[lo];
+        const int lu = i - ws.unit_offset[lo];
+        const int runs = (q.nc[2] + q.zr - 1) / q.zr;
+        const int column = lu / runs, run = lu - column * runs;
+        ws.units[i] = make_int2(q.cell_offset + column * q.nc[2] + run * q.zr, lo);
+    }
     if (i >= a.n_atoms) return;
     const NlSys& s = ws.sys[a.bidx[i]];
     Binned b = bin_atom(s, a.pos + 3 * (size_t)i);
-    ws.atom_cell[i] = b.cell;
     ws.atom_rank[i] = atomicAdd(ws.cell_count + b.cell, 1);
-    ws.cell_sys[b.cell] = a.bidx[i];
 }
 
 __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspace ws) {
@@ -426,53 +473,84 @@ __device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, i
     }
 }
 
+// A workgroup's unit of work is a run of up to kMaxRun cells that follow each other along
+// axis 2 (they are consecutive cell ids, so their atoms are one contiguous slice of the
+// sorted arrays).  The run's stencil is enumerated layer by layer along axis 2, so the
+// candidates a centre cell of the run has to look at are one contiguous range of the LDS tile;
+// what a range picks up beyond its own layers (ranges are widened to multiples of 64) lies
+// further than the stencil radius away and can never pass the distance test.
 template <bool HALF>
-__global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
-    __shared__ float4 c_pos[kTile];           // cell-local xyz of a candidate + its atom index
+__global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
+    __shared__ float4 c_pos[kTile];           // candidate: xyz relative to the run's first cell + atom index
     __shared__ int c_pk[kTile];               // packed (image of its cell - its own wrap)
-    __shared__ float4 ca_pos[kCenterChunk];   // centre atoms of this pass: local xyz + atom index
-    __shared__ int4 ca_w[kCenterChunk];       // their wrap integers
-    __shared__ int row_cnt[kCenterChunk];     // running row lengths
+    __shared__ float4 ca_pos[kCenterChunk];   // centre atoms of this pass: same frame + atom index
+    __shared__ int4 ca_w[kCenterChunk];       // their wrap integers; .w = place of their cell in the run | pad end << 2
+    __shared__ int4 ca_meta[kCenterChunk];    // per batch of stencil cells: flat slot of the centre itself, first and
+                                              // last candidate to scan; .w = running row length
     __shared__ int st_start[kStencilBatch];
     __shared__ int st_prefix[kStencilBatch + 1];
     __shared__ int st_q[kStencilBatch][3];
     __shared__ float st_off[kStencilBatch][3];
     __shared__ unsigned short hits[kWavesPerBlock][kHitCap];
 
-    const int total_cells = ws.hdr->total_cells;
+    const int total_units = ws.hdr->total_units;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
     const float rc2f = (float)a.rc2;
     // each XCD (consecutive workgroups go to the 8 XCDs round-robin) walks one contiguous
-    // eighth of the cells, so the stencil data it re-reads stays in its own L2
+    // eighth of the units, so the stencil data it re-reads stays in its own L2
     const int xcd = blockIdx.x % 8, slot0 = blockIdx.x / 8, stride = gridDim.x / 8;
-    const int per_xcd = (total_cells + 7) / 8;
+    const int per_xcd = (total_units + 7) / 8;
 
     for (int li = slot0; li < per_xcd; li += stride) {
         // NOTE: every thread of the workgroup takes the same path through this loop body
-        const int c = xcd * per_xcd + li;
-        if (c >= total_cells) break;
-        const int c_begin = ws.cell_start[c];
-        const int n_center = ws.cell_start[c + 1] - c_begin;
-        if (n_center == 0) continue;
-        const int sidx = __builtin_amdgcn_readfirstlane(ws.cell_sys[c]);
+        const int u = xcd * per_xcd + li;
+        if (u >= total_units) break;
+        const int2 unit = ws.units[u];
+        const int c0 = __builtin_amdgcn_readfirstlane(unit.x);
+        const int sidx = __builtin_amdgcn_readfirstlane(unit.y);
         if (a.rebuild && !a.rebuild[sidx]) continue;
         const NlSearchSys S = ws.ssys[sidx];
-        const int lc = c - S.cell_offset;
+        const int lc = c0 - S.cell_offset;
         const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
-        const int cz = lc % nc2, cy = (lc / nc2) % nc1, cx = lc / (nc2 * nc1);
+        const int cz0 = lc % nc2, cy = (lc / nc2) % nc1, cx = lc / (nc2 * nc1);
+        const int run_len = (nc2 - cz0) < S.zr ? (nc2 - cz0) : S.zr;
+        const int c_begin = ws.cell_start[c0];
+        // first centre atom (relative to c_begin) of the run's cells 1, 2, 3 and the run's end
+        int run_off[kMaxRun + 1];
+        run_off[0] = 0;
+#pragma unroll
+        for (int r = 1; r <= kMaxRun; ++r) run_off[r] = ws.cell_start[c0 + (r < run_len ? r : run_len)] - c_begin;
+        const int n_center = run_off[kMaxRun];
+        if (n_center == 0) continue;
         const int R0 = S.R[0], R1 = S.R[1], R2 = S.R[2];
-        const int e1 = 2 * R1 + 1, e2 = 2 * R2 + 1;
-        const int n_stencil = (2 * R0 + 1) * e1 * e2;
-        const int e_self = (R0 * e1 + R1) * e2 + R2;  // the stencil entry that is the centre cell itself
+        const int e1 = 2 * R1 + 1, e01 = (2 * R0 + 1) * e1;
+        const int n_layers = run_len + 2 * R2;
+        const int n_stencil = n_layers * e01;
+        // one batch of stencil cells and (checked below) one tile: rows are finished in place and
+        // every centre atom scans only the layers of its own cell's stencil
+        const bool one_batch = n_stencil <= kStencilBatch;
         const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
 
         for (int cc0 = 0; cc0 < n_center; cc0 += kCenterChunk) {
             const int n_cc = (n_center - cc0) < kCenterChunk ? (n_center - cc0) : kCenterChunk;
             if ((int)threadIdx.x < n_cc) {
-                ca_pos[threadIdx.x] = ws.sorted_pos[c_begin + cc0 + threadIdx.x];
-                ca_w[threadIdx.x] = ws.sorted_aux[c_begin + cc0 + threadIdx.x];
-                row_cnt[threadIdx.x] = 0;
+                const int ca_abs = cc0 + (int)threadIdx.x;
+                int r = 0;
+#pragma unroll
+                for (int q = 1; q < kMaxRun; ++q) r += (ca_abs >= run_off[q]) ? 1 : 0;
+                float4 p = ws.sorted_pos[c_begin + ca_abs];
+                int4 w = ws.sorted_aux[c_begin + ca_abs];
+                const float fr = (float)r;
+                p.x += fr * S.step[6];
+                p.y += fr * S.step[7];
+                p.z += fr * S.step[8];
+                // what the row must be padded up to afterwards: all of it, or what the previous build left
+                const int old_cnt = a.tail_mode ? a.K : a.nn[__float_as_int(p.w)];
+                w.w = r | ((old_cnt < a.K ? old_cnt : a.K) << 2);
+                ca_pos[threadIdx.x] = p;
+                ca_w[threadIdx.x] = w;
+                ca_meta[threadIdx.x].w = 0;
             }
 
             for (int sb = 0; sb < n_stencil; sb += kStencilBatch) {
@@ -482,8 +560,9 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                     int start = 0, count = 0, q0 = 0, q1 = 0, q2 = 0;
                     float o0 = 0.f, o1 = 0.f, o2 = 0.f;
                     if (si < n_stencil) {
-                        int oz = si % e2 - R2, oy = (si / e2) % e1 - R1, ox = si / (e2 * e1) - R0;
-                        int gx = cx + ox, gy = cy + oy, gz = cz + oz;
+                        const int layer = si / e01, in_layer = si - layer * e01;
+                        const int oz = layer - R2, oy = in_layer % e1 - R1, ox = in_layer / e1 - R0;
+                        int gx = cx + ox, gy = cy + oy, gz = cz0 + oz;
                         bool ok = true;
                         if (S.per[0]) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
                         if (S.per[1]) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
@@ -513,30 +592,66 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                 __syncthreads();
                 const int batch_total = st_prefix[kStencilBatch];
                 const int n_entries = (n_stencil - sb) < kStencilBatch ? (n_stencil - sb) : kStencilBatch;
-                // where the centre cell's own atoms sit in the flattened batch (-1: not in this batch)
-                const int self_flat0 = (e_self >= sb && e_self < sb + kStencilBatch) ? st_prefix[e_self - sb] + cc0 : -1;
+                const bool fused = one_batch && batch_total <= kTile;
+                if ((int)threadIdx.x < n_cc) {
+                    // The centre atom meets itself (shift 0) at exactly one slot of the flattened
+                    // stencil: in its own cell, i.e. layer r + R2, at the middle of that layer.
+                    const int r = ca_w[threadIdx.x].w & 3;
+                    const int e_self = (r + R2) * e01 + R0 * e1 + R1;
+                    int self_flat = -1;
+                    if (e_self >= sb && e_self < sb + kStencilBatch) {
+                        int first_of_cell = 0;  // run_off[r] without dynamic indexing
+#pragma unroll
+                        for (int q = 1; q < kMaxRun; ++q) first_of_cell = (r == q) ? run_off[q] : first_of_cell;
+                        self_flat = st_prefix[e_self - sb] + (cc0 + (int)threadIdx.x - first_of_cell);
+                    }
+                    // candidates to scan: the centre's own layers when rows are finished in place
+                    int lo = 0, hi = 0x7fffffff;
+                    if (fused) {
+                        lo = st_prefix[r * e01] & ~(kWave - 1);
+                        hi = (st_prefix[(r + 2 * R2 + 1) * e01] + kWave - 1) & ~(kWave - 1);
+                    }
+                    ca_meta[threadIdx.x].x = self_flat;
+                    ca_meta[threadIdx.x].y = lo;
+                    ca_meta[threadIdx.x].z = hi;
+                }
 
                 for (int t0 = 0; t0 < batch_total; t0 += kTile) {
                     const int tile_n = (batch_total - t0) < kTile ? (batch_total - t0) : kTile;
                     const int tile_pad = (tile_n + kWave - 1) & ~(kWave - 1);
-                    // ---- stage the tile: each wave copies whole stencil cells (contiguous in the
-                    //      sorted arrays) and shifts them by the cell's offset
-                    for (int e = wave; e < n_entries; e += kWavesPerBlock) {
-                        const int p0 = st_prefix[e], p1 = st_prefix[e + 1];
-                        const int lo_flat = p0 > t0 ? p0 : t0;
-                        const int hi_flat = p1 < t0 + tile_n ? p1 : t0 + tile_n;
-                        if (lo_flat >= hi_flat) continue;
-                        const int src0 = st_start[e] - p0;
-                        const float o0 = st_off[e][0], o1 = st_off[e][1], o2 = st_off[e][2];
-                        const int q0 = st_q[e][0], q1 = st_q[e][1], q2 = st_q[e][2];
-                        for (int flat = lo_flat + lane; flat < hi_flat; flat += kWave) {
-                            float4 p = ws.sorted_pos[src0 + flat];
-                            int4 w = ws.sorted_aux[src0 + flat];
-                            p.x += o0;
-                            p.y += o1;
-                            p.z += o2;
-                            c_pos[flat - t0] = p;
-                            c_pk[flat - t0] = pack_shift(q0 - w.x, q1 - w.y, q2 - w.z);
+                    // ---- stage the tile: thread t takes flat candidates t, t + 256, ...; all of a
+                    //      thread's global loads are in flight together (indices are clamped rather
+                    //      than branched over), then shifted by the stencil cell's offset
+                    {
+                        constexpr int kPer = (kTile + kBlock - 1) / kBlock;
+                        float4 sp[kPer];
+                        int4 sw[kPer];
+                        int se[kPer];
+#pragma unroll
+                        for (int i = 0; i < kPer; ++i) {
+                            const int f = (int)threadIdx.x + i * kBlock;
+                            const int flat = t0 + (f < tile_n ? f : tile_n - 1);
+                            int e = 0;  // the stencil cell this candidate belongs to
+#pragma unroll
+                            for (int step = kStencilBatch / 2; step > 0; step >>= 1)
+                                if (st_prefix[e + step] <= flat) e += step;
+                            const int src = st_start[e] + (flat - st_prefix[e]);
+                            se[i] = e;
+                            sp[i] = ws.sorted_pos[src];
+                            sw[i] = ws.sorted_aux[src];
+                        }
+#pragma unroll
+                        for (int i = 0; i < kPer; ++i) {
+                            const int f = (int)threadIdx.x + i * kBlock;
+                            if (f < tile_n) {
+                                const int e = se[i];
+                                float4 p = sp[i];
+                                p.x += st_off[e][0];
+                                p.y += st_off[e][1];
+                                p.z += st_off[e][2];
+                                c_pos[f] = p;
+                                c_pk[f] = pack_shift(st_q[e][0] - sw[i].x, st_q[e][1] - sw[i].y, st_q[e][2] - sw[i].z);
+                            }
                         }
                     }
                     // padding up to a multiple of 64: candidates that no centre atom can reach
@@ -544,8 +659,6 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                         c_pos[tile_n + threadIdx.x] = make_float4(3.0e38f, 0.f, 0.f, __int_as_float(-1));
                     __syncthreads();
 
-                    // the usual case, one batch and one tile: rows are finished right here
-                    const bool last_tile = (n_stencil <= kStencilBatch) && (batch_total <= kTile);
                     const ShiftSource shifts{c_pk, st_prefix, st_start, st_q, ws.sorted_aux, t0};
 
                     // ---- each wave: its centre atoms against the tile, 64 candidates a step
@@ -557,18 +670,22 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                         const int wi0 = __builtin_amdgcn_readfirstlane(wa.x);
                         const int wi1 = __builtin_amdgcn_readfirstlane(wa.y);
                         const int wi2 = __builtin_amdgcn_readfirstlane(wa.z);
-                        const int old_cnt = last_tile ? a.nn[i_atom] : 0;  // needed only at the end: load early
+                        const int hi_slot = __builtin_amdgcn_readfirstlane(wa.w) >> 2;
+                        const int4 meta = ca_meta[ca];
+                        const int self_flat = __builtin_amdgcn_readfirstlane(meta.x);
+                        const int k_self = self_flat >= 0 ? self_flat - t0 : -1;
+                        const int k_lo = __builtin_amdgcn_readfirstlane(meta.y);
+                        const int k_hi_all = __builtin_amdgcn_readfirstlane(meta.z);
+                        const int k_hi = k_hi_all < tile_pad ? k_hi_all : tile_pad;
+                        int base = __builtin_amdgcn_readfirstlane(meta.w);  // found before this tile
                         int32_t* row = a.nm + (size_t)i_atom * a.K;
                         int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
-                        int base = __builtin_amdgcn_readfirstlane(row_cnt[ca]);  // found before this tile
-                        int nh = 0;                                               // entries in the hit list
+                        int nh = 0;                                         // entries in the hit list
                         unsigned short* my_hits = hits[wave];
-                        // the centre atom meets itself (shift 0) at exactly one tile slot
-                        const int k_self = (self_flat0 >= 0) ? self_flat0 + ca - t0 : -1;
 
-                        // The centre atom always "finds" itself (distance 0, shift 0) at tile slot
-                        // k_self; that entry is dropped when the hit list is written out, which keeps
-                        // the test out of the per-candidate loop.
+                        // The self entry (distance 0) is always accepted by the distance test; it is
+                        // dropped when the hit list is written out, which keeps that comparison out
+                        // of the per-candidate loop.
                         auto flush = [&]() {
                             int removed = 0;  // 1 once the self entry has been passed
                             for (int l0 = 0; l0 < nh; l0 += kWave) {
@@ -577,7 +694,7 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                                 const int k = live ? my_hits[l] : -2;
                                 const unsigned long long ms = __builtin_amdgcn_ballot_w64(live && k == k_self);
                                 const int self_l = ms ? l0 + (int)__builtin_ctzll(ms) : 0x7fffffff;
-                                if (live && k != k_self && !(a.dbg & 2)) {
+                                if (live && k != k_self) {
                                     const int j = __float_as_int(c_pos[k].w);
                                     int s0, s1, s2;
                                     candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
@@ -597,61 +714,73 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                             nh = 0;
                         };
 
-                        const char* lds_addr = reinterpret_cast<const char*>(c_pos) + lane * sizeof(float4);
-                        for (int k0 = (a.dbg & 4) ? tile_pad : 0; k0 < tile_pad; k0 += kWave, lds_addr += kWave * sizeof(float4)) {
-                            const int k = k0 + lane;
-                            const float4 p = *reinterpret_cast<const float4*>(lds_addr);
+                        // One step: 64 candidates against the centre atom.  Accepted candidates are
+                        // appended to the wave's hit list; the rare step that has a candidate inside the
+                        // float32 uncertainty band (or, for half lists, an image of the centre atom
+                        // itself) takes a second, exact look at those candidates only.
+                        auto dist2 = [&](const float4& p) {
                             const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
-                            const float d2 = dx * dx + dy * dy + dz * dz;
-                            const unsigned long long m_hi = __builtin_amdgcn_ballot_w64(d2 < rc2_hi);
-                            const unsigned long long m_lo = __builtin_amdgcn_ballot_w64(d2 < rc2_lo);
-                            unsigned long long m;
-                            if (!HALF && m_hi == m_lo) {
-                                // the usual step: nobody is inside the uncertainty band
-                                m = m_lo;
-                                if (d2 < rc2_lo && !(a.dbg & 1)) {
-                                    const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
-                                                                                 __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-                                    my_hits[nh + before] = (unsigned short)k;
-                                }
+                            return dx * dx + dy * dy + dz * dz;
+                        };
+                        auto accept = [&](const int k, const float4& p, const float d2) {
+                            const bool lo = d2 < rc2_lo, hi = d2 < rc2_hi;
+                            const bool take = HALF ? (lo && i_atom < __float_as_int(p.w)) : lo;
+                            const unsigned long long m = __builtin_amdgcn_ballot_w64(take);
+                            if (take) {
+                                const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                             __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                my_hits[nh + before] = (unsigned short)k;
+                            }
+                            nh += __popcll(m);
+                            bool rare;
+                            if (HALF) {
+                                rare = __builtin_amdgcn_ballot_w64(hi && (!lo || __float_as_int(p.w) == i_atom)) != 0ull;
                             } else {
-                                bool in = d2 < rc2_hi;
-                                if (in && !(d2 < rc2_lo) && k != k_self) {
-                                    // inside the float32 uncertainty band: decide exactly
+                                rare = __builtin_amdgcn_ballot_w64(hi) != m;
+                            }
+                            if (rare) {
+                                bool in = false;
+                                if (hi && (!lo || (HALF && __float_as_int(p.w) == i_atom)) && k != k_self) {
                                     const int j = __float_as_int(p.w);
                                     int s0, s1, s2;
                                     candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
-                                    const float* pi = a.pos + 3 * (size_t)i_atom;
-                                    const float* pj = a.pos + 3 * (size_t)j;
-                                    double e0, e1d, e2d;
-                                    double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1, s2,
-                                                              ws.sys[sidx].h, e0, e1d, e2d);
-                                    in = r2 < a.rc2;
-                                }
-                                if (HALF && in && k != k_self) {
-                                    const int j = __float_as_int(p.w);
-                                    if (j == i_atom) {  // a periodic image of the centre atom: keep the positive shift
-                                        int s0, s1, s2;
-                                        candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
-                                        in = half_keep(i_atom, j, s0, s1, s2);
-                                    } else {
-                                        in = i_atom < j;
+                                    in = lo;
+                                    if (!lo) {  // inside the band: decide exactly
+                                        const float* pi = a.pos + 3 * (size_t)i_atom;
+                                        const float* pj = a.pos + 3 * (size_t)j;
+                                        double e0, e1d, e2d;
+                                        const double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1,
+                                                                        s2, ws.sys[sidx].h, e0, e1d, e2d);
+                                        in = r2 < a.rc2;
                                     }
+                                    if (HALF && in) in = half_keep(i_atom, j, s0, s1, s2);
                                 }
-                                m = __builtin_amdgcn_ballot_w64(in);
+                                const unsigned long long me = __builtin_amdgcn_ballot_w64(in);
                                 if (in) {
-                                    const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
-                                                                                 __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                    const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(me >> 32),
+                                                                                 __builtin_amdgcn_mbcnt_lo((unsigned)me, 0));
                                     my_hits[nh + before] = (unsigned short)k;
                                 }
+                                nh += __popcll(me);
                             }
-                            nh += __popcll(m);
-                            if (nh > kHitCap - kWave) flush();
+                        };
+                        int k0 = k_lo;
+                        for (; k0 + kWave < k_hi; k0 += 2 * kWave) {
+                            const int k = k0 + lane;
+                            const float4 pa = c_pos[k], pb = c_pos[k + kWave];
+                            const float da = dist2(pa), db = dist2(pb);
+                            accept(k, pa, da);
+                            accept(k + kWave, pb, db);
+                            if (nh > kHitCap - 3 * kWave) flush();
+                        }
+                        if (k0 < k_hi) {
+                            const int k = k0 + lane;
+                            const float4 pa = c_pos[k];
+                            accept(k, pa, dist2(pa));
                         }
                         flush();
-                        if (last_tile) {
+                        if (fused) {
                             // ---- count, and padding over what the previous build left beyond it
-                            const int hi_slot = a.tail_mode ? a.K : (old_cnt < a.K ? old_cnt : a.K);
                             for (int k = base + lane; k < hi_slot; k += kWave) {
                                 row[k] = a.n_atoms;
                                 if (srow) {
@@ -662,7 +791,7 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                             }
                             if (lane == 0) a.nn[i_atom] = base;
                         } else if (lane == 0) {
-                            row_cnt[ca] = base;
+                            ca_meta[ca].w = base;
                         }
                     }
                     __syncthreads();
@@ -670,15 +799,14 @@ __global__ __launch_bounds__(kBlock, 6) void nl_search_kernel(NlArgs a, NlWorksp
                 __syncthreads();  // everyone has read this batch's tables before wave 0 rewrites them
             }
 
-            if (n_stencil > kStencilBatch || st_prefix[kStencilBatch] > kTile) {
+            if (!(one_batch && st_prefix[kStencilBatch] <= kTile)) {
                 // several batches or tiles: counts were carried in LDS, finish the rows now
                 for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
                     const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ca_pos[ca].w));
-                    const int cnt = __builtin_amdgcn_readfirstlane(row_cnt[ca]);
-                    const int old_cnt = a.nn[i_atom];
+                    const int cnt = __builtin_amdgcn_readfirstlane(ca_meta[ca].w);
+                    const int hi_slot = __builtin_amdgcn_readfirstlane(ca_w[ca].w) >> 2;
                     int32_t* row = a.nm + (size_t)i_atom * a.K;
                     int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
-                    const int hi_slot = a.tail_mode ? a.K : (old_cnt < a.K ? old_cnt : a.K);
                     for (int k = cnt + lane; k < hi_slot; k += kWave) {
                         row[k] = a.n_atoms;
                         if (srow) {
@@ -744,7 +872,6 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     a.K = max_neighbors;
     a.half = half_fill ? 1 : 0;
     a.tail_mode = tail_mode ? 1 : 0;
-    { static int d = [] { const char* e = getenv("NVAMD_NL_DBG"); return e ? atoi(e) : 0; }(); a.dbg = d; }
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
@@ -759,7 +886,7 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     hipLaunchKernelGGL(nl_prepare_kernel, blocks(n_prep), blk, 0, st, a, ws);
     hipLaunchKernelGGL(nl_bounds_kernel, blocks(n_atoms), blk, 0, st, a, ws);
     hipLaunchKernelGGL(nl_grid_kernel, dim3(1), dim3(1024), 0, st, a, ws);
-    hipLaunchKernelGGL(nl_bin_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+    hipLaunchKernelGGL(nl_bin_kernel, blocks(n_prep > (size_t)n_atoms ? n_prep : (size_t)n_atoms), blk, 0, st, a, ws);
     scan::exclusive(scan::LoadArray{ws.cell_count}, &ws.hdr->total_cells, 0, ws.n_scan_blocks,
                     ws.block_sums, ws.cell_start, st);
     hipLaunchKernelGGL(nl_scatter_kernel, blocks(n_atoms), blk, 0, st, a, ws);
