@@ -657,6 +657,11 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                     // padding up to a multiple of 64: candidates that no centre atom can reach
                     if ((int)threadIdx.x < tile_pad - tile_n)
                         c_pos[tile_n + threadIdx.x] = make_float4(3.0e38f, 0.f, 0.f, __int_as_float(-1));
+                    // Every load above has landed before the centre loop starts (vmcnt(0)): otherwise
+                    // the loop would begin each turn with a wait on "the loads that may still be in
+                    // flight", which, the counter being in-order, waits for the previous centre
+                    // atom's row stores instead.
+                    __builtin_amdgcn_s_waitcnt(0x0F70);
                     __syncthreads();
 
                     const ShiftSource shifts{c_pk, st_prefix, st_start, st_q, ws.sorted_aux, t0};
