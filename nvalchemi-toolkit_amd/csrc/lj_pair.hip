@@ -17,6 +17,9 @@
 #include "common.h"
 #include "geom.h"
 
+#ifndef NVAMD_LJ_UNROLL
+#define NVAMD_LJ_UNROLL 4
+#endif
 namespace nvamd {
 namespace {
 
@@ -65,6 +68,15 @@ __global__ __launch_bounds__(kBlock) void lj_sys_range_kernel(const int32_t* __r
 
 // One pass over the rows [row0, row_end).  LDS_POS: neighbor positions come from the LDS stage
 // (atoms [span0, span0 + span_n)), otherwise from global memory.
+// 1/x for a normal, positive x: hardware estimate and two Newton steps (full double
+// precision without the scaling and fix-up steps of a general division)
+__device__ __forceinline__ double reciprocal(double x) {
+    double y = __builtin_amdgcn_rcp(x);
+    y = __builtin_fma(y, __builtin_fma(-x, y, 1.0), y);
+    y = __builtin_fma(y, __builtin_fma(-x, y, 1.0), y);
+    return y;
+}
+
 template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC>
 __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, int sys_base,
                                         const float* __restrict__ s_pos, int span0, int span_n,
@@ -94,7 +106,8 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
         // UNROLL row entries per lane are in flight at once: first every index and shift of the
         // chunk, then every neighbor position, then the arithmetic (the loop is latency bound
         // otherwise: two dependent trips to memory per entry)
-        constexpr int UNROLL = 4;
+        constexpr int UNROLL = NVAMD_LJ_UNROLL;
+        const int last_quad = cnt > 0 ? ((cnt - 1) & ~3) : 0;  // lanes beyond it re-read it: no extra lines
         for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
             int jj[UNROLL], s0[UNROLL], s1[UNROLL], s2[UNROLL];
             float xj[UNROLL], yj[UNROLL], zj[UNROLL];
@@ -102,17 +115,22 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 // each lane owns four consecutive entries: one 16-byte load of indices and three
                 // of shifts, so a row is read as contiguous 256 + 768 byte runs (K % 4 == 0)
                 const int kb = k0 + UNROLL * sub;
-                const int kq = kb <= a.K - 4 ? kb : a.K - 4;
-                const int4 j4 = *reinterpret_cast<const int4*>(row + kq);
-                jj[0] = j4.x; jj[1] = j4.y; jj[2] = j4.z; jj[3] = j4.w;
-                if (SHIFTS) {
-                    const int4* sp = reinterpret_cast<const int4*>(srow + 3 * kq);
-                    const int4 sa = sp[0], sb = sp[1], sc = sp[2];
-                    s0[0] = sa.x; s1[0] = sa.y; s2[0] = sa.z;
-                    s0[1] = sa.w; s1[1] = sb.x; s2[1] = sb.y;
-                    s0[2] = sb.z; s1[2] = sb.w; s2[2] = sc.x;
-                    s0[3] = sc.y; s1[3] = sc.z; s2[3] = sc.w;
-                } else {
+#pragma unroll
+                for (int v = 0; v < UNROLL / 4; ++v) {
+                    const int kv = kb + 4 * v;
+                    const int kq = kv < last_quad ? kv : last_quad;  // never past the row's last used quad
+                    const int4 j4 = *reinterpret_cast<const int4*>(row + kq);
+                    jj[4 * v + 0] = j4.x; jj[4 * v + 1] = j4.y; jj[4 * v + 2] = j4.z; jj[4 * v + 3] = j4.w;
+                    if (SHIFTS) {
+                        const int4* sp = reinterpret_cast<const int4*>(srow + 3 * kq);
+                        const int4 sa = sp[0], sb = sp[1], sc = sp[2];
+                        s0[4 * v + 0] = sa.x; s1[4 * v + 0] = sa.y; s2[4 * v + 0] = sa.z;
+                        s0[4 * v + 1] = sa.w; s1[4 * v + 1] = sb.x; s2[4 * v + 1] = sb.y;
+                        s0[4 * v + 2] = sb.z; s1[4 * v + 2] = sb.w; s2[4 * v + 2] = sc.x;
+                        s0[4 * v + 3] = sc.y; s1[4 * v + 3] = sc.z; s2[4 * v + 3] = sc.w;
+                    }
+                }
+                if (!SHIFTS) {
 #pragma unroll
                     for (int u = 0; u < UNROLL; ++u) s0[u] = s1[u] = s2[u] = 0;
                 }
@@ -157,7 +175,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 double d0, d1, d2;
                 double r2 = pair_d2_exact(xi, yi, zi, xj[u], yj[u], zj[u], s0[u], s1[u], s2[u], h, d0, d1, d2);
                 if (jj[u] < 0 || !(r2 < a.rc2)) continue;
-                double ir2 = 1.0 / r2;
+                const double ir2 = reciprocal(r2);
                 double q2 = a.sig2 * ir2;
                 double q6 = q2 * q2 * q2;
                 double q12 = q6 * q6;
@@ -236,19 +254,29 @@ __global__ __launch_bounds__(kBlockFull) void lj_matrix_kernel(LjArgs a) {
     const int sys_lo = a.bidx[row0];
     if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
 
-    // neighbors live in the systems of these rows: stage their positions in LDS when they fit
-    // (atom order carries no spatial locality, so gathers through the caches move a whole line
-    // per 12 useful bytes)
-    const int span0 = a.sys_first[sys_lo];
-    const int span_n = a.sys_last[a.bidx[row_end - 1]] - span0;
-    const bool staged = span_n > 0 && span_n <= a.lds_atoms;
-    if (staged) {
-        const float* src = a.pos + 3 * (size_t)span0;
-        for (int t = threadIdx.x; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
+    // Neighbors live in the system of their row: the rows are taken one system at a time, with
+    // that system's positions staged in LDS when they fit (atom order carries no spatial
+    // locality, so gathers through the caches move a whole line per 12 useful bytes).
+    for (int r = row0; r < row_end;) {
+        const int sys = a.bidx[r];
+        const int span0 = a.sys_first[sys];
+        const int span_end = a.sys_last[sys];
+        const int span_n = span_end - span0;
+        // rows of this system inside the block; a batch index that is not sorted (a system in
+        // several pieces) makes the range meaningless: then the rest of the block goes unstaged
+        const bool range_ok = span0 <= r && r < span_end;
+        const int seg_end = (range_ok && span_end < row_end) ? span_end : row_end;
+        const bool staged = range_ok && span_n <= a.lds_atoms;
+        if (staged) {
+            const float* src = a.pos + 3 * (size_t)span0;
+            for (int t = threadIdx.x; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
+        }
+        __syncthreads();
+        if (staged) lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_acc);
+        else lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_acc);
+        r = seg_end;
+        if (r < row_end) __syncthreads();  // the stage is about to be overwritten
     }
-    __syncthreads();
-    if (staged) lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC>(a, row0, row_end, sys_lo, s_pos, span0, span_n, s_acc);
-    else lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC>(a, row0, row_end, sys_lo, s_pos, 0, 0, s_acc);
 
     if (SYS) {
         __syncthreads();
