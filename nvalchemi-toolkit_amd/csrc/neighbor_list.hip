@@ -39,6 +39,7 @@ constexpr int kHitCap = 320;      // per-wave list of accepted candidates before
 constexpr int kPackOverflow = 1 << 30;
 static_assert(kMaxRun <= 4, "a centre atom's place in its run is kept in two bits");
 constexpr int kMaxCellsPerAxis = 1024;
+static_assert(kMaxCellsPerAxis <= 1024, "a search unit's cell coordinates are packed 10 bits each");
 constexpr int kMinCellCap = 8;    // a system may use at least this many cells
 constexpr int kMaxStencilRadius = 32;  // cells searched per axis and direction, at most
 
@@ -57,6 +58,7 @@ struct NlSys {
     int n_cells;
     int zr;            // cells per run along axis 2 (the search's unit of work)
     int n_units;       // runs in this system
+    int error;         // bit 0: cell degenerate or narrower than cutoff/kMaxStencilRadius
     int atom_begin, atom_end;
 };
 
@@ -85,7 +87,8 @@ struct NlWorkspace {
     NlSearchSys* ssys;   // (B)
     int* cell_offset;    // (B+1)
     int* unit_offset;    // (B+1) first unit of each system
-    int2* units;         // (C) per unit of search work: first cell of the run, system
+    int4* units;         // (C) per unit of search work: first cell of the run, system, that cell's
+                         //     coordinates packed 10 bits each, cells in the run
     int* atom_rank;      // (N)
     int* cell_count;     // (C)
     int* cell_start;     // (C+1)
@@ -97,7 +100,8 @@ struct NlWorkspace {
 };
 
 size_t max_cells_for(int n_atoms, int n_systems) {
-    return (size_t)n_atoms + (size_t)kMinCellCap * (size_t)n_systems + 1;
+    // (one more per system: the per-system path gives every system its own end-of-cells entry)
+    return (size_t)n_atoms + (size_t)(kMinCellCap + 1) * (size_t)n_systems + 1;
 }
 
 size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
@@ -117,7 +121,7 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
     p = take(B * sizeof(NlSearchSys)); if (ws) ws->ssys = reinterpret_cast<NlSearchSys*>(p);
     p = take((B + 1) * sizeof(int)); if (ws) ws->cell_offset = reinterpret_cast<int*>(p);
     p = take((B + 1) * sizeof(int)); if (ws) ws->unit_offset = reinterpret_cast<int*>(p);
-    p = take(C * sizeof(int2)); if (ws) ws->units = reinterpret_cast<int2*>(p);
+    p = take(C * sizeof(int4)); if (ws) ws->units = reinterpret_cast<int4*>(p);
     p = take(N * sizeof(int)); if (ws) ws->atom_rank = reinterpret_cast<int*>(p);
     p = take(C * sizeof(int)); if (ws) ws->cell_count = reinterpret_cast<int*>(p);
     p = take((C + 1) * sizeof(int)); if (ws) ws->cell_start = reinterpret_cast<int*>(p);
@@ -170,12 +174,8 @@ __device__ __forceinline__ void frac_of(const NlSys& s, const float* __restrict_
 }
 
 // ---- 1 prepare ------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspace ws) {
-    int t = blockIdx.x * kBlock + threadIdx.x;
-    if (t < ws.max_cells) ws.cell_count[t] = 0;
-    if (t == 0) ws.hdr->error = 0;
-    if (t >= a.n_systems) return;
-    NlSys s;
+// Per-system constants that do not depend on the atoms: cell, inverse, widths, periodic flags.
+__device__ __forceinline__ void system_setup(NlSys& s, const NlArgs& a, int t) {
     const bool has_cell = a.cell != nullptr;
 #pragma unroll
     for (int k = 0; k < 9; ++k) s.h[k] = has_cell ? (double)a.cell[9 * (size_t)t + k] : ((k % 4 == 0) ? 1.0 : 0.0);
@@ -189,16 +189,31 @@ __global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspac
         s.ext[d] = 1.0;
         s.nc[d] = 1;
         s.R[d] = 0;
-        ws.bounds[6 * (size_t)t + d] = 0xffffffffu;      // min key
-        ws.bounds[6 * (size_t)t + 3 + d] = 0u;           // max key
     }
 #pragma unroll
     for (int k = 0; k < 9; ++k) s.step[k] = s.h[k];
     s.tol = 0.f;
     s.cell_offset = 0;
     s.n_cells = 1;
+    s.zr = 1;
+    s.n_units = 0;
+    s.error = 0;
     s.atom_begin = a.ptr[t];
     s.atom_end = a.ptr[t + 1];
+}
+
+__global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspace ws) {
+    int t = blockIdx.x * kBlock + threadIdx.x;
+    if (t < ws.max_cells) ws.cell_count[t] = 0;
+    if (t == 0) ws.hdr->error = 0;
+    if (t >= a.n_systems) return;
+    NlSys s;
+    system_setup(s, a, t);
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        ws.bounds[6 * (size_t)t + d] = 0xffffffffu;      // min key
+        ws.bounds[6 * (size_t)t + 3 + d] = 0u;           // max key
+    }
     ws.sys[t] = s;
 }
 
@@ -220,6 +235,95 @@ __global__ __launch_bounds__(kBlock) void nl_bounds_kernel(NlArgs a, NlWorkspace
     }
 }
 
+// Cells per axis (width >= cutoff), stencil radius, run length, cell steps and the float32
+// tolerance of one system; bounds6 holds the order keys of the fractional bounding box
+// (min x,y,z then max x,y,z), read on non-periodic axes only.
+__device__ __forceinline__ void choose_grid(NlSys& s, const NlArgs& a, const uint32_t* bounds6, int* error_flag) {
+    const int n_at = s.atom_end - s.atom_begin;
+    for (int d = 0; d < 3; ++d) {
+        if (!s.per[d]) {
+            uint32_t kmin = bounds6[d], kmax = bounds6[3 + d];
+            if (kmin <= kmax && n_at > 0) {
+                double lo = (double)float_from_order_key(kmin), hi = (double)float_from_order_key(kmax);
+                s.lo[d] = lo;
+                s.ext[d] = hi - lo;
+            }
+            if (!(s.ext[d] > 1e-30)) s.ext[d] = 1e-30;
+        }
+        double span = s.ext[d] * s.width[d];
+        double q = floor(span / a.rcb);
+        int c = (q >= 1.0) ? (q > (double)kMaxCellsPerAxis ? kMaxCellsPerAxis : (int)q) : 1;
+        s.nc[d] = c;
+    }
+    int cap = n_at > kMinCellCap ? n_at : kMinCellCap;
+    while ((long long)s.nc[0] * s.nc[1] * s.nc[2] > (long long)cap) {
+        int m = 0;
+        if (s.nc[1] > s.nc[m]) m = 1;
+        if (s.nc[2] > s.nc[m]) m = 2;
+        if (s.nc[m] == 1) break;
+        s.nc[m] = (s.nc[m] + 1) / 2;
+    }
+    double len[3];
+    for (int d = 0; d < 3; ++d) {
+        double cw = s.ext[d] * s.width[d] / s.nc[d];
+        int R;
+        if (!s.per[d] && s.nc[d] == 1) R = 0;
+        else {
+            double r = ceil(a.rcb / cw);
+            if (r >= 1.0 && r <= (double)kMaxStencilRadius) R = (int)r;
+            else {
+                R = (r > (double)kMaxStencilRadius) ? kMaxStencilRadius : 1;
+                if (n_at > 0) atomicOr(error_flag, 1);
+            }
+            if (!s.per[d] && R > s.nc[d] - 1) R = s.nc[d] - 1;
+        }
+        s.R[d] = R;
+        double sc = s.ext[d] / s.nc[d];
+        double l2 = 0.0;
+        for (int k = 0; k < 3; ++k) {
+            s.step[3 * d + k] = sc * s.h[3 * d + k];
+            l2 += s.step[3 * d + k] * s.step[3 * d + k];
+        }
+        len[d] = sqrt(l2);
+    }
+    s.n_cells = n_at > 0 ? s.nc[0] * s.nc[1] * s.nc[2] : 0;
+    // Run length along axis 2: as long as the run's whole stencil is expected to fit one
+    // batch of stencil cells and one LDS tile, and its centre atoms one pass.
+    int zr = 1;
+    if (s.n_cells > 0) {
+        const double per_cell = 1.2 * (double)n_at / (double)s.n_cells;
+        const int e01 = (2 * s.R[0] + 1) * (2 * s.R[1] + 1);
+        for (int cand = 2; cand <= kMaxRun && cand <= s.nc[2]; ++cand) {
+            const int entries = (cand + 2 * s.R[2]) * e01;
+            if (entries > kStencilBatch) break;
+            if (entries * per_cell + kWave > (double)kTile) break;
+            if (cand * per_cell > (double)kCenterChunk) break;
+            zr = cand;
+        }
+        const int runs = (s.nc[2] + zr - 1) / zr;
+        zr = (s.nc[2] + runs - 1) / runs;  // same number of runs, evened out
+    }
+    s.zr = zr;
+    s.n_units = s.n_cells > 0 ? s.nc[0] * s.nc[1] * ((s.nc[2] + zr - 1) / zr) : 0;
+    // largest cell-local coordinate the search can meet
+    const double reach = (s.R[0] + 1) * len[0] + (s.R[1] + 1) * len[1] + (s.R[2] + zr) * len[2];
+    s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
+}
+
+__device__ __forceinline__ NlSearchSys search_view(const NlSys& s) {
+    NlSearchSys q;
+    for (int k = 0; k < 9; ++k) q.step[k] = (float)s.step[k];
+    q.tol = s.tol;
+    for (int d = 0; d < 3; ++d) {
+        q.nc[d] = s.nc[d];
+        q.R[d] = s.R[d];
+        q.per[d] = s.per[d];
+    }
+    q.cell_offset = s.cell_offset;
+    q.zr = s.zr;
+    return q;
+}
+
 // ---- 3 grid ---------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws) {
     // low word: cells, high word: search units (both totals stay below 2^31, so the packed
@@ -233,75 +337,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
         int ncell = 0, nunit = 0;
         if (t < a.n_systems) {
             NlSys s = ws.sys[t];
-            int n_at = s.atom_end - s.atom_begin;
-            for (int d = 0; d < 3; ++d) {
-                if (!s.per[d]) {
-                    uint32_t kmin = ws.bounds[6 * (size_t)t + d], kmax = ws.bounds[6 * (size_t)t + 3 + d];
-                    if (kmin <= kmax && n_at > 0) {
-                        double lo = (double)float_from_order_key(kmin), hi = (double)float_from_order_key(kmax);
-                        s.lo[d] = lo;
-                        s.ext[d] = hi - lo;
-                    }
-                    if (!(s.ext[d] > 1e-30)) s.ext[d] = 1e-30;
-                }
-                double span = s.ext[d] * s.width[d];
-                double q = floor(span / a.rcb);
-                int c = (q >= 1.0) ? (q > (double)kMaxCellsPerAxis ? kMaxCellsPerAxis : (int)q) : 1;
-                s.nc[d] = c;
-            }
-            int cap = n_at > kMinCellCap ? n_at : kMinCellCap;
-            while ((long long)s.nc[0] * s.nc[1] * s.nc[2] > (long long)cap) {
-                int m = 0;
-                if (s.nc[1] > s.nc[m]) m = 1;
-                if (s.nc[2] > s.nc[m]) m = 2;
-                if (s.nc[m] == 1) break;
-                s.nc[m] = (s.nc[m] + 1) / 2;
-            }
-            double len[3];
-            for (int d = 0; d < 3; ++d) {
-                double cw = s.ext[d] * s.width[d] / s.nc[d];
-                int R;
-                if (!s.per[d] && s.nc[d] == 1) R = 0;
-                else {
-                    double r = ceil(a.rcb / cw);
-                    if (r >= 1.0 && r <= (double)kMaxStencilRadius) R = (int)r;
-                    else {
-                        R = (r > (double)kMaxStencilRadius) ? kMaxStencilRadius : 1;
-                        if (n_at > 0) atomicOr(&ws.hdr->error, 1);
-                    }
-                    if (!s.per[d] && R > s.nc[d] - 1) R = s.nc[d] - 1;
-                }
-                s.R[d] = R;
-                double sc = s.ext[d] / s.nc[d];
-                double l2 = 0.0;
-                for (int k = 0; k < 3; ++k) {
-                    s.step[3 * d + k] = sc * s.h[3 * d + k];
-                    l2 += s.step[3 * d + k] * s.step[3 * d + k];
-                }
-                len[d] = sqrt(l2);
-            }
-            s.n_cells = n_at > 0 ? s.nc[0] * s.nc[1] * s.nc[2] : 0;
-            // Run length along axis 2: as long as the run's whole stencil is expected to fit one
-            // batch of stencil cells and one LDS tile, and its centre atoms one pass.
-            int zr = 1;
-            if (s.n_cells > 0) {
-                const double per_cell = 1.2 * (double)n_at / (double)s.n_cells;
-                const int e01 = (2 * s.R[0] + 1) * (2 * s.R[1] + 1);
-                for (int cand = 2; cand <= kMaxRun && cand <= s.nc[2]; ++cand) {
-                    const int entries = (cand + 2 * s.R[2]) * e01;
-                    if (entries > kStencilBatch) break;
-                    if (entries * per_cell + kWave > (double)kTile) break;
-                    if (cand * per_cell > (double)kCenterChunk) break;
-                    zr = cand;
-                }
-                const int runs = (s.nc[2] + zr - 1) / zr;
-                zr = (s.nc[2] + runs - 1) / runs;  // same number of runs, evened out
-            }
-            s.zr = zr;
-            s.n_units = s.n_cells > 0 ? s.nc[0] * s.nc[1] * ((s.nc[2] + zr - 1) / zr) : 0;
-            // largest cell-local coordinate the search can meet
-            const double reach = (s.R[0] + 1) * len[0] + (s.R[1] + 1) * len[1] + (s.R[2] + zr) * len[2];
-            s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
+            choose_grid(s, a, ws.bounds + 6 * (size_t)t, &ws.hdr->error);
             ncell = s.n_cells;
             nunit = s.n_units;
             ws.sys[t] = s;
@@ -324,18 +360,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
             ws.sys[t].cell_offset = off;
             ws.cell_offset[t] = off;
             ws.unit_offset[t] = (int)(unsigned)(excl >> 32);
-            const NlSys& s = ws.sys[t];
-            NlSearchSys q;
-            for (int k = 0; k < 9; ++k) q.step[k] = (float)s.step[k];
-            q.tol = s.tol;
-            for (int d = 0; d < 3; ++d) {
-                q.nc[d] = s.nc[d];
-                q.R[d] = s.R[d];
-                q.per[d] = s.per[d];
-            }
-            q.cell_offset = off;
-            q.zr = s.zr;
-            ws.ssys[t] = q;
+            ws.ssys[t] = search_view(ws.sys[t]);
         }
         __syncthreads();
         if (threadIdx.x == 1023) s_carry = carry + incl;
@@ -386,6 +411,14 @@ __device__ __forceinline__ Binned bin_atom(const NlSys& s, const float* __restri
     return b;
 }
 
+// Unit lu of a system: the run-th run of cells along axis 2 in column (cx, cy).
+__device__ __forceinline__ int4 make_unit(const NlSearchSys& q, int lu, int runs, int sys) {
+    const int column = lu / runs, run = lu - column * runs;
+    const int cx = column / q.nc[1], cy = column - cx * q.nc[1], cz0 = run * q.zr;
+    const int len = (q.nc[2] - cz0) < q.zr ? (q.nc[2] - cz0) : q.zr;
+    return make_int4(q.cell_offset + column * q.nc[2] + cz0, sys, (cx << 20) | (cy << 10) | cz0, len);
+}
+
 // Launched over max(atoms, cell bound) threads: thread t bins atom t and describes search unit t.
 __global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws) {
     int i = blockIdx.x * kBlock + threadIdx.x;
@@ -399,8 +432,7 @@ __global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws
         const NlSearchSys& q = ws.ssys[lo];
         const int lu = i - ws.unit_offset[lo];
         const int runs = (q.nc[2] + q.zr - 1) / q.zr;
-        const int column = lu / runs, run = lu - column * runs;
-        ws.units[i] = make_int2(q.cell_offset + column * q.nc[2] + run * q.zr, lo);
+        ws.units[i] = make_unit(q, lu, runs, lo);
     }
     if (i >= a.n_atoms) return;
     const NlSys& s = ws.sys[a.bidx[i]];
@@ -416,6 +448,195 @@ __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspac
     int slot = ws.cell_start[b.cell] + ws.atom_rank[i];
     ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
     ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
+}
+
+// ---- per-system path: 1-6 in one workgroup per system -----------------------------------------
+// For batches of many small systems.  One workgroup takes one system through set-up, bounds,
+// grid choice, histogram (in LDS), scan and scatter; no global histogram, no global scan.
+// Every system owns the cell ids [atom_begin + 9 s, ... + n_cells] (cells <= max(atoms, 8), plus
+// one end entry), so cell ids need no prefix sum over the systems either.  A system with more
+// cells than the LDS histogram holds is still handled, slowly, through global memory.
+constexpr int kSortBlock = 1024;
+constexpr int kSortCells = 8192;         // cells of a system whose histogram fits in LDS
+constexpr int kPerSystemMeanAtoms = 8192;  // the path is taken up to this many atoms per system on average
+
+__device__ __forceinline__ int block_exclusive_scan(int v, int* s_part, int* total) {
+    // kSortBlock threads; s_part holds one partial per wave
+    const int lane = lane_id(), wave = (int)threadIdx.x / kWave;
+    int incl = v;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        int up = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += up;
+    }
+    __syncthreads();  // s_part may still be read from a previous call
+    if (lane == kWave - 1) s_part[wave] = incl;
+    __syncthreads();
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kSortBlock / kWave; ++w) {
+        const int p = s_part[w];
+        before += (w < wave) ? p : 0;
+        all += p;
+    }
+    *total = all;
+    return before + incl - v;
+}
+
+__global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, NlWorkspace ws) {
+    __shared__ NlSys s_sys;
+    __shared__ uint32_t s_bounds[6];
+    __shared__ int s_err;
+    __shared__ int s_unit0;
+    __shared__ int s_hist[kSortCells];
+    __shared__ int s_part[kSortBlock / kWave];
+    const int t = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int begin = a.ptr[t], end = a.ptr[t + 1];
+    // up to kKeep atoms per thread stay in registers from here to the scatter; their positions
+    // are requested now, so that they arrive while thread 0 works out the system's grid
+    constexpr int kKeep = 4;
+    const bool kept = (end - begin) <= kKeep * kSortBlock;
+    float my_pos[kKeep][3];
+    if (kept) {
+#pragma unroll
+        for (int k = 0; k < kKeep; ++k) {
+            const int i = begin + tid + k * kSortBlock;
+            const float* r = a.pos + 3 * (size_t)(i < end ? i : (end > begin ? begin : 0));
+            my_pos[k][0] = r[0];
+            my_pos[k][1] = r[1];
+            my_pos[k][2] = r[2];
+        }
+    }
+    if (tid < 6) s_bounds[tid] = tid < 3 ? 0xffffffffu : 0u;
+    if (tid == 0) {
+        s_err = 0;
+        system_setup(s_sys, a, t);  // (worked on in place, in LDS)
+    }
+    __syncthreads();
+    const int cell_base = begin + (kMinCellCap + 1) * t;
+    const bool idle = end <= begin || (a.rebuild && !a.rebuild[t]);  // nothing to search: no cells, no units
+    // ---- bounds on non-periodic axes
+    if (!idle && !(s_sys.per[0] && s_sys.per[1] && s_sys.per[2])) {
+        for (int i = begin + tid; i < end; i += kSortBlock) {
+            double f[3];
+            frac_of(s_sys, a.pos + 3 * (size_t)i, f);
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                if (s_sys.per[d]) continue;
+                float lo = __double2float_rd(f[d]), hi = __double2float_ru(f[d]);
+                atomicMin(&s_bounds[d], float_order_key(lo));
+                atomicMax(&s_bounds[3 + d], float_order_key(hi));
+            }
+        }
+        __syncthreads();
+    }
+    // ---- grid
+    if (tid == 0) {
+        if (idle) {
+            s_sys.n_cells = 0;
+            s_sys.n_units = 0;
+        } else {
+            choose_grid(s_sys, a, s_bounds, &s_err);
+        }
+        s_sys.error = s_err;
+        s_sys.cell_offset = cell_base;
+        ws.cell_offset[t] = cell_base;
+        // this system's units: a contiguous piece of the unit list, wherever the counter stands
+        // (the order of systems in the list is of no consequence)
+        s_unit0 = s_sys.n_units > 0 ? atomicAdd(&ws.hdr->total_units, s_sys.n_units) : 0;
+        if (s_err) atomicOr(&ws.hdr->error, s_err);
+    }
+    __syncthreads();
+    {
+        // the system's record leaves LDS word by word
+        const int* src = reinterpret_cast<const int*>(&s_sys);
+        int* dst = reinterpret_cast<int*>(ws.sys + t);
+        for (int w = tid; w < (int)(sizeof(NlSys) / sizeof(int)); w += kSortBlock) dst[w] = src[w];
+        const NlSearchSys q = search_view(s_sys);
+        if (tid == 0) ws.ssys[t] = q;
+        const int n_units = s_sys.n_units, unit0 = s_unit0;
+        const int runs = (q.nc[2] + q.zr - 1) / q.zr;
+        for (int lu = tid; lu < n_units; lu += kSortBlock) ws.units[unit0 + lu] = make_unit(q, lu, runs, t);
+    }
+    if (idle) return;
+    const int n_cells = s_sys.n_cells;
+    const bool in_lds = n_cells <= kSortCells;
+    int* g_hist = ws.cell_count + cell_base;
+    int* g_start = ws.cell_start + cell_base;
+    // ---- histogram: rank of every atom inside its cell
+    for (int c = tid; c < n_cells; c += kSortBlock) {
+        if (in_lds) s_hist[c] = 0;
+        else g_hist[c] = 0;
+    }
+    __syncthreads();
+    Binned mine[kKeep];
+    int my_rank[kKeep];
+    if (kept) {
+#pragma unroll
+        for (int k = 0; k < kKeep; ++k) {
+            const int i = begin + tid + k * kSortBlock;
+            if (i < end) {
+                mine[k] = bin_atom(s_sys, my_pos[k]);
+                const int lc = mine[k].cell - cell_base;
+                my_rank[k] = in_lds ? atomicAdd(&s_hist[lc], 1) : atomicAdd(&g_hist[lc], 1);
+            }
+        }
+    } else {
+        for (int i = begin + tid; i < end; i += kSortBlock) {
+            const Binned b = bin_atom(s_sys, a.pos + 3 * (size_t)i);
+            const int lc = b.cell - cell_base;
+            ws.atom_rank[i] = in_lds ? atomicAdd(&s_hist[lc], 1) : atomicAdd(&g_hist[lc], 1);
+        }
+    }
+    __syncthreads();
+    // ---- scan: thread t owns a contiguous chunk of cells
+    {
+        const int chunk = (n_cells + kSortBlock - 1) / kSortBlock;
+        const int c_lo = tid * chunk < n_cells ? tid * chunk : n_cells;
+        const int c_hi = (c_lo + chunk) < n_cells ? (c_lo + chunk) : n_cells;
+        int sum = 0;
+        for (int c = c_lo; c < c_hi; ++c)
+            sum += in_lds ? s_hist[c] : __hip_atomic_load(&g_hist[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int total;
+        int running = begin + block_exclusive_scan(sum, s_part, &total);
+        for (int c = c_lo; c < c_hi; ++c) {
+            const int n = in_lds ? s_hist[c] : __hip_atomic_load(&g_hist[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (in_lds) {
+                s_hist[c] = running;
+                g_start[c] = running;
+            } else {
+                __hip_atomic_store(&g_start[c], running, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            running += n;
+        }
+        if (tid == 0) g_start[n_cells] = end;
+    }
+    __syncthreads();
+    // ---- scatter into cell order
+    auto place = [&](const Binned& b, int i, int rank) {
+        const int lc = b.cell - cell_base;
+        const int start = in_lds ? s_hist[lc] : __hip_atomic_load(&g_start[lc], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int slot = start + rank;
+        ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
+        ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
+    };
+    if (kept) {
+#pragma unroll
+        for (int k = 0; k < kKeep; ++k) {
+            const int i = begin + tid + k * kSortBlock;
+            if (i < end) place(mine[k], i, my_rank[k]);
+        }
+    } else {
+        for (int i = begin + tid; i < end; i += kSortBlock) place(bin_atom(s_sys, a.pos + 3 * (size_t)i), i, ws.atom_rank[i]);
+    }
+}
+
+// Before nl_system_sort_kernel: the unit counter and the error flag start at zero.
+__global__ void nl_reset_kernel(NlWorkspace ws) {
+    ws.hdr->total_units = 0;
+    ws.hdr->total_cells = 0;  // not used on the per-system path: cell ids are not dense
+    ws.hdr->error = 0;
 }
 
 // ---- 7 search -------------------------------------------------------------------------------
@@ -506,15 +727,15 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         // NOTE: every thread of the workgroup takes the same path through this loop body
         const int u = xcd * per_xcd + li;
         if (u >= total_units) break;
-        const int2 unit = ws.units[u];
+        const int4 unit = ws.units[u];
         const int c0 = __builtin_amdgcn_readfirstlane(unit.x);
         const int sidx = __builtin_amdgcn_readfirstlane(unit.y);
+        const int cxyz = __builtin_amdgcn_readfirstlane(unit.z);
+        const int run_len = __builtin_amdgcn_readfirstlane(unit.w);
         if (a.rebuild && !a.rebuild[sidx]) continue;
         const NlSearchSys S = ws.ssys[sidx];
-        const int lc = c0 - S.cell_offset;
         const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
-        const int cz0 = lc % nc2, cy = (lc / nc2) % nc1, cx = lc / (nc2 * nc1);
-        const int run_len = (nc2 - cz0) < S.zr ? (nc2 - cz0) : S.zr;
+        const int cz0 = cxyz & 1023, cy = (cxyz >> 10) & 1023, cx = cxyz >> 20;
         const int c_begin = ws.cell_start[c0];
         // first centre atom (relative to c_begin) of the run's cells 1, 2, 3 and the run's end
         int run_off[kMaxRun + 1];
@@ -887,14 +1108,22 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     dim3 blk(kBlock);
     auto blocks = [](size_t n) { return dim3((unsigned)((n + kBlock - 1) / kBlock)); };
-    size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
-    hipLaunchKernelGGL(nl_prepare_kernel, blocks(n_prep), blk, 0, st, a, ws);
-    hipLaunchKernelGGL(nl_bounds_kernel, blocks(n_atoms), blk, 0, st, a, ws);
-    hipLaunchKernelGGL(nl_grid_kernel, dim3(1), dim3(1024), 0, st, a, ws);
-    hipLaunchKernelGGL(nl_bin_kernel, blocks(n_prep > (size_t)n_atoms ? n_prep : (size_t)n_atoms), blk, 0, st, a, ws);
-    scan::exclusive(scan::LoadArray{ws.cell_count}, &ws.hdr->total_cells, 0, ws.n_scan_blocks,
-                    ws.block_sums, ws.cell_start, st);
-    hipLaunchKernelGGL(nl_scatter_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+    // (looked up on every call so that one process can exercise both paths)
+    const bool forbid_per_system = getenv("NVAMD_NL_NO_PER_SYSTEM") != nullptr;
+    if (!forbid_per_system && n_atoms / n_systems <= kPerSystemMeanAtoms) {
+        // many small systems: set-up to scatter in one workgroup per system
+        hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws);
+        hipLaunchKernelGGL(nl_system_sort_kernel, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
+    } else {
+        size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
+        hipLaunchKernelGGL(nl_prepare_kernel, blocks(n_prep), blk, 0, st, a, ws);
+        hipLaunchKernelGGL(nl_bounds_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+        hipLaunchKernelGGL(nl_grid_kernel, dim3(1), dim3(1024), 0, st, a, ws);
+        hipLaunchKernelGGL(nl_bin_kernel, blocks(n_prep > (size_t)n_atoms ? n_prep : (size_t)n_atoms), blk, 0, st, a, ws);
+        scan::exclusive(scan::LoadArray{ws.cell_count}, &ws.hdr->total_cells, 0, ws.n_scan_blocks,
+                        ws.block_sums, ws.cell_start, st);
+        hipLaunchKernelGGL(nl_scatter_kernel, blocks(n_atoms), blk, 0, st, a, ws);
+    }
     // one workgroup per cell; the grid is a fixed size (the cell count lives on the device)
     // and strides over the cells
     unsigned n_search = 8u * 2048u;

@@ -17,6 +17,18 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True, params=["per_system", "global_sort"])
+def sort_path(request, monkeypatch):
+    """Every test runs twice: with the workgroup-per-system sort that batches of small systems
+    take by default, and with the global histogram/scan/scatter pipeline that large systems take
+    (forced here through the library's environment switch, which is read on every call)."""
+    if request.param == "global_sort":
+        monkeypatch.setenv("NVAMD_NL_NO_PER_SYSTEM", "1")
+    else:
+        monkeypatch.delenv("NVAMD_NL_NO_PER_SYSTEM", raising=False)
+    return request.param
+
+
 def gpu_build(P, C, pb, ptr, rc, K, half=False, tail_mode=1, flags=None, prev=None):
     from nvalchemi_amd import _lib
 
@@ -178,3 +190,30 @@ def test_repeated_builds_are_identical_as_sets():
     ea = oracle.matrix_to_edges(*(t.cpu().numpy() for t in a))
     eb = oracle.matrix_to_edges(*(t.cpu().numpy() for t in b))
     assert np.array_equal(ea, eb)
+
+
+def test_per_system_path_with_a_system_too_large_for_its_lds_histogram(sort_path):
+    """A batch whose mean system size selects the workgroup-per-system sort, with one system whose
+    cell count exceeds the LDS histogram (8192 cells): that system goes through global memory."""
+    rng = np.random.default_rng(11)
+    counts = [5, 20000, 0, 7, 300]
+    L_big = 60.0  # cutoff 2.0: 29^3 cells, halved once along x to fit the cap of 20000: 12615 > 8192
+    P, C, pb = [], [], []
+    for n in counts:
+        L = L_big if n > 1000 else 6.0
+        P.append(rng.uniform(0, L, size=(n, 3)))
+        C.append(np.eye(3) * L)
+        pb.append([True, True, True])
+    P = np.concatenate(P).astype(np.float32)
+    C = np.stack(C).astype(np.float32)
+    pb = np.array(pb, dtype=bool)
+    ptr = ptr_from_counts(counts)
+    rc = 2.0
+    K = 96  # the 300 atoms in the 6^3 box are the dense ones (about 46 neighbors on average)
+    nm_r, nn_r, sh_r = oracle.nl_cell(P, C, pb, ptr, rc, K)
+    assert nn_r.max() < K
+    ref = oracle.matrix_to_edges(nm_r, nn_r, sh_r)
+    nm, nn, sh = gpu_build(P, C, pb, ptr, rc, K)
+    assert np.array_equal(nn.cpu().numpy(), nn_r)
+    got = oracle.matrix_to_edges(nm.cpu().numpy(), nn.cpu().numpy(), sh.cpu().numpy())
+    assert np.array_equal(got, ref)
