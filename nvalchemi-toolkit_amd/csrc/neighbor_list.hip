@@ -73,6 +73,22 @@ struct NlSearchSys {
     int zr;
 };
 
+// One unit of search work: a run of cells along axis 2, with what the enumeration of its
+// stencil needs from its system, so that the search kernel reaches the cell table with one
+// round trip to memory less.
+struct __attribute__((aligned(32))) NlUnit {
+    int c0;           // first cell of the run (global id)
+    int sidx;         // system
+    int cxyz;         // that cell's coordinates, 10 bits each: cx << 20 | cy << 10 | cz
+    int run_len;      // cells in the run
+    int nc_pack;      // cells per axis minus one, 10 bits each: (nc0-1) | (nc1-1) << 10 | (nc2-1) << 20
+    int rper_pack;    // stencil radii, 6 bits each, then the periodic flags: R0 | R1 << 6 | R2 << 12 | per << 18
+    int cell_offset;  // first cell of the system
+    int pad;
+};
+static_assert(sizeof(NlUnit) == 32, "read as two 16-byte words");
+static_assert(kMaxStencilRadius < 64, "stencil radii are packed 6 bits each");
+
 struct NlHeader {
     int total_cells;
     int error;  // bit 0: a system's cell is degenerate or narrower than cutoff/kMaxStencilRadius
@@ -87,8 +103,7 @@ struct NlWorkspace {
     NlSearchSys* ssys;   // (B)
     int* cell_offset;    // (B+1)
     int* unit_offset;    // (B+1) first unit of each system
-    int4* units;         // (C) per unit of search work: first cell of the run, system, that cell's
-                         //     coordinates packed 10 bits each, cells in the run
+    NlUnit* units;       // (C) the search's units of work
     int* atom_rank;      // (N)
     int* cell_count;     // (C)
     int* cell_start;     // (C+1)
@@ -121,7 +136,7 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
     p = take(B * sizeof(NlSearchSys)); if (ws) ws->ssys = reinterpret_cast<NlSearchSys*>(p);
     p = take((B + 1) * sizeof(int)); if (ws) ws->cell_offset = reinterpret_cast<int*>(p);
     p = take((B + 1) * sizeof(int)); if (ws) ws->unit_offset = reinterpret_cast<int*>(p);
-    p = take(C * sizeof(int4)); if (ws) ws->units = reinterpret_cast<int4*>(p);
+    p = take(C * sizeof(NlUnit)); if (ws) ws->units = reinterpret_cast<NlUnit*>(p);
     p = take(N * sizeof(int)); if (ws) ws->atom_rank = reinterpret_cast<int*>(p);
     p = take(C * sizeof(int)); if (ws) ws->cell_count = reinterpret_cast<int*>(p);
     p = take((C + 1) * sizeof(int)); if (ws) ws->cell_start = reinterpret_cast<int*>(p);
@@ -143,6 +158,7 @@ struct NlArgs {
     const int32_t* bidx;
     const uint8_t* rebuild;
     int n_atoms, n_systems, K, half, tail_mode;
+    int unit_group;  // units are dealt to the XCDs in groups of this many (a power of two)
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -412,11 +428,20 @@ __device__ __forceinline__ Binned bin_atom(const NlSys& s, const float* __restri
 }
 
 // Unit lu of a system: the run-th run of cells along axis 2 in column (cx, cy).
-__device__ __forceinline__ int4 make_unit(const NlSearchSys& q, int lu, int runs, int sys) {
+__device__ __forceinline__ NlUnit make_unit(const NlSearchSys& q, int lu, int runs, int sys) {
     const int column = lu / runs, run = lu - column * runs;
     const int cx = column / q.nc[1], cy = column - cx * q.nc[1], cz0 = run * q.zr;
-    const int len = (q.nc[2] - cz0) < q.zr ? (q.nc[2] - cz0) : q.zr;
-    return make_int4(q.cell_offset + column * q.nc[2] + cz0, sys, (cx << 20) | (cy << 10) | cz0, len);
+    NlUnit u;
+    u.c0 = q.cell_offset + column * q.nc[2] + cz0;
+    u.sidx = sys;
+    u.cxyz = (cx << 20) | (cy << 10) | cz0;
+    u.run_len = (q.nc[2] - cz0) < q.zr ? (q.nc[2] - cz0) : q.zr;
+    u.nc_pack = (q.nc[0] - 1) | ((q.nc[1] - 1) << 10) | ((q.nc[2] - 1) << 20);
+    u.rper_pack = q.R[0] | (q.R[1] << 6) | (q.R[2] << 12) | ((q.per[0] ? 1 : 0) << 18) | ((q.per[1] ? 1 : 0) << 19) |
+                  ((q.per[2] ? 1 : 0) << 20);
+    u.cell_offset = q.cell_offset;
+    u.pad = 0;
+    return u;
 }
 
 // Launched over max(atoms, cell bound) threads: thread t bins atom t and describes search unit t.
@@ -705,7 +730,8 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     __shared__ float4 c_pos[kTile];           // candidate: xyz relative to the run's first cell + atom index
     __shared__ int c_pk[kTile];               // packed (image of its cell - its own wrap)
     __shared__ float4 ca_pos[kCenterChunk];   // centre atoms of this pass: same frame + atom index
-    __shared__ int4 ca_w[kCenterChunk];       // their wrap integers; .w = place of their cell in the run | pad end << 2
+    __shared__ int4 ca_w[kCenterChunk];       // their wrap integers; .w = place of their cell in the run
+    __shared__ int ca_pad[kCenterChunk];      // slot up to which their row has to be padded afterwards
     __shared__ int4 ca_meta[kCenterChunk];    // per batch of stencil cells: flat slot of the centre itself, first and
                                               // last candidate to scan; .w = running row length
     __shared__ int st_start[kStencilBatch];
@@ -718,23 +744,33 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
     const float rc2f = (float)a.rc2;
-    // each XCD (consecutive workgroups go to the 8 XCDs round-robin) walks one contiguous
-    // eighth of the units, so the stencil data it re-reads stays in its own L2
+    // Consecutive workgroups go to the 8 XCDs round-robin; the units are dealt to the XCDs in
+    // groups of consecutive units, so the stencil data an XCD re-reads stays in its own L2.  The
+    // dealing does not depend on the number of units: a workgroup asks for its first unit and
+    // for that number at the same time.
     const int xcd = blockIdx.x % 8, slot0 = blockIdx.x / 8, stride = gridDim.x / 8;
-    const int per_xcd = (total_units + 7) / 8;
+    const int group = a.unit_group;  // a power of two
+    const int last_unit = ws.max_cells - 1;
 
-    for (int li = slot0; li < per_xcd; li += stride) {
+    for (int li = slot0;; li += stride) {
         // NOTE: every thread of the workgroup takes the same path through this loop body
-        const int u = xcd * per_xcd + li;
-        if (u >= total_units) break;
-        const int4 unit = ws.units[u];
+        const int round0 = (li / group) * 8 * group;  // first unit of this round of 8 groups
+        const int u = round0 + xcd * group + li % group;
+        const int4* rec = reinterpret_cast<const int4*>(ws.units + (u < last_unit ? u : last_unit));
+        const int4 unit = rec[0], grid = rec[1];  // (asked for before u is known to exist)
+        if (round0 >= total_units) break;
+        if (u >= total_units) continue;
         const int c0 = __builtin_amdgcn_readfirstlane(unit.x);
         const int sidx = __builtin_amdgcn_readfirstlane(unit.y);
         const int cxyz = __builtin_amdgcn_readfirstlane(unit.z);
         const int run_len = __builtin_amdgcn_readfirstlane(unit.w);
+        const int nc_pack = __builtin_amdgcn_readfirstlane(grid.x);
+        const int rper = __builtin_amdgcn_readfirstlane(grid.y);
+        const int cell_offset = __builtin_amdgcn_readfirstlane(grid.z);
         if (a.rebuild && !a.rebuild[sidx]) continue;
-        const NlSearchSys S = ws.ssys[sidx];
-        const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
+        const NlSearchSys S = ws.ssys[sidx];  // (the cell steps and the tolerance are taken from here)
+        const int nc0 = (nc_pack & 1023) + 1, nc1 = ((nc_pack >> 10) & 1023) + 1, nc2 = ((nc_pack >> 20) & 1023) + 1;
+        const int per0 = (rper >> 18) & 1, per1 = (rper >> 19) & 1, per2 = (rper >> 20) & 1;
         const int cz0 = cxyz & 1023, cy = (cxyz >> 10) & 1023, cx = cxyz >> 20;
         const int c_begin = ws.cell_start[c0];
         // first centre atom (relative to c_begin) of the run's cells 1, 2, 3 and the run's end
@@ -744,7 +780,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         for (int r = 1; r <= kMaxRun; ++r) run_off[r] = ws.cell_start[c0 + (r < run_len ? r : run_len)] - c_begin;
         const int n_center = run_off[kMaxRun];
         if (n_center == 0) continue;
-        const int R0 = S.R[0], R1 = S.R[1], R2 = S.R[2];
+        const int R0 = rper & 63, R1 = (rper >> 6) & 63, R2 = (rper >> 12) & 63;
         const int e1 = 2 * R1 + 1, e01 = (2 * R0 + 1) * e1;
         const int n_layers = run_len + 2 * R2;
         const int n_stencil = n_layers * e01;
@@ -755,6 +791,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
 
         for (int cc0 = 0; cc0 < n_center; cc0 += kCenterChunk) {
             const int n_cc = (n_center - cc0) < kCenterChunk ? (n_center - cc0) : kCenterChunk;
+            int pad_end = 0;
             if ((int)threadIdx.x < n_cc) {
                 const int ca_abs = cc0 + (int)threadIdx.x;
                 int r = 0;
@@ -766,9 +803,11 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                 p.x += fr * S.step[6];
                 p.y += fr * S.step[7];
                 p.z += fr * S.step[8];
-                // what the row must be padded up to afterwards: all of it, or what the previous build left
-                const int old_cnt = a.tail_mode ? a.K : a.nn[__float_as_int(p.w)];
-                w.w = r | ((old_cnt < a.K ? old_cnt : a.K) << 2);
+                // what the row must be padded up to afterwards: all of it, or what the previous build
+                // left.  That count is a gather two loads deep; it is asked for here and stored to LDS
+                // only after the tile has been staged, so nothing before that waits for it.
+                pad_end = a.tail_mode ? a.K : a.nn[__float_as_int(p.w)];
+                w.w = r;
                 ca_pos[threadIdx.x] = p;
                 ca_w[threadIdx.x] = w;
                 ca_meta[threadIdx.x].w = 0;
@@ -785,11 +824,11 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         const int oz = layer - R2, oy = in_layer % e1 - R1, ox = in_layer / e1 - R0;
                         int gx = cx + ox, gy = cy + oy, gz = cz0 + oz;
                         bool ok = true;
-                        if (S.per[0]) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
-                        if (S.per[1]) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
-                        if (S.per[2]) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
+                        if (per0) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
+                        if (per1) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
+                        if (per2) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
                         if (ok) {
-                            int c2 = S.cell_offset + (gx * nc1 + gy) * nc2 + gz;
+                            int c2 = cell_offset + (gx * nc1 + gy) * nc2 + gz;
                             start = ws.cell_start[c2];
                             count = ws.cell_start[c2 + 1] - start;
                             float fx = (float)ox, fy = (float)oy, fz = (float)oz;
@@ -817,7 +856,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                 if ((int)threadIdx.x < n_cc) {
                     // The centre atom meets itself (shift 0) at exactly one slot of the flattened
                     // stencil: in its own cell, i.e. layer r + R2, at the middle of that layer.
-                    const int r = ca_w[threadIdx.x].w & 3;
+                    const int r = ca_w[threadIdx.x].w;
                     const int e_self = (r + R2) * e01 + R0 * e1 + R1;
                     int self_flat = -1;
                     if (e_self >= sb && e_self < sb + kStencilBatch) {
@@ -882,6 +921,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                     // the loop would begin each turn with a wait on "the loads that may still be in
                     // flight", which, the counter being in-order, waits for the previous centre
                     // atom's row stores instead.
+                    if ((int)threadIdx.x < n_cc) ca_pad[threadIdx.x] = pad_end < a.K ? pad_end : a.K;
                     __builtin_amdgcn_s_waitcnt(0x0F70);
                     __syncthreads();
 
@@ -896,7 +936,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         const int wi0 = __builtin_amdgcn_readfirstlane(wa.x);
                         const int wi1 = __builtin_amdgcn_readfirstlane(wa.y);
                         const int wi2 = __builtin_amdgcn_readfirstlane(wa.z);
-                        const int hi_slot = __builtin_amdgcn_readfirstlane(wa.w) >> 2;
+                        const int hi_slot = __builtin_amdgcn_readfirstlane(ca_pad[ca]);
                         const int4 meta = ca_meta[ca];
                         const int self_flat = __builtin_amdgcn_readfirstlane(meta.x);
                         const int k_self = self_flat >= 0 ? self_flat - t0 : -1;
@@ -1030,7 +1070,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                 for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
                     const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ca_pos[ca].w));
                     const int cnt = __builtin_amdgcn_readfirstlane(ca_meta[ca].w);
-                    const int hi_slot = __builtin_amdgcn_readfirstlane(ca_w[ca].w) >> 2;
+                    const int hi_slot = __builtin_amdgcn_readfirstlane(ca_pad[ca]);
                     int32_t* row = a.nm + (size_t)i_atom * a.K;
                     int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
                     for (int k = cnt + lane; k < hi_slot; k += kWave) {
@@ -1098,6 +1138,8 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     a.K = max_neighbors;
     a.half = half_fill ? 1 : 0;
     a.tail_mode = tail_mode ? 1 : 0;
+    a.unit_group = 1;
+    while (a.unit_group < 64 && (long long)a.unit_group * 8192 <= (long long)n_atoms) a.unit_group *= 2;
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
