@@ -35,6 +35,15 @@ for p in (ROOT, ROOT / "nvalchemi-toolkit_amd"):
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch on the default workload (256 boxes, seed 0), from rocprofv3 --pmc runs of
+# this script (FETCH_SIZE, then WRITE_SIZE; averages over the timed steps).  FETCH_SIZE reads
+# half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
+# bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
+MEASURED_TRAFFIC_BYTES = {
+    "nl": 1024 * (2 * (38459 + 6050) + (846514 + 59010)),   # search + per-system sort
+    "lj": 1024 * (2 * (522080 + 2442) + 16207),             # pair kernel + system ranges
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -218,7 +227,9 @@ def main() -> int:
     if stages:
         nl = stages["nl"]
         result["roofline"] = {"bound": "hbm", "achieved": nl["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                              "frac": nl["frac"], "traffic": None, "kernel": "neighbor build (nvamd_nl_build)",
+                              "frac": nl["frac"],
+                              "traffic": MEASURED_TRAFFIC_BYTES["nl"] if (B == 256 and args.relax_steps == 50) else None,
+                              "kernel": "neighbor build (nvamd_nl_build)",
                               "alg_bytes_per_launch": nl["alg_bytes"], "ms_per_launch": nl["ms"]}
         result["stages"] = stages
     if not args.no_cpu_baseline:
