@@ -159,6 +159,26 @@ int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces
 int32_t nvamd_segment_fmax(const float* forces, const int32_t* batch_idx, int32_t n_atoms,
                            int32_t n_systems, float* fmax, void* stream);
 
+/* Verlet-skin displacement test: replaces the Warp launch behind
+ * nvalchemi::_batch_neighbor_list_rebuild_inplace (nvalchemi/dynamics/_ops/neighbor_list_rebuild.py:37-139,
+ * called at nvalchemi/hooks/neighbor_list.py:295-311).  rebuild_flags (M) bool is cleared, then set for
+ * every system with an atom whose displacement from reference_positions exceeds threshold (strictly);
+ * with cell and pbc the displacement is taken by the minimum-image convention on the periodic axes
+ * (cell and pbc both given or both null).  With update_reference != 0 the reference positions of all
+ * atoms of the flagged systems are overwritten with the current ones. */
+int32_t nvamd_nl_rebuild_check(float* reference_positions, const float* current_positions,
+                               const int32_t* batch_idx, const float* cell, const uint8_t* pbc,
+                               int32_t n_atoms, int32_t n_systems, double threshold,
+                               int32_t update_reference, uint8_t* rebuild_flags, void* stream);
+
+/* Wrap positions into the cell, in place: replaces nvalchemi_hooks::wrap_positions and the masking
+ * after it (nvalchemi/hooks/periodic.py:42-114).  All three fractional coordinates are reduced to
+ * [0, 1) (frac = r . inv(cell), rows of cell = lattice vectors) and mapped back; of the result, the
+ * Cartesian components whose pbc flag is set replace the old ones, the others are kept (:111-113). */
+int32_t nvamd_wrap_positions(float* positions, const float* cell, const uint8_t* pbc,
+                             const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif

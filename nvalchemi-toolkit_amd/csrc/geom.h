@@ -32,6 +32,24 @@ __device__ __forceinline__ double pair_d2_exact(float xi, float yi, float zi, fl
     return (d0 * d0 + d1 * d1) + d2 * d2;
 }
 
+// inverse of a 3x3 matrix given row-major (adjugate over determinant)
+__device__ __forceinline__ void inv3(const double* m, double* inv) {
+    double c00 = m[4] * m[8] - m[5] * m[7];
+    double c01 = m[5] * m[6] - m[3] * m[8];
+    double c02 = m[3] * m[7] - m[4] * m[6];
+    double det = m[0] * c00 + m[1] * c01 + m[2] * c02;
+    double id = 1.0 / det;
+    inv[0] = c00 * id;
+    inv[1] = (m[2] * m[7] - m[1] * m[8]) * id;
+    inv[2] = (m[1] * m[5] - m[2] * m[4]) * id;
+    inv[3] = c01 * id;
+    inv[4] = (m[0] * m[8] - m[2] * m[6]) * id;
+    inv[5] = (m[2] * m[3] - m[0] * m[5]) * id;
+    inv[6] = c02 * id;
+    inv[7] = (m[1] * m[6] - m[0] * m[7]) * id;
+    inv[8] = (m[0] * m[4] - m[1] * m[3]) * id;
+}
+
 // blockIdx -> logical block so that each of the 8 XCDs (which receive consecutive
 // workgroups round-robin) walks one contiguous eighth of the index space and keeps its
 // own slice of the gathered data in its L2.

@@ -165,23 +165,6 @@ struct NlArgs {
     int32_t* shifts;
 };
 
-__device__ __forceinline__ void inv3(const double* m, double* inv) {
-    double c00 = m[4] * m[8] - m[5] * m[7];
-    double c01 = m[5] * m[6] - m[3] * m[8];
-    double c02 = m[3] * m[7] - m[4] * m[6];
-    double det = m[0] * c00 + m[1] * c01 + m[2] * c02;
-    double id = 1.0 / det;
-    inv[0] = c00 * id;
-    inv[1] = (m[2] * m[7] - m[1] * m[8]) * id;
-    inv[2] = (m[1] * m[5] - m[2] * m[4]) * id;
-    inv[3] = c01 * id;
-    inv[4] = (m[0] * m[8] - m[2] * m[6]) * id;
-    inv[5] = (m[2] * m[3] - m[0] * m[5]) * id;
-    inv[6] = c02 * id;
-    inv[7] = (m[1] * m[6] - m[0] * m[7]) * id;
-    inv[8] = (m[0] * m[4] - m[1] * m[3]) * id;
-}
-
 __device__ __forceinline__ void frac_of(const NlSys& s, const float* __restrict__ r, double* f) {
     double x = (double)r[0], y = (double)r[1], z = (double)r[2];
     f[0] = x * s.hinv[0] + y * s.hinv[3] + z * s.hinv[6];

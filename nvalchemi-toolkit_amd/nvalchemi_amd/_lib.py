@@ -40,6 +40,8 @@ _SIGNATURES = {
     "nvamd_fire_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_fire_step": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
+    "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
+    "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -280,3 +282,28 @@ def segment_fmax(forces, batch_idx, fmax) -> None:
     _check(library().nvamd_segment_fmax(
         _dev(forces, "forces", torch.float32, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         N, M, _dev(fmax, "fmax", torch.float32, (M,)), _stream(forces.device)), "nvamd_segment_fmax")
+
+
+def nl_rebuild_check(reference_positions, current_positions, batch_idx, rebuild_flags, threshold: float,
+                     update_reference: bool = False, cell=None, pbc=None) -> None:
+    N = current_positions.shape[0]
+    M = rebuild_flags.shape[0]
+    if (cell is None) != (pbc is None):
+        cell = pbc = None  # the displacement is plain unless both are given
+    _check(library().nvamd_nl_rebuild_check(
+        _dev(reference_positions, "reference_positions", torch.float32, (N, 3)),
+        _dev(current_positions, "current_positions", torch.float32, (N, 3)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _opt(cell, "cell", torch.float32, (M, 3, 3)), _opt(_as_u8(pbc), "pbc", torch.uint8, (M, 3)),
+        N, M, float(threshold), int(bool(update_reference)),
+        _dev(_as_u8(rebuild_flags), "rebuild_flags", torch.uint8, (M,)),
+        _stream(current_positions.device)), "nvamd_nl_rebuild_check")
+
+
+def wrap_positions(positions, cell, pbc, batch_idx) -> None:
+    N = positions.shape[0]
+    M = cell.shape[0]
+    _check(library().nvamd_wrap_positions(
+        _dev(positions, "positions", torch.float32, (N, 3)), _dev(cell, "cell", torch.float32, (M, 3, 3)),
+        _dev(_as_u8(pbc), "pbc", torch.uint8, (M, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        N, M, _stream(positions.device)), "nvamd_wrap_positions")

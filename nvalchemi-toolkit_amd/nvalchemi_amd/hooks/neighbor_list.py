@@ -11,8 +11,11 @@ over-estimated, never below the override; :401-486), and the published batch key
 Differences in mechanism, not in results: there are no staging copies (the kernels read the
 batch tensors directly), and the padding of rows is maintained by the build kernel itself
 instead of a masked fill over the whole ``(N,K)`` buffers after every build (:377-380).
-With ``skin > 0`` the list is searched out to ``cutoff + skin`` as the reference does, but it
-is rebuilt on every call (the displacement test that skips rebuilds is not implemented).
+With ``skin > 0`` the list is searched out to ``cutoff + skin`` and, from the second call on, only
+the systems in which some atom moved more than ``skin / 2`` since their last build are rebuilt
+(:295-311): the displacement test writes the per-system ``_rebuild_flags`` and refreshes
+``_ref_positions`` for the flagged systems, and the build kernel leaves the rows of the others as
+they are.  The potential applies the bare cutoff to the wider list.
 """
 
 from __future__ import annotations
@@ -22,6 +25,7 @@ from enum import Enum
 import torch
 
 from .._neighbor_ops import ceil16, estimate_max_neighbors, neighbor_list
+from ..dynamics._ops.neighbor_list_rebuild import batch_neighbor_list_rebuild_inplace
 from ..models.base import NeighborConfig, NeighborListFormat
 from ..neighbors import _write_neighbor_data_to_batch
 from ._context import HookContext
@@ -65,9 +69,15 @@ class NeighborListHook:
         self._neighbor_list_method: str | None = None
         self._actual_max_k: torch.Tensor | None = None
         self._first_build: bool = True
+        # Verlet-skin state: positions at the last build of each system, per-system flags
+        self._ref_positions: torch.Tensor | None = None
+        self._rebuild_flags: torch.Tensor | None = None
 
     def __call__(self, ctx: HookContext, stage: Enum) -> None:
         self._rebuild(ctx.batch)
+        # first build: initialise the skin reference (one-time clone)
+        if self.skin > 0.0 and self._ref_positions is None:
+            self._ref_positions = ctx.batch.positions.detach().clone()
 
     # ------------------------------------------------------------------
     def _rebuild(self, batch) -> None:
@@ -89,8 +99,21 @@ class NeighborListHook:
             self._alloc_N = N
             self._alloc_B = B
 
+        if self._rebuild_flags is None or self._rebuild_flags.shape[0] != B \
+                or self._rebuild_flags.device != positions.device:
+            # all true, so that a first build (before the reference exists) is a full one
+            self._rebuild_flags = torch.ones(B, dtype=torch.bool, device=positions.device)
+            self._ref_positions = None
+        if self.skin > 0.0 and self._ref_positions is not None:
+            batch_neighbor_list_rebuild_inplace(
+                reference_positions=self._ref_positions, current_positions=positions,
+                batch_idx=batch.batch_idx, rebuild_flags=self._rebuild_flags,
+                skin_distance_threshold=self.skin / 2, update_reference_positions=True,
+                cell=cell if periodic else None, pbc=pbc)
+
         cutoff = self.config.cutoff + self.skin
-        self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
+        self._build(batch, cutoff, cell, pbc,
+                    rebuild_flags=self._rebuild_flags if (self.skin > 0.0 and self._ref_positions is not None) else None)
 
         if self._first_build:
             # the one host synchronisation: validate K against the actual maximum
@@ -130,6 +153,9 @@ class NeighborListHook:
         self._realloc_k(N, batch.device, pbc)
         self._first_build = True
         self._actual_max_k = None
+        # new buffers hold no list: the next build is a full one and re-initialises the reference
+        self._ref_positions = None
+        self._rebuild_flags = None
 
     def _realloc_k(self, N: int, device: torch.device, pbc: torch.Tensor | None) -> None:
         K = self._max_neighbors

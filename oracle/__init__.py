@@ -60,6 +60,11 @@ def lib() -> ctypes.CDLL:
             [_f32p] * 5 + [_i32p, _u8p, ctypes.c_int32, ctypes.c_int32]
         L.orc_fmax.restype = None
         L.orc_fmax.argtypes = [_f32p, _i32p, ctypes.c_int32, ctypes.c_int32, _f32p]
+        L.orc_rebuild_check.restype = None
+        L.orc_rebuild_check.argtypes = [_f32p, _f32p, _i32p, _f32p, _u8p, ctypes.c_int32, ctypes.c_int32,
+                                        ctypes.c_double, ctypes.c_int32, _u8p]
+        L.orc_wrap_positions.restype = None
+        L.orc_wrap_positions.argtypes = [_f32p, _f32p, _u8p, _i32p, ctypes.c_int32]
         L.orc_num_threads.restype = ctypes.c_int32
         _lib = L
     return _lib
@@ -233,3 +238,25 @@ def fmax(forces, batch_idx, n_systems: int) -> np.ndarray:
     lib().orc_fmax(_p(f, _f32p), _p(_i32(batch_idx), _i32p), f.shape[0], int(n_systems),
                    _p(out, _f32p))
     return out
+
+
+def rebuild_check(reference_positions, current_positions, batch_idx, n_systems: int, threshold: float,
+                  update_reference: bool = False, cell=None, pbc=None):
+    """Verlet-skin displacement test -> ``(flags (M) bool, reference positions after the call)``."""
+    ref = _f32(reference_positions).copy()
+    cur = _f32(current_positions)
+    c = None if cell is None else _f32(cell).reshape(-1, 9)
+    p = None if (pbc is None or cell is None) else _u8(pbc).reshape(-1, 3)
+    flags = np.zeros(int(n_systems), dtype=np.uint8)
+    lib().orc_rebuild_check(_p(ref, _f32p), _p(cur, _f32p), _p(_i32(batch_idx), _i32p), _p(c, _f32p),
+                            _p(p, _u8p), ref.shape[0], int(n_systems), float(threshold),
+                            int(update_reference), _p(flags, _u8p))
+    return flags.astype(bool), ref
+
+
+def wrap_positions(positions, cell, pbc, batch_idx) -> np.ndarray:
+    """Positions wrapped into their cells (a copy), per-axis flags as the reference applies them."""
+    pos = _f32(positions).copy()
+    lib().orc_wrap_positions(_p(pos, _f32p), _p(_f32(cell).reshape(-1, 9), _f32p),
+                             _p(_u8(pbc).reshape(-1, 3), _u8p), _p(_i32(batch_idx), _i32p), pos.shape[0])
+    return pos

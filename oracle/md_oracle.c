@@ -22,6 +22,9 @@
  *                                nvalchemi/dynamics/optimizers/fire.py:69-76,182-219,
  *                                nvalchemi/distributed/_dynamics_coordinator.py:296-322
  *   orc_fmax                     nvalchemi/dynamics/base.py:304-349
+ *   orc_rebuild_check            nvalchemi/dynamics/_ops/neighbor_list_rebuild.py:37-139 (the
+ *                                displacement kernel itself is in the absent wheel)
+ *   orc_wrap_positions           nvalchemi/hooks/periodic.py:42-114
  *
  * Pinning status (what checks each function; see tests/test_oracle_*.py):
  *   orc_nl_brute   pinned: hand geometries restated from the reference tests
@@ -44,6 +47,15 @@
  *                  notes (reductions at entry; mixing with the stored alpha; per-atom
  *                  maxstep clamp; vanilla branch only).  Checked by invariants only.
  *   orc_fmax       pinned: in-tree Torch definition is complete; literal cases.
+ *   orc_rebuild_check  pinned by the reference's own cases (flags cleared on every call, 1.0 over a
+ *                  threshold of 0.5 flags, 0.1 does not, per-system selectivity, reference refreshed
+ *                  only when flagged: test/hooks/test_neighbor_list_hook.py:166-246).  PARITY UNPINNED:
+ *                  strict versus non-strict comparison at the threshold, the minimum-image form of the
+ *                  displacement, and whether the refresh covers the flagged system's unmoved atoms
+ *                  (taken: strict, nearest image on periodic axes, whole system).
+ *   orc_wrap_positions  pinned by the documented formula (frac = r . inv(cell), frac mod 1, back;
+ *                  nvalchemi/hooks/periodic.py:159-163) and the in-tree masking (:111-113); the
+ *                  float32 rounding of the absent Warp kernel is unpinned (computed in double here).
  *
  * Numerical definition of the neighbor set: the pair (i, j, S) is a neighbor iff
  *   d = (r_j - r_i) + (S0*a0 + S1*a1 + S2*a2),  d.d < rc*rc
@@ -553,4 +565,59 @@ ORC_API int32_t orc_num_threads(void) {
 #else
     return 1;
 #endif
+}
+
+/* Verlet-skin displacement test.  flags (M) are cleared, then set for systems holding an atom
+ * that moved more than threshold from ref; with cell/pbc the nearest image on periodic axes.
+ * With update_reference, ref <- cur for all atoms of flagged systems. */
+ORC_API void orc_rebuild_check(float* ref, const float* cur, const int32_t* batch_idx, const float* cell,
+                               const uint8_t* pbc, int32_t n_atoms, int32_t n_systems, double threshold,
+                               int32_t update_reference, uint8_t* flags) {
+    int i, k;
+    for (i = 0; i < n_systems; ++i) flags[i] = 0;
+    for (i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        double d[3];
+        for (k = 0; k < 3; ++k) d[k] = (double)cur[3 * (size_t)i + k] - (double)ref[3 * (size_t)i + k];
+        if (cell && pbc && (pbc[3 * s] | pbc[3 * s + 1] | pbc[3 * s + 2])) {
+            orc_sys_t sys;
+            double f[3];
+            orc_sys_init(&sys, cell + 9 * (size_t)s, pbc + 3 * (size_t)s);
+            f[0] = (d[0] * sys.hinv[0] + d[1] * sys.hinv[3]) + d[2] * sys.hinv[6];
+            f[1] = (d[0] * sys.hinv[1] + d[1] * sys.hinv[4]) + d[2] * sys.hinv[7];
+            f[2] = (d[0] * sys.hinv[2] + d[1] * sys.hinv[5]) + d[2] * sys.hinv[8];
+            for (k = 0; k < 3; ++k)
+                if (sys.per[k]) f[k] -= rint(f[k]);
+            for (k = 0; k < 3; ++k) d[k] = (f[0] * sys.h[k] + f[1] * sys.h[3 + k]) + f[2] * sys.h[6 + k];
+        }
+        if ((d[0] * d[0] + d[1] * d[1]) + d[2] * d[2] > threshold * threshold) flags[s] = 1;
+    }
+    if (update_reference)
+        for (i = 0; i < n_atoms; ++i)
+            if (flags[batch_idx[i]])
+                for (k = 0; k < 3; ++k) ref[3 * (size_t)i + k] = cur[3 * (size_t)i + k];
+}
+
+/* Wrap into the cell: all three fractional coordinates mod 1, back to Cartesian, and of that
+ * the components whose own pbc flag is set (the others keep their old value). */
+ORC_API void orc_wrap_positions(float* pos, const float* cell, const uint8_t* pbc, const int32_t* batch_idx,
+                                int32_t n_atoms) {
+    int i, k;
+    for (i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        orc_sys_t sys;
+        double f[3], w[3];
+        if (!(pbc[3 * s] | pbc[3 * s + 1] | pbc[3 * s + 2])) continue;
+        orc_sys_init(&sys, cell + 9 * (size_t)s, pbc + 3 * (size_t)s);
+        {
+            double x = pos[3 * (size_t)i], y = pos[3 * (size_t)i + 1], z = pos[3 * (size_t)i + 2];
+            f[0] = (x * sys.hinv[0] + y * sys.hinv[3]) + z * sys.hinv[6];
+            f[1] = (x * sys.hinv[1] + y * sys.hinv[4]) + z * sys.hinv[7];
+            f[2] = (x * sys.hinv[2] + y * sys.hinv[5]) + z * sys.hinv[8];
+        }
+        for (k = 0; k < 3; ++k) f[k] -= floor(f[k]);
+        for (k = 0; k < 3; ++k) w[k] = (f[0] * sys.h[k] + f[1] * sys.h[3 + k]) + f[2] * sys.h[6 + k];
+        for (k = 0; k < 3; ++k)
+            if (sys.per[k]) pos[3 * (size_t)i + k] = (float)w[k];
+    }
 }
