@@ -71,6 +71,7 @@ struct NlSearchSys {
     int per[3];
     int cell_offset;
     int zr;
+    float half_diag;  // half of the longest body diagonal of one cell
 };
 
 // One unit of search work: a run of cells along axis 2, with what the enumeration of its
@@ -84,7 +85,7 @@ struct __attribute__((aligned(32))) NlUnit {
     int nc_pack;      // cells per axis minus one, 10 bits each: (nc0-1) | (nc1-1) << 10 | (nc2-1) << 20
     int rper_pack;    // stencil radii, 6 bits each, then the periodic flags: R0 | R1 << 6 | R2 << 12 | per << 18
     int cell_offset;  // first cell of the system
-    int pad;
+    int first_centre; // the unit covers centre atoms first_centre .. +kCenterChunk of the run; -1: all of them
 };
 static_assert(sizeof(NlUnit) == 32, "read as two 16-byte words");
 static_assert(kMaxStencilRadius < 64, "stencil radii are packed 6 bits each");
@@ -320,6 +321,17 @@ __device__ __forceinline__ NlSearchSys search_view(const NlSys& s) {
     }
     q.cell_offset = s.cell_offset;
     q.zr = s.zr;
+    float d2max = 0.f;
+    for (int sg = 0; sg < 4; ++sg) {
+        const float a = (sg & 1) ? -1.f : 1.f, b = (sg & 2) ? -1.f : 1.f;
+        float d2 = 0.f;
+        for (int k = 0; k < 3; ++k) {
+            const float v = q.step[k] + a * q.step[3 + k] + b * q.step[6 + k];
+            d2 += v * v;
+        }
+        d2max = d2 > d2max ? d2 : d2max;
+    }
+    q.half_diag = 0.5f * sqrtf(d2max) * 1.0001f;
     return q;
 }
 
@@ -423,7 +435,7 @@ __device__ __forceinline__ NlUnit make_unit(const NlSearchSys& q, int lu, int ru
     u.rper_pack = q.R[0] | (q.R[1] << 6) | (q.R[2] << 12) | ((q.per[0] ? 1 : 0) << 18) | ((q.per[1] ? 1 : 0) << 19) |
                   ((q.per[2] ? 1 : 0) << 20);
     u.cell_offset = q.cell_offset;
-    u.pad = 0;
+    u.first_centre = -1;
     return u;
 }
 
@@ -496,7 +508,8 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
     __shared__ uint32_t s_bounds[6];
     __shared__ int s_err;
     __shared__ int s_unit0;
-    __shared__ int s_hist[kSortCells];
+    __shared__ NlSearchSys s_view;
+    __shared__ int s_hist[kSortCells + 1];  // counts, then first atoms (and the end of the last cell)
     __shared__ int s_part[kSortBlock / kWave];
     const int t = blockIdx.x;
     const int tid = threadIdx.x;
@@ -550,9 +563,6 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         s_sys.error = s_err;
         s_sys.cell_offset = cell_base;
         ws.cell_offset[t] = cell_base;
-        // this system's units: a contiguous piece of the unit list, wherever the counter stands
-        // (the order of systems in the list is of no consequence)
-        s_unit0 = s_sys.n_units > 0 ? atomicAdd(&ws.hdr->total_units, s_sys.n_units) : 0;
         if (s_err) atomicOr(&ws.hdr->error, s_err);
     }
     __syncthreads();
@@ -562,10 +572,10 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         int* dst = reinterpret_cast<int*>(ws.sys + t);
         for (int w = tid; w < (int)(sizeof(NlSys) / sizeof(int)); w += kSortBlock) dst[w] = src[w];
         const NlSearchSys q = search_view(s_sys);
-        if (tid == 0) ws.ssys[t] = q;
-        const int n_units = s_sys.n_units, unit0 = s_unit0;
-        const int runs = (q.nc[2] + q.zr - 1) / q.zr;
-        for (int lu = tid; lu < n_units; lu += kSortBlock) ws.units[unit0 + lu] = make_unit(q, lu, runs, t);
+        if (tid == 0) {
+            ws.ssys[t] = q;
+            s_view = q;
+        }
     }
     if (idle) return;
     const int n_cells = s_sys.n_cells;
@@ -618,7 +628,10 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
             }
             running += n;
         }
-        if (tid == 0) g_start[n_cells] = end;
+        if (tid == 0) {
+            g_start[n_cells] = end;
+            if (in_lds) s_hist[n_cells] = end;
+        }
     }
     __syncthreads();
     // ---- scatter into cell order
@@ -637,6 +650,40 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         }
     } else {
         for (int i = begin + tid; i < end; i += kSortBlock) place(bin_atom(s_sys, a.pos + 3 * (size_t)i), i, ws.atom_rank[i]);
+    }
+    __syncthreads();
+    // ---- the system's units of search work.  A run of cells with more centre atoms than one
+    //      pass of the search takes is split into one unit per pass (so that a system that is one
+    //      crowded cell does not end up on a single workgroup); empty runs get none.
+    {
+        const NlSearchSys& q = s_view;
+        const int n_runs = s_sys.n_units;
+        const int runs = (q.nc[2] + q.zr - 1) / q.zr;
+        auto first_atom = [&](int lc) {
+            return in_lds ? s_hist[lc] : __hip_atomic_load(&g_start[lc], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
+        auto passes_of = [&](const NlUnit& u) {
+            const int lc0 = u.c0 - cell_base;
+            const int n_centre = first_atom(lc0 + u.run_len) - first_atom(lc0);
+            return (n_centre + kCenterChunk - 1) / kCenterChunk;
+        };
+        int mine_units = 0;
+        for (int lu = tid; lu < n_runs; lu += kSortBlock) mine_units += passes_of(make_unit(q, lu, runs, t));
+        int total;
+        const int before = block_exclusive_scan(mine_units, s_part, &total);
+        // a contiguous piece of the unit list, wherever the counter stands (the order of the
+        // systems in the list is of no consequence)
+        if (tid == 0) s_unit0 = total > 0 ? atomicAdd(&ws.hdr->total_units, total) : 0;
+        __syncthreads();
+        NlUnit* out = ws.units + s_unit0 + before;
+        for (int lu = tid; lu < n_runs; lu += kSortBlock) {
+            NlUnit u = make_unit(q, lu, runs, t);
+            const int passes = passes_of(u);
+            for (int k = 0; k < passes; ++k) {
+                u.first_centre = passes > 1 ? k * kCenterChunk : -1;
+                *out++ = u;
+            }
+        }
     }
 }
 
@@ -727,6 +774,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
     const float rc2f = (float)a.rc2;
+    const float cull_reach = (float)a.rcb * 1.001f;
     // Consecutive workgroups go to the 8 XCDs round-robin; the units are dealt to the XCDs in
     // groups of consecutive units, so the stencil data an XCD re-reads stays in its own L2.  The
     // dealing does not depend on the number of units: a workgroup asks for its first unit and
@@ -772,8 +820,12 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         const bool one_batch = n_stencil <= kStencilBatch;
         const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
 
-        for (int cc0 = 0; cc0 < n_center; cc0 += kCenterChunk) {
-            const int n_cc = (n_center - cc0) < kCenterChunk ? (n_center - cc0) : kCenterChunk;
+        // the run's centre atoms, one pass at a time; or the one pass this unit stands for
+        const int first_centre = __builtin_amdgcn_readfirstlane(grid.w);
+        const int cc_begin = first_centre >= 0 ? first_centre : 0;
+        const int cc_end = (first_centre >= 0 && first_centre + kCenterChunk < n_center) ? first_centre + kCenterChunk : n_center;
+        for (int cc0 = cc_begin; cc0 < cc_end; cc0 += kCenterChunk) {
+            const int n_cc = (cc_end - cc0) < kCenterChunk ? (cc_end - cc0) : kCenterChunk;
             int pad_end = 0;
             if ((int)threadIdx.x < n_cc) {
                 const int ca_abs = cc0 + (int)threadIdx.x;
@@ -811,13 +863,27 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         if (per1) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
                         if (per2) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
                         if (ok) {
-                            int c2 = cell_offset + (gx * nc1 + gy) * nc2 + gz;
-                            start = ws.cell_start[c2];
-                            count = ws.cell_start[c2 + 1] - start;
                             float fx = (float)ox, fy = (float)oy, fz = (float)oz;
                             o0 = fx * S.step[0] + fy * S.step[3] + fz * S.step[6];
                             o1 = fx * S.step[1] + fy * S.step[4] + fz * S.step[7];
                             o2 = fx * S.step[2] + fy * S.step[5] + fz * S.step[8];
+                            // Skewed cells put far-away images into the stencil.  A cell whose centre is
+                            // further than the search radius plus two half-diagonals from the centre of
+                            // every cell of the run holds no neighbor (no two points of two cells are
+                            // closer than their centres minus the half-diagonals): it is left empty.
+                            float best = 3.0e38f;
+                            for (int r = 0; r < run_len; ++r) {
+                                const float dx = o0 - (float)r * S.step[6], dy = o1 - (float)r * S.step[7],
+                                            dz = o2 - (float)r * S.step[8];
+                                const float d2 = dx * dx + dy * dy + dz * dz;
+                                best = d2 < best ? d2 : best;
+                            }
+                            const float lim = cull_reach + 2.0f * S.half_diag;
+                            if (best <= lim * lim) {
+                                int c2 = cell_offset + (gx * nc1 + gy) * nc2 + gz;
+                                start = ws.cell_start[c2];
+                                count = ws.cell_start[c2 + 1] - start;
+                            }
                         }
                     }
                     int incl = count;
