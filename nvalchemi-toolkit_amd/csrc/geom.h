@@ -17,6 +17,27 @@ struct Cell64 {
     double h[9];
 };
 
+// S . cell in the fixed association of the definition above (cell given as float32 rows)
+__device__ __forceinline__ void shift_vector(const float* __restrict__ cell, int s0, int s1, int s2, double& tx,
+                                             double& ty, double& tz) {
+#pragma clang fp contract(off)
+    const double a = (double)s0, b = (double)s1, c = (double)s2;
+    tx = (a * (double)cell[0] + b * (double)cell[3]) + c * (double)cell[6];
+    ty = (a * (double)cell[1] + b * (double)cell[4]) + c * (double)cell[7];
+    tz = (a * (double)cell[2] + b * (double)cell[5]) + c * (double)cell[8];
+}
+
+// d = (r_j - r_i) + t and its square, t = S . cell already evaluated
+__device__ __forceinline__ double pair_d2_shifted(float xi, float yi, float zi, float xj, float yj, float zj,
+                                                  double tx, double ty, double tz, double& d0, double& d1,
+                                                  double& d2) {
+#pragma clang fp contract(off)
+    d0 = ((double)xj - (double)xi) + tx;
+    d1 = ((double)yj - (double)yi) + ty;
+    d2 = ((double)zj - (double)zi) + tz;
+    return (d0 * d0 + d1 * d1) + d2 * d2;
+}
+
 __device__ __forceinline__ double pair_d2_exact(float xi, float yi, float zi, float xj, float yj,
                                                 float zj, int s0, int s1, int s2,
                                                 const double* __restrict__ h, double& d0,

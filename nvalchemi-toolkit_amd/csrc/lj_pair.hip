@@ -80,6 +80,7 @@ __device__ __forceinline__ double reciprocal(double x) {
 template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC>
 __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, int sys_base,
                                         const float* __restrict__ s_pos, int span0, int span_n,
+                                        const double (*s_shift)[3], int table_sys,
                                         double (*s_acc)[VIRIAL ? 7 : 1]) {
     constexpr int G = kBlockFull / LPR;
     const int g = threadIdx.x / LPR;
@@ -92,15 +93,10 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
         cnt = cnt < a.K ? cnt : a.K;
         const float* pi = a.pos + 3 * (size_t)i;
         const float xi = pi[0], yi = pi[1], zi = pi[2];
-        double h[9];
-        if (SHIFTS) {
-            const float* c = a.cells + 9 * (size_t)sys;
-#pragma unroll
-            for (int k = 0; k < 9; ++k) h[k] = (double)c[k];
-        } else {
-#pragma unroll
-            for (int k = 0; k < 9; ++k) h[k] = 0.0;
-        }
+        // shift . cell comes from the LDS table of the system in hand (shifts of -1, 0, 1) or, for
+        // anything else, from the cell in memory: the nine cell components stay out of the registers
+        const bool tabled = SHIFTS && sys == table_sys;
+        const float* cell_row = SHIFTS ? a.cells + 9 * (size_t)sys : nullptr;
         const int32_t* row = a.nm + (size_t)i * a.K;
         const int32_t* srow = SHIFTS ? a.shifts + (size_t)i * a.K * 3 : nullptr;
         // UNROLL row entries per lane are in flight at once: first every index and shift of the
@@ -172,8 +168,20 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
             }
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
+                double t0 = 0.0, t1 = 0.0, t2 = 0.0;
+                if (SHIFTS) {
+                    const unsigned c0 = (unsigned)(s0[u] + 1), c1 = (unsigned)(s1[u] + 1), c2 = (unsigned)(s2[u] + 1);
+                    if (tabled && c0 < 3u && c1 < 3u && c2 < 3u) {
+                        const double* t = s_shift[(c0 * 3 + c1) * 3 + c2];
+                        t0 = t[0];
+                        t1 = t[1];
+                        t2 = t[2];
+                    } else if (jj[u] >= 0) {
+                        shift_vector(cell_row, s0[u], s1[u], s2[u], t0, t1, t2);
+                    }
+                }
                 double d0, d1, d2;
-                double r2 = pair_d2_exact(xi, yi, zi, xj[u], yj[u], zj[u], s0[u], s1[u], s2[u], h, d0, d1, d2);
+                double r2 = pair_d2_shifted(xi, yi, zi, xj[u], yj[u], zj[u], t0, t1, t2, d0, d1, d2);
                 if (jj[u] < 0 || !(r2 < a.rc2)) continue;
                 const double ir2 = reciprocal(r2);
                 double q2 = a.sig2 * ir2;
@@ -239,10 +247,12 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
 }
 
 template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool VEC>
-__global__ __launch_bounds__(kBlockFull) void lj_matrix_kernel(LjArgs a) {
+// (six waves per SIMD: three workgroups per CU; the virial variant needs more registers than that leaves)
+__global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_matrix_kernel(LjArgs a) {
     constexpr int NV = VIRIAL ? 7 : 1;
     __shared__ double s_acc[kSysSlots][NV];
     __shared__ float s_pos[3 * kLdsAtoms];
+    __shared__ double s_shift[27][3];  // shift . cell of the system in hand, shifts -1..1 per axis
 
     // a workgroup owns rows_per_block consecutive rows; workgroups are numbered so that each
     // XCD walks one contiguous eighth of the atoms
@@ -271,9 +281,16 @@ __global__ __launch_bounds__(kBlockFull) void lj_matrix_kernel(LjArgs a) {
             const float* src = a.pos + 3 * (size_t)span0;
             for (int t = threadIdx.x; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
         }
+        if (SHIFTS && threadIdx.x < 27) {
+            const int t = threadIdx.x;
+            shift_vector(a.cells + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
+                         s_shift[t][2]);
+        }
         __syncthreads();
-        if (staged) lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_acc);
-        else lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_acc);
+        if (staged)
+            lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift, sys, s_acc);
+        else
+            lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys, s_acc);
         r = seg_end;
         if (r < row_end) __syncthreads();  // the stage is about to be overwritten
     }

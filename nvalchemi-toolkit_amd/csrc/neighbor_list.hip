@@ -72,6 +72,7 @@ struct NlSearchSys {
     int cell_offset;
     int zr;
     float half_diag;  // half of the longest body diagonal of one cell
+    float cull_far;   // distance of the farthest stencil cell centre from its run's nearest cell centre
 };
 
 // One unit of search work: a run of cells along axis 2, with what the enumeration of its
@@ -332,6 +333,18 @@ __device__ __forceinline__ NlSearchSys search_view(const NlSys& s) {
         d2max = d2 > d2max ? d2 : d2max;
     }
     q.half_diag = 0.5f * sqrtf(d2max) * 1.0001f;
+    // the stencil cell furthest from a run's nearest cell is a corner of the stencil
+    float far2 = 0.f;
+    for (int sg = 0; sg < 4; ++sg) {
+        const float a = (sg & 1) ? -1.f : 1.f, b = (sg & 2) ? -1.f : 1.f;
+        float d2 = 0.f;
+        for (int k = 0; k < 3; ++k) {
+            const float v = (float)q.R[0] * q.step[k] + a * (float)q.R[1] * q.step[3 + k] + b * (float)q.R[2] * q.step[6 + k];
+            d2 += v * v;
+        }
+        far2 = d2 > far2 ? d2 : far2;
+    }
+    q.cull_far = sqrtf(far2) * 1.0001f;
     return q;
 }
 
@@ -819,6 +832,8 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         // every centre atom scans only the layers of its own cell's stencil
         const bool one_batch = n_stencil <= kStencilBatch;
         const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
+        // (square cells never have a stencil cell out of reach: the test is skipped for them)
+        const bool may_cull = S.cull_far > cull_reach + 2.0f * S.half_diag;
 
         // the run's centre atoms, one pass at a time; or the one pass this unit stands for
         const int first_centre = __builtin_amdgcn_readfirstlane(grid.w);
@@ -871,8 +886,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             // further than the search radius plus two half-diagonals from the centre of
                             // every cell of the run holds no neighbor (no two points of two cells are
                             // closer than their centres minus the half-diagonals): it is left empty.
-                            float best = 3.0e38f;
-                            for (int r = 0; r < run_len; ++r) {
+                            float best = 0.f;
+                            if (may_cull) best = 3.0e38f;
+                            for (int r = 0; may_cull && r < run_len; ++r) {
                                 const float dx = o0 - (float)r * S.step[6], dy = o1 - (float)r * S.step[7],
                                             dz = o2 - (float)r * S.step[8];
                                 const float d2 = dx * dx + dy * dy + dz * dz;
