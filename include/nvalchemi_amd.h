@@ -159,6 +159,30 @@ int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces
 int32_t nvamd_segment_fmax(const float* forces, const int32_t* batch_idx, int32_t n_atoms,
                            int32_t n_systems, float* fmax, void* stream);
 
+/* The same, walking the rows in a given order: row_order (N) i32 is a permutation of 0..N-1 in which
+ * the atoms of each system stay together and in system order (e.g. the cell order of the last neighbor
+ * build, nvamd_nl_atom_order), or null.  Results do not depend on it; for systems too large to stage in
+ * LDS, an order with spatial locality keeps the gathers of neighbor positions in the caches.  No
+ * counterpart in the reference. */
+int32_t nvamd_lj_energy_forces_ordered(const float* positions, const float* cells,
+                                       const int32_t* neighbor_matrix,
+                                       const int32_t* neighbor_matrix_shifts,
+                                       const int32_t* num_neighbors, const int32_t* batch_idx,
+                                       const int32_t* row_order, int32_t n_atoms, int32_t max_neighbors,
+                                       int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
+                                       double cutoff, double switch_width, int32_t half_list,
+                                       float* atomic_energies, float* forces, float* virials,
+                                       float* system_energies, void* workspace, size_t workspace_bytes,
+                                       void* stream);
+
+/* Atom indices in the cell order of the neighbor build that last used this workspace with the same
+ * n_atoms / n_systems: atom_order[k] for k in a system's range [batch_ptr[s], batch_ptr[s+1]) are that
+ * system's atoms, cell by cell.  With rebuild_flags, only the ranges of flagged systems are written
+ * (the others were not sorted by that build).  No counterpart in the reference. */
+int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
+                            const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                            int32_t* atom_order, void* stream);
+
 /* Verlet-skin displacement test: replaces the Warp launch behind
  * nvalchemi::_batch_neighbor_list_rebuild_inplace (nvalchemi/dynamics/_ops/neighbor_list_rebuild.py:37-139,
  * called at nvalchemi/hooks/neighbor_list.py:295-311).  rebuild_flags (M) bool is cleared, then set for

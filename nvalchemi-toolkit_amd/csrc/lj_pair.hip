@@ -39,6 +39,7 @@ struct LjArgs {
     double* sys_acc;  // (B, 1 + 9): energy then virial, fp64, zeroed before the launch
     unsigned n_blocks;
     int rows_per_block;
+    const int32_t* order;      // (N) row k of the kernel's walk is atom order[k]; null: the identity
     const int32_t* sys_first;  // (B) first atom of each non-empty system
     const int32_t* sys_last;   // (B) one past its last atom
     int lds_atoms;             // stage positions in LDS when the systems of a run have at most this many atoms
@@ -85,7 +86,8 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
     constexpr int G = kBlockFull / LPR;
     const int g = threadIdx.x / LPR;
     const int sub = threadIdx.x % LPR;
-    for (int i = row0 + g; i < row_end; i += G) {
+    for (int k_row = row0 + g; k_row < row_end; k_row += G) {
+        const int i = a.order ? a.order[k_row] : k_row;
         double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
         double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;  // xx xy xz yy yz zz
         const int sys = a.bidx[i];
@@ -261,14 +263,14 @@ __global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_matrix_kernel(L
     const int row0 = (int)lb * a.rows_per_block;
     const int row_end = (row0 + a.rows_per_block) < a.n_atoms ? (row0 + a.rows_per_block) : a.n_atoms;
     if (row0 >= row_end) return;
-    const int sys_lo = a.bidx[row0];
+    const int sys_lo = a.bidx[a.order ? a.order[row0] : row0];
     if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
 
     // Neighbors live in the system of their row: the rows are taken one system at a time, with
     // that system's positions staged in LDS when they fit (atom order carries no spatial
     // locality, so gathers through the caches move a whole line per 12 useful bytes).
     for (int r = row0; r < row_end;) {
-        const int sys = a.bidx[r];
+        const int sys = a.bidx[a.order ? a.order[r] : r];
         const int span0 = a.sys_first[sys];
         const int span_end = a.sys_last[sys];
         const int span_n = span_end - span0;
@@ -478,6 +480,22 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
                                             int32_t half_list, float* atomic_energies, float* forces,
                                             float* virials, float* system_energies, void* workspace,
                                             size_t workspace_bytes, void* stream) {
+    return nvamd_lj_energy_forces_ordered(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
+                                          batch_idx, nullptr, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
+                                          sigma, cutoff, switch_width, half_list, atomic_energies, forces, virials,
+                                          system_energies, workspace, workspace_bytes, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_ordered(const float* positions, const float* cells,
+                                                    const int32_t* neighbor_matrix,
+                                                    const int32_t* neighbor_matrix_shifts,
+                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
+                                                    const int32_t* row_order, int32_t n_atoms,
+                                                    int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
+                                                    double epsilon, double sigma, double cutoff,
+                                                    double switch_width, int32_t half_list, float* atomic_energies,
+                                                    float* forces, float* virials, float* system_energies,
+                                                    void* workspace, size_t workspace_bytes, void* stream) {
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
     if (switch_width != 0.0)
@@ -515,6 +533,7 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
     a.sys_acc = nullptr;
     a.n_blocks = 0;
     a.rows_per_block = 0;
+    a.order = half_list ? nullptr : row_order;  // (the half-list kernel walks rows in index order)
     a.sys_first = nullptr;
     a.sys_last = nullptr;
     a.lds_atoms = getenv("NVAMD_LJ_NO_LDS") ? 0 : kLdsAtoms;

@@ -1154,10 +1154,38 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     }
 }
 
+__global__ __launch_bounds__(kBlock) void nl_atom_order_kernel(const float4* __restrict__ sorted_pos,
+                                                               const int32_t* __restrict__ bidx,
+                                                               const uint8_t* __restrict__ flags, int n_atoms,
+                                                               int32_t* __restrict__ order) {
+    int k = blockIdx.x * kBlock + threadIdx.x;
+    if (k >= n_atoms) return;
+    // slot k of the sorted arrays belongs to the system atom k belongs to (both are laid out by batch_ptr)
+    if (flags && !flags[bidx[k]]) return;
+    order[k] = __float_as_int(sorted_pos[k].w);
+}
+
 }  // namespace
 }  // namespace nvamd
 
 using namespace nvamd;
+
+NVAMD_EXPORT int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
+                                         const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                                         int32_t* atom_order, void* stream) {
+    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "atom order: negative size");
+    if (n_atoms == 0 || n_systems == 0) return NVAMD_OK;
+    if (!atom_order || !batch_idx) return fail(NVAMD_ERR_INVALID_ARGUMENT, "atom order: null buffer");
+    size_t need = carve(nullptr, nullptr, n_atoms, n_systems);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "atom order: workspace %zu < %zu bytes", workspace_bytes, need);
+    NlWorkspace ws;
+    carve(&ws, static_cast<char*>(const_cast<void*>(workspace)), n_atoms, n_systems);
+    hipLaunchKernelGGL(nl_atom_order_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), ws.sorted_pos, batch_idx, rebuild_flags, n_atoms, atom_order);
+    NVAMD_LAUNCH_CHECK("atom order launch");
+    return NVAMD_OK;
+}
 
 NVAMD_EXPORT int32_t nvamd_nl_workspace_bytes(int32_t n_atoms, int32_t n_systems, size_t* bytes) {
     if (!bytes || n_atoms < 0 || n_systems < 0)

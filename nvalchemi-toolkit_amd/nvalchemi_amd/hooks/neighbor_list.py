@@ -24,6 +24,7 @@ from enum import Enum
 
 import torch
 
+from .. import _lib
 from .._neighbor_ops import ceil16, estimate_max_neighbors, neighbor_list
 from ..dynamics._ops.neighbor_list_rebuild import batch_neighbor_list_rebuild_inplace
 from ..models.base import NeighborConfig, NeighborListFormat
@@ -127,11 +128,35 @@ class NeighborListHook:
                     self._realloc_k(N, positions.device, pbc)
                     self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
 
+        self._publish_row_order(batch, N, B)
         _write_neighbor_data_to_batch(
             batch=batch, neighbor_matrix=self._neighbor_matrix, num_neighbors=self._num_neighbors,
             neighbor_matrix_shifts=self._neighbor_matrix_shifts,
             format=NeighborListFormat.COO if self._neighbor_list_flag else NeighborListFormat.MATRIX,
             cutoff=self.config.cutoff)
+
+    #: systems larger than this do not fit the pair kernel's LDS stage (csrc/lj_pair.hip kLdsAtoms)
+    _ROW_ORDER_MIN_ATOMS = 4096
+
+    def _publish_row_order(self, batch, N: int, B: int) -> None:
+        """For batches with systems too large for the pair kernel to stage in LDS, leave the
+        atoms' cell order of this build on the batch (``_neighbor_row_order``): a pair kernel that
+        walks its rows in that order gathers neighbor positions from the caches instead of HBM.
+        Not part of the reference; purely a hint (any model may ignore it)."""
+        if N == 0 or batch.max_num_nodes <= self._ROW_ORDER_MIN_ATOMS:
+            if getattr(batch, "_neighbor_row_order", None) is not None:
+                object.__setattr__(batch, "_neighbor_row_order", None)
+            self._atom_order = None
+            return
+        fresh = (getattr(self, "_atom_order", None) is None or self._atom_order.shape[0] != N
+                 or self._atom_order.device != batch.positions.device)
+        if fresh:
+            self._atom_order = torch.empty(N, dtype=torch.int32, device=batch.positions.device)
+        flags = None
+        if not fresh and self.skin > 0.0 and self._ref_positions is not None:
+            flags = self._rebuild_flags  # systems that were not rebuilt keep the order of their last build
+        _lib.nl_atom_order(batch.batch_idx, B, self._atom_order, flags)
+        object.__setattr__(batch, "_neighbor_row_order", self._atom_order)
 
     def _build(self, batch, cutoff, cell, pbc, rebuild_flags) -> None:
         neighbor_list(positions=batch.positions, cutoff=cutoff, cell=cell, pbc=pbc,

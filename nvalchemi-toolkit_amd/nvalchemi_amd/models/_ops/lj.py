@@ -94,10 +94,13 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
                                   neighbor_matrix_shifts: Tensor | None, num_neighbors: Tensor,
                                   batch_idx: Tensor, fill_value: int, epsilon: float, sigma: float,
                                   cutoff: float, switch_width: float, half_list: bool,
-                                  compute_virial: bool = False, out: dict | None = None):
+                                  compute_virial: bool = False, out: dict | None = None,
+                                  row_order: Tensor | None = None):
     """Fused launch: ``(atomic_energies (N), forces (N,3), system_energies (B), virials (B,9) |
     None)``.  ``neighbor_matrix_shifts=None`` means all shifts are zero (no ``(N,K,3)`` zeros
-    tensor is needed).  ``out`` may carry preallocated result tensors under those names."""
+    tensor is needed).  ``out`` may carry preallocated result tensors under those names.
+    ``row_order`` (a permutation of the atoms that keeps every system together, e.g. the cell
+    order of the neighbor build) only changes the order in which rows are worked on."""
     _check_dtype(positions)
     N = positions.shape[0]
     B = cells.shape[0]
@@ -119,5 +122,5 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
             w = torch.empty(B, 9, dtype=dt, device=dev)
     _lib.lj_energy_forces(positions, cells, neighbor_matrix, _shifts_or_none(neighbor_matrix_shifts),
                           num_neighbors, batch_idx, fill_value, epsilon, sigma, cutoff, switch_width,
-                          half_list, e, f, virials=w, system_energies=es)
+                          half_list, e, f, virials=w, system_energies=es, row_order=row_order)
     return e, f, es, w

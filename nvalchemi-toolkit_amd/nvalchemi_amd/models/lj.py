@@ -121,6 +121,16 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             keys.add("stress")
         return keys
 
+    @staticmethod
+    def _row_order_of(data, N: int, device) -> torch.Tensor | None:
+        """The cell order the neighbor hook left on the batch for systems too large to stage
+        in LDS (it keeps the pair kernel's gathers in the caches), if it fits this batch."""
+        order = getattr(data, "_neighbor_row_order", None)
+        if (isinstance(order, torch.Tensor) and order.shape == (N,) and order.dtype == torch.int32
+                and order.device == device and order.is_contiguous()):
+            return order
+        return None
+
     # ------------------------------------------------------------------
     def forward(self, data: AtomicData | Batch, out: dict | None = None, **kwargs: Any) -> OrderedDict:
         """``OrderedDict`` with ``energy (B,1)``, ``forces (N,3)`` and optionally
@@ -155,7 +165,8 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             positions.contiguous(), cells, inp["neighbor_matrix"].contiguous(),
             None if shifts is None else shifts.contiguous(), inp["num_neighbors"].contiguous(),
             inp["batch_idx"].contiguous(), inp["fill_value"], self.epsilon, self.sigma, self.cutoff,
-            self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs)
+            self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs,
+            row_order=self._row_order_of(data, N, positions.device))
         model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
         if virials is not None:
             model_output["virial"] = virials.view(B, 3, 3)

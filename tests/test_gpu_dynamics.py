@@ -302,3 +302,40 @@ def test_one_md_step_replays_from_a_captured_graph():
             assert torch.equal(graphed[key], eager[key]), key
         assert torch.equal(graphed["nn"], eager["nn"])
     assert float(scratch) == float(scratch)
+
+
+def test_hook_leaves_the_cell_order_for_large_systems_and_the_model_uses_it():
+    from nvalchemi_amd.hooks import HookContext
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    rng = np.random.default_rng(3)
+    n_big, n_small, rho = 6000, 300, 0.8
+    P, C, ptr = [], [], [0]
+    for n in (n_small, n_big):
+        L = (n / rho) ** (1 / 3)
+        P.append(rng.uniform(0, L, (n, 3)).astype(np.float32))
+        C.append(np.eye(3, dtype=np.float32) * L)
+        ptr.append(ptr[-1] + n)
+    P, C, ptr = np.concatenate(P), np.stack(C), np.array(ptr, np.int32)
+    N = len(P)
+    pb = np.ones((2, 3), bool)
+    batch = make_batch(P, np.full(N, 18, np.int64), np.ones(N, np.float32), C, pb, ptr)
+    model = LennardJonesModelWrapper(epsilon=1.0, sigma=0.5, cutoff=2.5)
+    hook = model.make_neighbor_hooks()[0]
+    hook(HookContext(batch=batch), None)
+    order = batch._neighbor_row_order
+    assert order is not None and order.dtype == torch.int32 and order.shape == (N,)
+    o = order.cpu().numpy()
+    for s in range(2):  # a permutation of each system's own range
+        assert np.array_equal(np.sort(o[ptr[s]:ptr[s + 1]]), np.arange(ptr[s], ptr[s + 1]))
+    with_order = model(batch)
+    object.__setattr__(batch, "_neighbor_row_order", None)
+    without = model(batch)
+    assert torch.equal(with_order["forces"], without["forces"])
+    assert torch.allclose(with_order["energy"], without["energy"], rtol=1e-6, atol=0)
+    # a batch of small systems gets no order
+    small = make_batch(P[:n_small], np.full(n_small, 18, np.int64), np.ones(n_small, np.float32), C[:1], pb[:1],
+                       np.array([0, n_small], np.int32))
+    hook2 = model.make_neighbor_hooks()[0]
+    hook2(HookContext(batch=small), None)
+    assert getattr(small, "_neighbor_row_order", None) is None

@@ -245,6 +245,19 @@ def test_four_million_atom_single_box():
     assert_symmetric(i, j, S, N)
     eps, sig = 0.01, 1.5  # random positions: keep the repulsive wall short
     e, f, w, es = gpu_lj(pos, cell, nm, sh, nn, bidx, eps, sig, rc, virial=True)
+    # the same with the rows walked in the build's cell order (what the hook arranges for systems
+    # this large): a permutation of the atoms, and identical per-atom results
+    from nvalchemi_amd import _lib
+
+    order = torch.empty(N, dtype=torch.int32, device=DEV)
+    _lib.nl_atom_order(bidx, 1, order)
+    assert torch.equal(order.long().sort().values, torch.arange(N, device=DEV))
+    e2, f2 = torch.empty_like(e), torch.empty_like(f)
+    es2 = torch.empty_like(es)
+    _lib.lj_energy_forces(pos, cell, nm, sh, nn, bidx, N, eps, sig, rc, 0.0, False, e2, f2, None, es2, row_order=order)
+    torch.cuda.synchronize()
+    assert torch.equal(e2, e) and torch.equal(f2, f)
+    assert abs(float(es2[0]) - float(es[0])) <= 1e-6 * abs(float(es[0]))
     e_sys, f64, w_tr = torch_lj_over_edges(pos, cell, bidx, i, j, S, eps, sig, rc, 1)
     del i, j, S
     assert math.isfinite(float(es[0]))

@@ -267,3 +267,34 @@ def test_matrix_to_coo_row_major():
     ii, kk = np.nonzero(np.arange(K)[None, :] < clamped[:, None])
     assert np.array_equal(nl.cpu().numpy(), np.stack([ii, nm[ii, kk]], 1))
     assert np.array_equal(nls.cpu().numpy(), sh[ii, kk])
+
+
+def test_lj_row_order_changes_nothing_but_the_walk():
+    """``row_order`` only permutes the order in which rows are worked on: per-atom outputs are
+    bit-identical, per-system sums equal to rounding (their accumulation order differs)."""
+    from nvalchemi_amd import _lib
+
+    P, C, pb, ptr = periodic_batch(seed=61, n_systems=5, n_lo=200, n_hi=700, density=0.8)
+    rc, K = 2.5, 96
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, rc, K)
+    bi = oracle.batch_idx_from_ptr(ptr)
+    N, B = len(P), len(C)
+    rng = np.random.default_rng(7)
+    # a permutation that keeps every system together and in place (as the build's cell order does),
+    # and one that does not (any permutation must still give the same per-atom results)
+    inside = np.concatenate([ptr[s] + rng.permutation(ptr[s + 1] - ptr[s]) for s in range(B)]).astype(np.int32)
+    anywhere = rng.permutation(N).astype(np.int32)
+    args = (T(P, torch.float32), T(C, torch.float32), T(nm), T(sh), T(nn), T(bi), N, 1.0, 1.0, rc, 0.0, False)
+    res = []
+    for order in (None, inside, anywhere):
+        e = torch.empty(N, device=DEV)
+        f = torch.empty((N, 3), device=DEV)
+        w = torch.empty((B, 9), device=DEV)
+        es = torch.empty(B, device=DEV)
+        _lib.lj_energy_forces(*args, e, f, w, es, row_order=None if order is None else T(order))
+        torch.cuda.synchronize()
+        res.append((e.cpu().numpy(), f.cpu().numpy(), w.cpu().numpy(), es.cpu().numpy()))
+    for e, f, w, es in res[1:]:
+        assert np.array_equal(e, res[0][0]) and np.array_equal(f, res[0][1])
+        assert np.allclose(es, res[0][3], rtol=1e-6, atol=0)
+        assert np.allclose(w, res[0][2], rtol=1e-5, atol=1e-5 * np.abs(res[0][2]).max())
