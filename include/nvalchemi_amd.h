@@ -183,6 +183,23 @@ int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const
                             const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
                             int32_t* atom_order, void* stream);
 
+/* Per-system reductions of a per-atom float32 vector: replace the Warp launches behind
+ * nvalchemi_hooks::segmented_sum / _max / _min / _mean (nvalchemi/dynamics/hooks/_utils.py:58-136;
+ * scatter_reduce_per_graph :172-212).  batch_idx (n) i32 must be sorted.  op: 0 sum, 1 max, 2 min, 3 mean.
+ * out (m) f32; segments without elements give 0 (sum, mean), -inf (max), +inf (min).  Sums are
+ * accumulated in float64 and rounded once. */
+int32_t nvamd_segment_workspace_bytes(int32_t n_segments, size_t* bytes);
+int32_t nvamd_segment_reduce(const float* values, const int32_t* batch_idx, int32_t n_values,
+                             int32_t n_segments, int32_t op, float* out, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/* Kinetic energy per system, 1/2 sum m |v|^2: replaces nvalchemi_hooks::compute_kinetic_energy
+ * (nvalchemi/dynamics/hooks/_utils.py:138-155; kinetic_energy_per_graph :215-243).  Workspace as for
+ * nvamd_segment_reduce. */
+int32_t nvamd_kinetic_energy(const float* velocities, const float* masses, const int32_t* batch_idx,
+                             int32_t n_atoms, int32_t n_systems, float* kinetic_energy, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
 /* Verlet-skin displacement test: replaces the Warp launch behind
  * nvalchemi::_batch_neighbor_list_rebuild_inplace (nvalchemi/dynamics/_ops/neighbor_list_rebuild.py:37-139,
  * called at nvalchemi/hooks/neighbor_list.py:295-311).  rebuild_flags (M) bool is cleared, then set for

@@ -42,6 +42,9 @@ _SIGNATURES = {
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_lj_energy_forces_ordered": (_i32, [_vp] * 7 + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_nl_atom_order": (_i32, [_vp, _c.c_size_t, _vp, _vp, _i32, _i32, _vp, _vp]),
+    "nvamd_segment_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_segment_reduce": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_kinetic_energy": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
 }
@@ -322,3 +325,28 @@ def wrap_positions(positions, cell, pbc, batch_idx) -> None:
         _dev(positions, "positions", torch.float32, (N, 3)), _dev(cell, "cell", torch.float32, (M, 3, 3)),
         _dev(_as_u8(pbc), "pbc", torch.uint8, (M, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         N, M, _stream(positions.device)), "nvamd_wrap_positions")
+
+
+SEGMENT_OPS = {"sum": 0, "amax": 1, "amin": 2, "mean": 3}
+
+
+def segment_reduce(values, batch_idx, out, op: str) -> None:
+    lib = library()
+    n = values.shape[0]
+    m = out.shape[0]
+    ws = workspaces.get(values.device, "segment", _size(lib.nvamd_segment_workspace_bytes, m))
+    _check(lib.nvamd_segment_reduce(
+        _dev(values, "values", torch.float32, (n,)), _dev(batch_idx, "batch_idx", torch.int32, (n,)),
+        n, m, SEGMENT_OPS[op], _dev(out, "out", torch.float32, (m,)), ws.data_ptr(), ws.numel(),
+        _stream(values.device)), "nvamd_segment_reduce")
+
+
+def kinetic_energy(velocities, masses, batch_idx, out) -> None:
+    lib = library()
+    n = velocities.shape[0]
+    m = out.shape[0]
+    ws = workspaces.get(velocities.device, "segment", _size(lib.nvamd_segment_workspace_bytes, m))
+    _check(lib.nvamd_kinetic_energy(
+        _dev(velocities, "velocities", torch.float32, (n, 3)), _dev(masses, "masses", torch.float32, (n,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (n,)), n, m, _dev(out, "kinetic_energy", torch.float32, (m,)),
+        ws.data_ptr(), ws.numel(), _stream(velocities.device)), "nvamd_kinetic_energy")

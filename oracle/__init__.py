@@ -260,3 +260,35 @@ def wrap_positions(positions, cell, pbc, batch_idx) -> np.ndarray:
     lib().orc_wrap_positions(_p(pos, _f32p), _p(_f32(cell).reshape(-1, 9), _f32p),
                              _p(_u8(pbc).reshape(-1, 3), _u8p), _p(_i32(batch_idx), _i32p), pos.shape[0])
     return pos
+
+
+def segment_reduce(values, batch_idx, n_segments: int, op: str) -> np.ndarray:
+    """Per-segment ``sum`` / ``amax`` / ``amin`` / ``mean`` of a float32 vector (numpy restatement of
+    nvalchemi/dynamics/hooks/_utils.py:58-136: sums in float64, rounded once; empty segments give
+    0, -inf, +inf, 0)."""
+    v = _f32(values)
+    idx = _i32(batch_idx)
+    m = int(n_segments)
+    if op == "amax":
+        out = np.full(m, -np.inf, dtype=np.float32)
+        np.maximum.at(out, idx, v)
+        return out
+    if op == "amin":
+        out = np.full(m, np.inf, dtype=np.float32)
+        np.minimum.at(out, idx, v)
+        return out
+    acc = np.zeros(m, dtype=np.float64)
+    np.add.at(acc, idx, v.astype(np.float64))
+    if op == "sum":
+        return acc.astype(np.float32)
+    cnt = np.bincount(idx, minlength=m).astype(np.float64)
+    return np.where(cnt > 0, acc / np.maximum(cnt, 1), 0.0).astype(np.float32)
+
+
+def kinetic_energy(velocities, masses, batch_idx, n_systems: int) -> np.ndarray:
+    """``0.5 sum m |v|^2`` per system (nvalchemi/dynamics/hooks/_utils.py:215-243), float64 sum, rounded once."""
+    v = _f32(velocities).astype(np.float64)
+    per_atom = 0.5 * _f32(masses).astype(np.float64) * ((v[:, 0] * v[:, 0] + v[:, 1] * v[:, 1]) + v[:, 2] * v[:, 2])
+    acc = np.zeros(int(n_systems), dtype=np.float64)
+    np.add.at(acc, _i32(batch_idx), per_atom)
+    return acc.astype(np.float32)

@@ -298,3 +298,32 @@ def test_lj_row_order_changes_nothing_but_the_walk():
         assert np.array_equal(e, res[0][0]) and np.array_equal(f, res[0][1])
         assert np.allclose(es, res[0][3], rtol=1e-6, atol=0)
         assert np.allclose(w, res[0][2], rtol=1e-5, atol=1e-5 * np.abs(res[0][2]).max())
+
+
+def test_segmented_observables_match_oracle():
+    from nvalchemi_amd.dynamics.hooks import (KB_EV, kinetic_energy_per_graph, scatter_reduce_per_graph,
+                                              temperature_per_graph)
+
+    rng = np.random.default_rng(8)
+    counts = [0, 5, 1, 300, 0, 64, 65, 2000, 0]  # empty systems, wave-sized and longer runs
+    B = len(counts)
+    idx = np.repeat(np.arange(B), counts).astype(np.int32)
+    N = len(idx)
+    vals = rng.normal(0, 3, N).astype(np.float32)
+    for op in ("sum", "amax", "amin", "mean"):
+        got = scatter_reduce_per_graph(T(vals), T(idx), B, reduce=op).cpu().numpy()
+        want = oracle.segment_reduce(vals, idx, B, op)
+        if op in ("amax", "amin"):
+            assert np.array_equal(got, want), op
+        else:
+            assert np.allclose(got, want, rtol=1e-6, atol=1e-6), op
+    vel = rng.normal(0, 0.1, (N, 3)).astype(np.float32)
+    mass = rng.uniform(1, 60, N).astype(np.float32)
+    ke = kinetic_energy_per_graph(T(vel), T(mass).unsqueeze(-1), T(idx), B)
+    assert ke.shape == (B, 1)
+    want = oracle.kinetic_energy(vel, mass, idx, B)
+    assert np.allclose(ke.cpu().numpy().ravel(), want, rtol=1e-6, atol=0)
+    n_at = torch.tensor(counts, device=DEV)
+    temp = temperature_per_graph(T(vel), T(mass), T(idx), B, n_at).cpu().numpy()
+    ok = np.array(counts) > 0
+    assert np.allclose(temp[ok], 2 * want[ok] / (3 * np.array(counts)[ok] * KB_EV), rtol=2e-6)

@@ -143,3 +143,21 @@ def test_fmax_is_max_atom_force_norm_per_system():
     F = np.array([[3, 4, 0], [0, 0, 1], [0, 0, 0], [1, 2, 2]], dtype=np.float32)
     out = oracle.fmax(F, [0, 0, 2, 2], 3)
     assert out[0] == 5 and out[1] == -np.inf and out[2] == 3
+
+
+def test_segment_reductions_and_kinetic_energy_literals():
+    """The per-system observables of nvalchemi/dynamics/hooks/_utils.py:172-290 on cases small enough
+    to check by hand, including an empty system."""
+    v = np.array([1.0, -2.0, 3.0, 0.5, 4.0], np.float32)
+    idx = np.array([0, 0, 0, 2, 2], np.int32)
+    assert oracle.segment_reduce(v, idx, 3, "sum").tolist() == [2.0, 0.0, 4.5]
+    assert oracle.segment_reduce(v, idx, 3, "amax").tolist() == [3.0, -np.inf, 4.0]
+    assert oracle.segment_reduce(v, idx, 3, "amin").tolist() == [-2.0, np.inf, 0.5]
+    assert np.allclose(oracle.segment_reduce(v, idx, 3, "mean"), [2.0 / 3.0, 0.0, 2.25])
+    vel = np.array([[1, 2, 2], [0, 3, 4], [1, 0, 0]], np.float32)
+    m = np.array([2.0, 1.0, 4.0], np.float32)
+    assert oracle.kinetic_energy(vel, m, np.array([0, 0, 1], np.int32), 3).tolist() == [9.0 + 12.5, 2.0, 0.0]
+    # T = 2 KE / (3 N kB): one atom of mass m and speed v has T = m v^2 / (3 kB)
+    kb = 8.617333262e-5
+    ke = oracle.kinetic_energy(np.array([[0.1, 0, 0]], np.float32), np.array([12.0], np.float32), [0], 1)[0]
+    assert abs(2 * ke / (3 * 1 * kb) - 12.0 * 0.01 / (3 * kb)) < 1e-3
