@@ -159,21 +159,26 @@ int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces
 int32_t nvamd_segment_fmax(const float* forces, const int32_t* batch_idx, int32_t n_atoms,
                            int32_t n_systems, float* fmax, void* stream);
 
-/* The same, walking the rows in a given order: row_order (N) i32 is a permutation of 0..N-1 in which
- * the atoms of each system stay together and in system order (e.g. the cell order of the last neighbor
- * build, nvamd_nl_atom_order), or null.  Results do not depend on it; for systems too large to stage in
- * LDS, an order with spatial locality keeps the gathers of neighbor positions in the caches.  No
- * counterpart in the reference. */
-int32_t nvamd_lj_energy_forces_ordered(const float* positions, const float* cells,
-                                       const int32_t* neighbor_matrix,
-                                       const int32_t* neighbor_matrix_shifts,
-                                       const int32_t* num_neighbors, const int32_t* batch_idx,
-                                       const int32_t* row_order, int32_t n_atoms, int32_t max_neighbors,
-                                       int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
-                                       double cutoff, double switch_width, int32_t half_list,
-                                       float* atomic_energies, float* forces, float* virials,
-                                       float* system_energies, void* workspace, size_t workspace_bytes,
-                                       void* stream);
+/* The same, with two optional hints; results do not depend on either.  No counterpart in the reference.
+ * row_order (N) i32 or null: a permutation of 0..N-1 in which the atoms of each system stay together and in
+ *   system order (e.g. the cell order of the last neighbor build, nvamd_nl_atom_order); the kernel walks its
+ *   rows in it.  For systems too large to stage in LDS, an order with spatial locality keeps the gathers of
+ *   neighbor positions in the caches.
+ * neighbor_list_cutoff: the cutoff (skin included) that the neighbor matrix was built with, or 0 if unknown.
+ *   Every listed pair is then closer than that; in a system whose cell has all three perpendicular widths
+ *   above twice it, no pair has two listed images, the listed image is the nearest one, and the kernel
+ *   derives the shift from the positions instead of reading neighbor_matrix_shifts (12 of the 16 bytes per
+ *   pair).  A matrix that holds pairs beyond this cutoff makes the results wrong: pass 0 when in doubt. */
+int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells,
+                                      const int32_t* neighbor_matrix,
+                                      const int32_t* neighbor_matrix_shifts,
+                                      const int32_t* num_neighbors, const int32_t* batch_idx,
+                                      const int32_t* row_order, double neighbor_list_cutoff, int32_t n_atoms,
+                                      int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
+                                      double epsilon, double sigma, double cutoff, double switch_width,
+                                      int32_t half_list, float* atomic_energies, float* forces, float* virials,
+                                      float* system_energies, void* workspace, size_t workspace_bytes,
+                                      void* stream);
 
 /* Atom indices in the cell order of the neighbor build that last used this workspace with the same
  * n_atoms / n_systems: atom_order[k] for k in a system's range [batch_ptr[s], batch_ptr[s+1]) are that

@@ -43,6 +43,7 @@ struct LjArgs {
     const int32_t* sys_first;  // (B) first atom of each non-empty system
     const int32_t* sys_last;   // (B) one past its last atom
     int lds_atoms;             // stage positions in LDS when the systems of a run have at most this many atoms
+    double list_rc;            // cutoff the neighbor list was built with (0: unknown, shifts are always read)
 };
 
 template <int LPR>
@@ -78,11 +79,21 @@ __device__ __forceinline__ double reciprocal(double x) {
     return y;
 }
 
-template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC>
+// IMG: the shifts are not read.  Every pair of the list is closer than half of every
+// perpendicular width of its cell, so the listed image is the nearest one and its shift is
+// -rint((r_j - r_i) . H^-1) (float32 is ample: the listed image's fractional components stay
+// below 0.49995 in magnitude).
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC, bool IMG>
 __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, int sys_base,
                                         const float* __restrict__ s_pos, int span0, int span_n,
-                                        const double (*s_shift)[3], int table_sys,
+                                        const double (*s_shift)[3], int table_sys, const float* s_hinv,
                                         double (*s_acc)[VIRIAL ? 7 : 1]) {
+    float hi[9];
+    if (IMG) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k)
+            hi[k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_hinv[k])));
+    }
     constexpr int G = kBlockFull / LPR;
     const int g = threadIdx.x / LPR;
     const int sub = threadIdx.x % LPR;
@@ -119,7 +130,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                     const int kq = kv < last_quad ? kv : last_quad;  // never past the row's last used quad
                     const int4 j4 = *reinterpret_cast<const int4*>(row + kq);
                     jj[4 * v + 0] = j4.x; jj[4 * v + 1] = j4.y; jj[4 * v + 2] = j4.z; jj[4 * v + 3] = j4.w;
-                    if (SHIFTS) {
+                    if (SHIFTS && !IMG) {
                         const int4* sp = reinterpret_cast<const int4*>(srow + 3 * kq);
                         const int4 sa = sp[0], sb = sp[1], sc = sp[2];
                         s0[4 * v + 0] = sa.x; s1[4 * v + 0] = sa.y; s2[4 * v + 0] = sa.z;
@@ -128,7 +139,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                         s0[4 * v + 3] = sc.y; s1[4 * v + 3] = sc.z; s2[4 * v + 3] = sc.w;
                     }
                 }
-                if (!SHIFTS) {
+                if (!SHIFTS || IMG) {
 #pragma unroll
                     for (int u = 0; u < UNROLL; ++u) s0[u] = s1[u] = s2[u] = 0;
                 }
@@ -143,7 +154,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 const int kq = k < cnt ? k : cnt - 1;
                 jj[u] = row[kq];
                 s0[u] = s1[u] = s2[u] = 0;
-                if (SHIFTS) {
+                if (SHIFTS && !IMG) {
                     s0[u] = srow[3 * kq + 0];
                     s1[u] = srow[3 * kq + 1];
                     s2[u] = srow[3 * kq + 2];
@@ -171,6 +182,12 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 double t0 = 0.0, t1 = 0.0, t2 = 0.0;
+                if (IMG) {
+                    const float dx = xj[u] - xi, dy = yj[u] - yi, dz = zj[u] - zi;
+                    s0[u] = -(int)__builtin_rintf(dx * hi[0] + dy * hi[3] + dz * hi[6]);
+                    s1[u] = -(int)__builtin_rintf(dx * hi[1] + dy * hi[4] + dz * hi[7]);
+                    s2[u] = -(int)__builtin_rintf(dx * hi[2] + dy * hi[5] + dz * hi[8]);
+                }
                 if (SHIFTS) {
                     const unsigned c0 = (unsigned)(s0[u] + 1), c1 = (unsigned)(s1[u] + 1), c2 = (unsigned)(s2[u] + 1);
                     if (tabled && c0 < 3u && c1 < 3u && c2 < 3u) {
@@ -255,6 +272,8 @@ __global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_matrix_kernel(L
     __shared__ double s_acc[kSysSlots][NV];
     __shared__ float s_pos[3 * kLdsAtoms];
     __shared__ double s_shift[27][3];  // shift . cell of the system in hand, shifts -1..1 per axis
+    __shared__ float s_hinv[9];        // its inverse cell
+    __shared__ int s_img;              // its pairs' shifts follow from the positions alone
 
     // a workgroup owns rows_per_block consecutive rows; workgroups are numbered so that each
     // XCD walks one contiguous eighth of the atoms
@@ -288,11 +307,44 @@ __global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_matrix_kernel(L
             shift_vector(a.cells + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
                          s_shift[t][2]);
         }
+        if (SHIFTS && threadIdx.x == 32) {
+            // shifts need not be read when the list's cutoff is below half of every perpendicular
+            // width of the cell (1 / |column of the inverse|): then no pair has two listed images
+            int ok = 0;
+            if (a.list_rc > 0.0) {
+                const float* c = a.cells + 9 * (size_t)sys;
+                double h[9], hv[9];
+                for (int k = 0; k < 9; ++k) h[k] = (double)c[k];
+                inv3(h, hv);  // (a singular cell gives infinities or NaNs: they fail the test below)
+                {
+                    ok = 1;
+                    const double lim = 1.0 / (2.0002 * a.list_rc);  // |column| must stay below this
+                    for (int k = 0; k < 3; ++k) {
+                        const double n2 = hv[k] * hv[k] + hv[3 + k] * hv[3 + k] + hv[6 + k] * hv[6 + k];
+                        if (!(n2 < lim * lim)) ok = 0;
+                    }
+                    for (int k = 0; k < 9; ++k) s_hinv[k] = (float)hv[k];
+                }
+            }
+            s_img = ok;
+        }
         __syncthreads();
-        if (staged)
-            lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift, sys, s_acc);
-        else
-            lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys, s_acc);
+        const bool img = SHIFTS && s_img != 0;
+        if (staged) {
+            if (img)
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, SHIFTS>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
+                                                                     sys, s_hinv, s_acc);
+            else
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, false>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
+                                                                    sys, s_hinv, s_acc);
+        } else {
+            if (img)
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, SHIFTS>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
+                                                                      s_hinv, s_acc);
+            else
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, false>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
+                                                                     s_hinv, s_acc);
+        }
         r = seg_end;
         if (r < row_end) __syncthreads();  // the stage is about to be overwritten
     }
@@ -480,17 +532,18 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
                                             int32_t half_list, float* atomic_energies, float* forces,
                                             float* virials, float* system_energies, void* workspace,
                                             size_t workspace_bytes, void* stream) {
-    return nvamd_lj_energy_forces_ordered(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
-                                          batch_idx, nullptr, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
-                                          sigma, cutoff, switch_width, half_list, atomic_energies, forces, virials,
-                                          system_energies, workspace, workspace_bytes, stream);
+    return nvamd_lj_energy_forces_hinted(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
+                                         batch_idx, nullptr, 0.0, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
+                                         sigma, cutoff, switch_width, half_list, atomic_energies, forces, virials,
+                                         system_energies, workspace, workspace_bytes, stream);
 }
 
-NVAMD_EXPORT int32_t nvamd_lj_energy_forces_ordered(const float* positions, const float* cells,
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells,
                                                     const int32_t* neighbor_matrix,
                                                     const int32_t* neighbor_matrix_shifts,
                                                     const int32_t* num_neighbors, const int32_t* batch_idx,
-                                                    const int32_t* row_order, int32_t n_atoms,
+                                                    const int32_t* row_order, double neighbor_list_cutoff,
+                                                    int32_t n_atoms,
                                                     int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
                                                     double epsilon, double sigma, double cutoff,
                                                     double switch_width, int32_t half_list, float* atomic_energies,
@@ -537,6 +590,11 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_ordered(const float* positions, cons
     a.sys_first = nullptr;
     a.sys_last = nullptr;
     a.lds_atoms = getenv("NVAMD_LJ_NO_LDS") ? 0 : kLdsAtoms;
+    // (a list built with a smaller cutoff than the potential's would be the caller's mistake:
+    // the larger of the two is the safe bound)
+    a.list_rc = (neighbor_list_cutoff > 0.0 && !half_list && !getenv("NVAMD_LJ_READ_SHIFTS"))
+                    ? (neighbor_list_cutoff > cutoff ? neighbor_list_cutoff : cutoff)
+                    : 0.0;
     const bool shifts = neighbor_matrix_shifts != nullptr;
     char* w = static_cast<char*>(workspace);
     const size_t nsys = (size_t)(n_systems > 0 ? n_systems : 1);

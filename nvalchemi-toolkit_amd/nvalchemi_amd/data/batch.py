@@ -123,7 +123,7 @@ class _Storage:
 
 
 _GROUP_ORDER = ("atoms", "edges", "system")
-_RESERVED = {"_storage", "device", "_neighbor_list_cutoff", "_neighbor_row_order"}
+_RESERVED = {"_storage", "device", "_neighbor_list_cutoff", "_neighbor_row_order", "_neighbor_search_cutoff"}
 
 
 class Batch:

@@ -133,7 +133,7 @@ class NeighborListHook:
             batch=batch, neighbor_matrix=self._neighbor_matrix, num_neighbors=self._num_neighbors,
             neighbor_matrix_shifts=self._neighbor_matrix_shifts,
             format=NeighborListFormat.COO if self._neighbor_list_flag else NeighborListFormat.MATRIX,
-            cutoff=self.config.cutoff)
+            cutoff=self.config.cutoff, search_cutoff=None if self.config.half_list else cutoff)
 
     #: systems larger than this do not fit the pair kernel's LDS stage (csrc/lj_pair.hip kLdsAtoms)
     _ROW_ORDER_MIN_ATOMS = 4096

@@ -95,12 +95,15 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
                                   batch_idx: Tensor, fill_value: int, epsilon: float, sigma: float,
                                   cutoff: float, switch_width: float, half_list: bool,
                                   compute_virial: bool = False, out: dict | None = None,
-                                  row_order: Tensor | None = None):
+                                  row_order: Tensor | None = None, neighbor_list_cutoff: float = 0.0):
     """Fused launch: ``(atomic_energies (N), forces (N,3), system_energies (B), virials (B,9) |
     None)``.  ``neighbor_matrix_shifts=None`` means all shifts are zero (no ``(N,K,3)`` zeros
     tensor is needed).  ``out`` may carry preallocated result tensors under those names.
     ``row_order`` (a permutation of the atoms that keeps every system together, e.g. the cell
-    order of the neighbor build) only changes the order in which rows are worked on."""
+    order of the neighbor build) only changes the order in which rows are worked on.
+    ``neighbor_list_cutoff`` (the radius the matrix was searched with, 0.0 if unknown) lets the
+    kernel derive shifts from positions, instead of reading them, in systems whose cell is wider
+    than twice that radius in every direction; the results are the same."""
     _check_dtype(positions)
     N = positions.shape[0]
     B = cells.shape[0]
@@ -122,5 +125,6 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
             w = torch.empty(B, 9, dtype=dt, device=dev)
     _lib.lj_energy_forces(positions, cells, neighbor_matrix, _shifts_or_none(neighbor_matrix_shifts),
                           num_neighbors, batch_idx, fill_value, epsilon, sigma, cutoff, switch_width,
-                          half_list, e, f, virials=w, system_energies=es, row_order=row_order)
+                          half_list, e, f, virials=w, system_energies=es, row_order=row_order,
+                          neighbor_list_cutoff=neighbor_list_cutoff)
     return e, f, es, w

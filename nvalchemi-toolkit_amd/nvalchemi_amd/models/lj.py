@@ -131,6 +131,16 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             return order
         return None
 
+    @staticmethod
+    def _search_cutoff_of(data, neighbor_matrix: torch.Tensor) -> float:
+        """The radius the neighbor matrix in hand was searched with, if the builder left it on the
+        batch for exactly this tensor; 0.0 (unknown) otherwise."""
+        stamp = getattr(data, "_neighbor_search_cutoff", None)
+        if (isinstance(stamp, tuple) and len(stamp) == 3 and stamp[1] == neighbor_matrix.data_ptr()
+                and stamp[2] == tuple(neighbor_matrix.shape)):
+            return float(stamp[0])
+        return 0.0
+
     # ------------------------------------------------------------------
     def forward(self, data: AtomicData | Batch, out: dict | None = None, **kwargs: Any) -> OrderedDict:
         """``OrderedDict`` with ``energy (B,1)``, ``forces (N,3)`` and optionally
@@ -161,12 +171,14 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             if (isinstance(e_out, torch.Tensor) and e_out.numel() == B and e_out.dtype == positions.dtype
                     and e_out.is_contiguous() and e_out.device == positions.device):
                 bufs["system_energies"] = e_out.view(B)
+        neighbor_matrix = inp["neighbor_matrix"].contiguous()
         _, forces, sys_e, virials = lj_energy_forces_system_batch(
-            positions.contiguous(), cells, inp["neighbor_matrix"].contiguous(),
+            positions.contiguous(), cells, neighbor_matrix,
             None if shifts is None else shifts.contiguous(), inp["num_neighbors"].contiguous(),
             inp["batch_idx"].contiguous(), inp["fill_value"], self.epsilon, self.sigma, self.cutoff,
             self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs,
-            row_order=self._row_order_of(data, N, positions.device))
+            row_order=self._row_order_of(data, N, positions.device),
+            neighbor_list_cutoff=self._search_cutoff_of(data, neighbor_matrix))
         model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
         if virials is not None:
             model_output["virial"] = virials.view(B, 3, 3)

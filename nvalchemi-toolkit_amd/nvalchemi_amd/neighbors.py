@@ -20,9 +20,14 @@ __all__ = ["compute_neighbors"]
 
 def _write_neighbor_data_to_batch(batch: Batch, neighbor_matrix: torch.Tensor, num_neighbors: torch.Tensor,
                                   neighbor_matrix_shifts: torch.Tensor | None,
-                                  format: NeighborListFormat, cutoff: float) -> None:
+                                  format: NeighborListFormat, cutoff: float,
+                                  search_cutoff: float | None = None) -> None:
     """Publish neighbor data on *batch* (MATRIX: three atom keys; COO: a new edges group
-    with per-graph edge counts) and stamp the cutoff."""
+    with per-graph edge counts) and stamp the cutoff.  ``search_cutoff`` is the radius the
+    matrix was actually searched with (cutoff plus skin, a full list); it is kept on the batch
+    together with the identity of the matrix so that a pair kernel may derive shifts from
+    positions where the cell is wide enough."""
+    object.__setattr__(batch, "_neighbor_search_cutoff", None)
     if format == NeighborListFormat.COO:
         coo = get_neighbor_list_from_neighbor_matrix(neighbor_matrix, num_neighbors,
                                                      neighbor_matrix_shifts, fill_value=batch.num_nodes)
@@ -48,6 +53,9 @@ def _write_neighbor_data_to_batch(batch: Batch, neighbor_matrix: torch.Tensor, n
         atoms["num_neighbors"] = num_neighbors
         if neighbor_matrix_shifts is not None:
             atoms["neighbor_matrix_shifts"] = neighbor_matrix_shifts
+        if search_cutoff is not None:
+            object.__setattr__(batch, "_neighbor_search_cutoff",
+                               (float(search_cutoff), neighbor_matrix.data_ptr(), tuple(neighbor_matrix.shape)))
     batch._neighbor_list_cutoff = cutoff
 
 
@@ -104,4 +112,5 @@ def compute_neighbors(batch: Batch, cutoff: float | None = None, *, config: Neig
             break
         max_neighbors = int(actual_max * 1.5) + 1
 
-    _write_neighbor_data_to_batch(batch, nb_matrix, nb_counts, nb_shifts, format, cutoff)
+    _write_neighbor_data_to_batch(batch, nb_matrix, nb_counts, nb_shifts, format, cutoff,
+                                  search_cutoff=None if half_list else cutoff)

@@ -300,6 +300,69 @@ def test_lj_row_order_changes_nothing_but_the_walk():
         assert np.allclose(w, res[0][2], rtol=1e-5, atol=1e-5 * np.abs(res[0][2]).max())
 
 
+@pytest.mark.parametrize("name,kw,rc_list,rc", [
+    ("wide orthorhombic", dict(n_systems=4, n_lo=300, n_hi=900, density=0.8), 2.5, 2.5),
+    ("wide, list with a skin", dict(n_systems=4, n_lo=300, n_hi=900, density=0.8), 3.0, 2.5),
+    ("wide triclinic", dict(n_systems=4, n_lo=500, n_hi=900, density=0.6, triclinic=True), 2.2, 2.2),
+    ("unwrapped positions", dict(n_systems=3, n_lo=300, n_hi=600, density=0.7, spread=2.5), 2.5, 2.5),
+    ("slab", dict(n_systems=3, n_lo=300, n_hi=600, density=0.7, pbc=[True, True, False]), 2.5, 2.5),
+    # cells narrower than twice the list cutoff: several images of a pair are listed, shifts must be read
+    ("narrow", dict(n_systems=4, n_lo=20, n_hi=60, density=0.8), 2.5, 2.5),
+    # some systems wide, some narrow, and some between twice the cutoff and twice the list cutoff
+    ("mixed", dict(n_systems=9, n_lo=30, n_hi=700, density=0.8), 3.2, 2.5),
+])
+def test_lj_shifts_derived_from_positions(name, kw, rc_list, rc):
+    """With the list's cutoff given, the kernel derives shifts from positions wherever the cell is
+    wide enough and reads them elsewhere: per-atom results are bit-identical to reading them
+    everywhere, and the stored shifts are not consulted in wide cells (garbage there changes nothing)."""
+    from nvalchemi_amd import _lib
+
+    P, C, pb, ptr = periodic_batch(seed=67, **kw)
+    K = 160
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, rc_list, K)
+    assert nn.max() <= K
+    bi = oracle.batch_idx_from_ptr(ptr)
+    N, B = len(P), len(C)
+    # perpendicular widths decide which systems qualify (the kernel's own test, restated)
+    hinv = np.linalg.inv(C.astype(np.float64))
+    widths = 1.0 / np.linalg.norm(hinv, axis=1)  # (B, 3): 1 / |column k of the inverse|
+    wide = (widths > 2.0002 * rc_list).all(axis=1)
+    if name in ("narrow",):
+        assert not wide.any()
+    elif name == "mixed":
+        assert wide.any() and (~wide).any()
+    else:
+        assert wide.all()
+
+    def run(shifts, hint):
+        e = torch.empty(N, device=DEV)
+        f = torch.empty((N, 3), device=DEV)
+        w = torch.empty((B, 9), device=DEV)
+        es = torch.empty(B, device=DEV)
+        _lib.lj_energy_forces(T(P, torch.float32), T(C, torch.float32), T(nm), T(shifts), T(nn), T(bi), N, 1.0, 1.0,
+                              rc, 0.0, False, e, f, w, es, neighbor_list_cutoff=hint)
+        torch.cuda.synchronize()
+        return e.cpu().numpy(), f.cpu().numpy(), w.cpu().numpy(), es.cpu().numpy()
+
+    read = run(sh, 0.0)
+    derived = run(sh, rc_list)
+    for a, b in zip(read, derived):
+        assert np.array_equal(a, b), name
+    # oracle parity of the derived path
+    ref = oracle.lj_matrix(P, C, nm, sh, nn, bi, N, 1.0, 1.0, rc, virial=True)
+    assert_close({"atomic_energies": derived[0], "forces": derived[1], "virials": derived[2], "energy": derived[3]},
+                 ref, name)
+    # shifts of wide systems scrambled: the derived path must not notice
+    junk = sh.copy()
+    rows = wide[bi]
+    junk[rows] = 7
+    scrambled = run(junk, rc_list)
+    for a, b in zip(read, scrambled):
+        assert np.array_equal(a, b), name
+    if wide.any():
+        assert not np.array_equal(run(junk, 0.0)[1], read[1])  # (the test has teeth: read, they matter)
+
+
 def test_segmented_observables_match_oracle():
     from nvalchemi_amd.dynamics.hooks import (KB_EV, kinetic_energy_per_graph, scatter_reduce_per_graph,
                                               temperature_per_graph)
