@@ -101,7 +101,10 @@ int32_t nvamd_nl_matrix_to_coo(const int32_t* neighbor_matrix,
  *   atomic_energies (N) f32, forces (N,3) f32: overwritten.
  *   virials (B,9) f32 or NULL: W = -sum r_ij (x) F_ij, row-major, overwritten.
  *   system_energies (B) f32 or NULL: fp64 sum of the float32 atomic energies, overwritten.
- *   switch_width must be 0 (the C2 switching function is not implemented).
+ *   switch_width in [0, cutoff]: 0 is plain truncation; otherwise the pair energy is multiplied by
+ *     S(t) = 1 - t^3 (10 - 15 t + 6 t^2), t = (r - (cutoff - switch_width)) / switch_width, between
+ *     cutoff - switch_width and cutoff (the least-degree polynomial that keeps energy, force and force
+ *     gradient continuous; the reference's own polynomial is inside its absent kernel library).
  *   workspace: nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list); always required.
  * ---------------------------------------------------------------------------------------- */
 int32_t nvamd_lj_workspace_bytes(int32_t n_atoms, int32_t n_systems, int32_t half_list,

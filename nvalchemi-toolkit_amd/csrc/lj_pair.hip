@@ -44,7 +44,23 @@ struct LjArgs {
     const int32_t* sys_last;   // (B) one past its last atom
     int lds_atoms;             // stage positions in LDS when the systems of a run have at most this many atoms
     double list_rc;            // cutoff the neighbor list was built with (0: unknown, shifts are always read)
+    double r_on, inv_sw;       // switching region [r_on, cutoff] and 1 / its width (0, 0: no switching)
 };
+
+// Switching between r_on and the cutoff: u(r) S(t), t = (r - r_on) / width,
+// S = 1 - t^3 (10 - 15 t + 6 t^2): the polynomial of least degree with S(0) = 1, S(1) = 0 and
+// vanishing first and second derivatives at both ends (energy, force and force gradient stay
+// continuous).  On entry u is the pair energy and gg = u'(r) / r; both are replaced.
+__device__ __forceinline__ void apply_switch(const LjArgs& a, double r2, double& u, double& gg) {
+    const double r = __builtin_sqrt(r2);
+    if (!(r > a.r_on)) return;
+    const double t = (r - a.r_on) * a.inv_sw;
+    const double omt = 1.0 - t;
+    const double S = 1.0 - t * t * t * (10.0 - 15.0 * t + 6.0 * t * t);
+    const double dS = -30.0 * t * t * omt * omt * a.inv_sw;
+    gg = gg * S + u * dS / r;
+    u = u * S;
+}
 
 template <int LPR>
 __device__ __forceinline__ double group_sum(double v) {
@@ -83,7 +99,7 @@ __device__ __forceinline__ double reciprocal(double x) {
 // perpendicular width of its cell, so the listed image is the nearest one and its shift is
 // -rint((r_j - r_i) . H^-1) (float32 is ample: the listed image's fractional components stay
 // below 0.49995 in magnitude).
-template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC, bool IMG>
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC, bool IMG, bool SWITCH>
 __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, int sys_base,
                                         const float* __restrict__ s_pos, int span0, int span_n,
                                         const double (*s_shift)[3], int table_sys, const float* s_hinv,
@@ -206,8 +222,10 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 double q2 = a.sig2 * ir2;
                 double q6 = q2 * q2 * q2;
                 double q12 = q6 * q6;
-                e += 0.5 * (a.c4eps * (q12 - q6));
+                double uu = a.c4eps * (q12 - q6);
                 double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
+                if (SWITCH) apply_switch(a, r2, uu, gg);
+                e += 0.5 * uu;
                 fx += gg * d0;
                 fy += gg * d1;
                 fz += gg * d2;
@@ -265,9 +283,9 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
     }
 }
 
-template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool VEC>
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool VEC, bool SWITCH>
 // (six waves per SIMD: three workgroups per CU; the virial variant needs more registers than that leaves)
-__global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_matrix_kernel(LjArgs a) {
+__global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_matrix_kernel(LjArgs a) {
     constexpr int NV = VIRIAL ? 7 : 1;
     __shared__ double s_acc[kSysSlots][NV];
     __shared__ float s_pos[3 * kLdsAtoms];
@@ -332,17 +350,17 @@ __global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_matrix_kernel(L
         const bool img = SHIFTS && s_img != 0;
         if (staged) {
             if (img)
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, SHIFTS>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, SHIFTS, SWITCH>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
                                                                      sys, s_hinv, s_acc);
             else
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, false>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, false, SWITCH>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
                                                                     sys, s_hinv, s_acc);
         } else {
             if (img)
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, SHIFTS>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, SHIFTS, SWITCH>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
                                                                       s_hinv, s_acc);
             else
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, false>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
+                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, false, SWITCH>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
                                                                      s_hinv, s_acc);
         }
         r = seg_end;
@@ -400,6 +418,7 @@ __global__ __launch_bounds__(kBlock) void lj_half_kernel(LjHalfArgs p) {
         double q2 = a.sig2 * ir2, q6 = q2 * q2 * q2, q12 = q6 * q6;
         double u = a.c4eps * (q12 - q6);
         double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;
+        if (a.inv_sw > 0.0) apply_switch(a, r2, u, gg);
         e += 0.5 * u;
         fx += gg * d[0]; fy += gg * d[1]; fz += gg * d[2];
         double* aj = p.atom_acc + 4 * (size_t)j;
@@ -480,11 +499,16 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
     dim3 grid(per * 8), blk(kBlockFull);
     // 16-byte row loads need aligned rows: K a multiple of 4 and aligned base pointers
     const bool vec = a.K >= 4 && a.K % 4 == 0 && aligned16(a.nm) && (!a.shifts || aligned16(a.shifts));
+    const bool sw = a.inv_sw > 0.0;
+#define NVAMD_LJ_LAUNCH(V, S, Y, W)                                                                  \
+    {                                                                                                \
+        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true, W>), grid, blk, 0, st, b); \
+        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false, W>), grid, blk, 0, st, b);    \
+        return;                                                                                      \
+    }
 #define NVAMD_LJ_CASE(V, S, Y)                                                                 \
     if (virial == V && shifts == S && sys == Y) {                                              \
-        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true>), grid, blk, 0, st, b); \
-        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false>), grid, blk, 0, st, b);    \
-        return;                                                                                \
+        if (sw) NVAMD_LJ_LAUNCH(V, S, Y, true) else NVAMD_LJ_LAUNCH(V, S, Y, false)            \
     }
     NVAMD_LJ_CASE(false, false, false)
     NVAMD_LJ_CASE(false, false, true)
@@ -493,6 +517,7 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
     NVAMD_LJ_CASE(true, false, true)
     NVAMD_LJ_CASE(true, true, true)
 #undef NVAMD_LJ_CASE
+#undef NVAMD_LJ_LAUNCH
 }
 
 int lanes_per_row(int K) {
@@ -551,8 +576,8 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const
                                                     void* workspace, size_t workspace_bytes, void* stream) {
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
-    if (switch_width != 0.0)
-        return fail(NVAMD_ERR_UNSUPPORTED, "lj: switch_width > 0 (C2 switching) is not implemented");
+    if (!(switch_width >= 0.0) || switch_width > cutoff)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: switch_width %g outside [0, cutoff]", switch_width);
     if (n_atoms > 0 && (!positions || !num_neighbors || !batch_idx || !atomic_energies || !forces))
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: null per-atom buffer");
     if (n_atoms > 0 && max_neighbors > 0 && !neighbor_matrix)
@@ -590,6 +615,8 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const
     a.sys_first = nullptr;
     a.sys_last = nullptr;
     a.lds_atoms = getenv("NVAMD_LJ_NO_LDS") ? 0 : kLdsAtoms;
+    a.r_on = switch_width > 0.0 ? cutoff - switch_width : 0.0;
+    a.inv_sw = switch_width > 0.0 ? 1.0 / switch_width : 0.0;
     // (a list built with a smaller cutoff than the potential's would be the caller's mistake:
     // the larger of the two is the safe bound)
     a.list_rc = (neighbor_list_cutoff > 0.0 && !half_list && !getenv("NVAMD_LJ_READ_SHIFTS"))

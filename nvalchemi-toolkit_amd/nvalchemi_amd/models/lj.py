@@ -32,7 +32,9 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
     epsilon, sigma, cutoff : float
         Well depth, zero-crossing distance, cutoff radius.
     switch_width : float
-        Must be ``0.0``: the C2 switching function is not implemented.
+        Width of the C2-continuous switching region below ``cutoff``; ``0.0`` (default) is plain
+        truncation.  The pair energy is multiplied by ``1 - t^3 (10 - 15 t + 6 t^2)`` with
+        ``t = (r - (cutoff - switch_width)) / switch_width``.
     half_list : bool
         ``True`` if the neighbor matrix holds each pair once.
     """
@@ -40,8 +42,8 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
     def __init__(self, epsilon: float, sigma: float, cutoff: float, switch_width: float = 0.0,
                  half_list: bool = False) -> None:
         super().__init__()
-        if switch_width != 0.0:
-            raise NotImplementedError("switch_width > 0 (C2 switching) is not implemented")
+        if not 0.0 <= switch_width <= cutoff:
+            raise ValueError(f"switch_width {switch_width} outside [0, cutoff]")
         self.epsilon = epsilon
         self.sigma = sigma
         self.cutoff = cutoff

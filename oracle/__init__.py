@@ -51,6 +51,11 @@ def lib() -> ctypes.CDLL:
                                     ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
                                     ctypes.c_double, ctypes.c_double, ctypes.c_double,
                                     ctypes.c_int32, _f32p, _f32p, _f32p, _f32p]
+        L.orc_lj_matrix_switched.restype = ctypes.c_int32
+        L.orc_lj_matrix_switched.argtypes = [_f32p, _f32p, _i32p, _i32p, _i32p, _i32p, ctypes.c_int32,
+                                             ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                             ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double,
+                                             ctypes.c_int32, _f32p, _f32p, _f32p, _f32p]
         L.orc_vv_pre.restype = None
         L.orc_vv_pre.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _i32p, _u8p, ctypes.c_int32]
         L.orc_vv_post.restype = None
@@ -167,7 +172,7 @@ def nl_cell(positions, cell, pbc, batch_ptr, cutoff: float, max_neighbors: int, 
 
 
 def lj_matrix(positions, cells, neighbor_matrix, shifts, num_neighbors, batch_idx, fill_value,
-              epsilon, sigma, cutoff, half=False, virial=False):
+              epsilon, sigma, cutoff, half=False, virial=False, switch_width=0.0):
     """LJ over the dense matrix -> dict(atomic_energies, forces, energy[, virials])."""
     pos = _f32(positions)
     N = pos.shape[0]
@@ -182,10 +187,10 @@ def lj_matrix(positions, cells, neighbor_matrix, shifts, num_neighbors, batch_id
     f = np.zeros((N, 3), dtype=np.float32)
     w = np.zeros((B, 9), dtype=np.float32) if virial else None
     es = np.zeros(B, dtype=np.float32)
-    lib().orc_lj_matrix(_p(pos, _f32p), _p(cells, _f32p), _p(nm, _i32p), _p(sh, _i32p), _p(nn, _i32p),
-                        _p(bi, _i32p), N, K, B, int(fill_value), float(epsilon), float(sigma),
-                        float(cutoff), int(half), _p(e, _f32p), _p(f, _f32p), _p(w, _f32p),
-                        _p(es, _f32p))
+    lib().orc_lj_matrix_switched(_p(pos, _f32p), _p(cells, _f32p), _p(nm, _i32p), _p(sh, _i32p), _p(nn, _i32p),
+                                 _p(bi, _i32p), N, K, B, int(fill_value), float(epsilon), float(sigma),
+                                 float(cutoff), float(switch_width), int(half), _p(e, _f32p), _p(f, _f32p),
+                                 _p(w, _f32p), _p(es, _f32p))
     out = {"atomic_energies": e, "forces": f, "energy": es}
     if virial:
         out["virials"] = w

@@ -38,8 +38,11 @@
  *                  W = -dE/d(strain) by finite differences, sum F = 0.
  *                  Still unpinned by anything the reference holds: whether the truncated
  *                  potential is energy-shifted at the cutoff (taken as NOT shifted), the
- *                  C2 switching polynomial for switch_width > 0 (not implemented), the
- *                  half-list energy attribution.
+ *                  half-list energy attribution, and the C2 switching polynomial for
+ *                  switch_width > 0: PARITY UNPINNED (the reference only says "C2-continuous ...
+ *                  between cutoff - switch_width and cutoff"; the quintic of least degree is
+ *                  taken and checked for what C2 continuity demands: S = 1 / 0 and zero slope
+ *                  and curvature at the ends, S(1/2) = 1/2, F = -dE/dr by finite differences).
  *   orc_vv_*       pinned: harmonic-oscillator closed form, time reversibility.
  *   orc_fire_step  PARITY UNPINNED against the reference: the exact ordering of FIRE's
  *                  sub-steps is only visible inside the absent wheel.  The restatement
@@ -362,13 +365,37 @@ ORC_API int32_t orc_nl_cell(const float* pos, const float* cell, const uint8_t* 
  *           (nvalchemi/models/lj.py:467-477)
  * Half list: each pair once; e split half/half, force applied to both atoms.
  * ---------------------------------------------------------------------------------------- */
+ORC_API int32_t orc_lj_matrix_switched(const float* pos, const float* cells, const int32_t* nm,
+                                       const int32_t* shifts, const int32_t* nn, const int32_t* batch_idx,
+                                       int32_t n_atoms, int32_t K, int32_t n_systems, int32_t fill_value,
+                                       double epsilon, double sigma, double cutoff, double switch_width,
+                                       int32_t half, float* atomic_energies, float* forces, float* virials,
+                                       float* system_energies);
+
 ORC_API int32_t orc_lj_matrix(const float* pos, const float* cells, const int32_t* nm,
                               const int32_t* shifts, const int32_t* nn, const int32_t* batch_idx,
                               int32_t n_atoms, int32_t K, int32_t n_systems, int32_t fill_value,
                               double epsilon, double sigma, double cutoff, int32_t half,
                               float* atomic_energies, float* forces, float* virials,
                               float* system_energies) {
+    return orc_lj_matrix_switched(pos, cells, nm, shifts, nn, batch_idx, n_atoms, K, n_systems, fill_value,
+                                  epsilon, sigma, cutoff, 0.0, half, atomic_energies, forces, virials,
+                                  system_energies);
+}
+
+/* switch_width > 0: u(r) is multiplied by S(t) = 1 - 10 t^3 + 15 t^4 - 6 t^5, t = (r - r_on) / width,
+ * r_on = cutoff - width, for r_on < r < cutoff (nvalchemi/models/_ops/lj.py:158-160 describes a
+ * "C2-continuous switching region applied between cutoff - switch_width and cutoff"; the polynomial
+ * itself is in the absent kernel library: this is the one of least degree with S(0) = 1, S(1) = 0 and
+ * zero first and second derivatives at both ends). */
+ORC_API int32_t orc_lj_matrix_switched(const float* pos, const float* cells, const int32_t* nm,
+                                       const int32_t* shifts, const int32_t* nn, const int32_t* batch_idx,
+                                       int32_t n_atoms, int32_t K, int32_t n_systems, int32_t fill_value,
+                                       double epsilon, double sigma, double cutoff, double switch_width,
+                                       int32_t half, float* atomic_energies, float* forces, float* virials,
+                                       float* system_energies) {
     double rc2 = cutoff * cutoff, sig2 = sigma * sigma;
+    double r_on = cutoff - switch_width;
     double* e = (double*)calloc((size_t)n_atoms, sizeof(double));
     double* f = (double*)calloc((size_t)n_atoms * 3, sizeof(double));
     double* w = (double*)calloc((size_t)n_systems * 9, sizeof(double));
@@ -392,6 +419,16 @@ ORC_API int32_t orc_lj_matrix(const float* pos, const float* cells, const int32_
             double s2 = sig2 * ir2, s6 = s2 * s2 * s2, s12 = s6 * s6;
             double u = 4.0 * epsilon * (s12 - s6);
             double g = -24.0 * epsilon * (2.0 * s12 - s6) * ir2; /* u'(r)/r */
+            if (switch_width > 0.0) {
+                double r = sqrt(r2);
+                if (r > r_on) {
+                    double t = (r - r_on) / switch_width;
+                    double S = 1.0 - 10.0 * t * t * t + 15.0 * t * t * t * t - 6.0 * t * t * t * t * t;
+                    double dS = (-30.0 * t * t + 60.0 * t * t * t - 30.0 * t * t * t * t) / switch_width;
+                    g = g * S + u * dS / r;
+                    u = u * S;
+                }
+            }
             double pf = half ? 1.0 : 0.5;
             if (half) {
                 e[i] += 0.5 * u;

@@ -25,7 +25,8 @@ def T(a, dtype=None):
     return t.to(DEV)
 
 
-def gpu_lj(P, C, nm, sh, nn, bi, eps, sig, rc, half=False, virial=False, sys_e=True):
+def gpu_lj(P, C, nm, sh, nn, bi, eps, sig, rc, half=False, virial=False, sys_e=True, switch_width=0.0,
+           neighbor_list_cutoff=0.0):
     from nvalchemi_amd import _lib
 
     N, B = len(P), len(C)
@@ -34,7 +35,8 @@ def gpu_lj(P, C, nm, sh, nn, bi, eps, sig, rc, half=False, virial=False, sys_e=T
     w = torch.empty((B, 9), dtype=torch.float32, device=DEV) if virial else None
     es = torch.empty(B, dtype=torch.float32, device=DEV) if sys_e else None
     _lib.lj_energy_forces(T(P, torch.float32), T(C, torch.float32), T(nm), None if sh is None else T(sh),
-                          T(nn), T(bi), N, eps, sig, rc, 0.0, half, e, f, w, es)
+                          T(nn), T(bi), N, eps, sig, rc, switch_width, half, e, f, w, es,
+                          neighbor_list_cutoff=neighbor_list_cutoff)
     torch.cuda.synchronize()
     out = {"atomic_energies": e.cpu().numpy(), "forces": f.cpu().numpy()}
     if virial:
@@ -108,6 +110,29 @@ def test_lj_half_list_matches_full_list_totals():
     ref = oracle.lj_matrix(P, C, nm, sh, nn, bi, len(P), 1.0, 1.0, 2.5, half=True, virial=True)
     got = gpu_lj(P, C, nm, sh, nn, bi, 1.0, 1.0, 2.5, half=True, virial=True)
     assert_close(got, ref, "half")
+
+
+@pytest.mark.parametrize("half", [False, True])
+@pytest.mark.parametrize("name,kw,rc,eps,sig", LJ_CASES, ids=[c[0] for c in LJ_CASES])
+def test_lj_switched_matches_oracle(name, kw, rc, eps, sig, half):
+    """switch_width > 0: energy, forces, virial and system energies against the oracle, full list
+    (shifts read and derived) and half list; the switch changes the result where it should."""
+    P, C, pb, ptr = periodic_batch(**kw)
+    bi = oracle.batch_idx_from_ptr(ptr)
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, rc, 8, half=half)
+    K = int(nn.max()) + 2
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, rc, K, half=half)
+    width = 0.3 * rc
+    ref = oracle.lj_matrix(P, C, nm, sh, nn, bi, len(P), eps, sig, rc, half=half, virial=True, switch_width=width)
+    got = gpu_lj(P, C, nm, sh, nn, bi, eps, sig, rc, half=half, virial=True, switch_width=width)
+    assert_close(got, ref, name)
+    plain = gpu_lj(P, C, nm, sh, nn, bi, eps, sig, rc, half=half, virial=True)
+    # (random positions: a few close pairs dominate the totals, so compare atom by atom)
+    assert np.mean(plain["atomic_energies"] != got["atomic_energies"]) > 0.5
+    if not half:
+        derived = gpu_lj(P, C, nm, sh, nn, bi, eps, sig, rc, virial=True, switch_width=width, neighbor_list_cutoff=rc)
+        assert np.array_equal(derived["forces"], got["forces"])
+        assert np.array_equal(derived["atomic_energies"], got["atomic_energies"])
 
 
 def test_lj_cutoff_filters_a_wider_list():

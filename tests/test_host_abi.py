@@ -49,9 +49,9 @@ def test_error_codes_and_messages_cross_the_boundary():
     # invalid arguments are rejected before anything touches a device
     rc = lib.nvamd_nl_build(None, None, None, None, None, None, 10, 1, -1.0, 8, 0, 0, None, None, None, None, 0, None)
     assert rc == 1 and b"cutoff" in lib.nvamd_last_error()
-    rc = lib.nvamd_lj_energy_forces(None, None, None, None, None, None, 0, 0, 0, 0, 1.0, 1.0, 1.0, 0.5, 0,
+    rc = lib.nvamd_lj_energy_forces(None, None, None, None, None, None, 0, 0, 0, 0, 1.0, 1.0, 1.0, 1.5, 0,
                                     None, None, None, None, None, 0, None)
-    assert rc == 4 and b"switch_width" in lib.nvamd_last_error()
+    assert rc == 1 and b"switch_width" in lib.nvamd_last_error()
 
 
 def test_cpu_tensors_are_refused_not_emulated():

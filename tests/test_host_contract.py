@@ -111,8 +111,9 @@ def test_neighbor_config_defaults_and_lj_model_config():
     assert len(hooks) == 1 and hooks[0].stage == DynamicsStage.BEFORE_COMPUTE and hooks[0]._max_neighbors_override == 48
     with pytest.raises(KeyError):
         lj(two_systems())
-    with pytest.raises(NotImplementedError):
-        LennardJonesModelWrapper(0.01, 3.4, 8.5, switch_width=0.5)
+    assert LennardJonesModelWrapper(0.01, 3.4, 8.5, switch_width=0.5).switch_width == 0.5
+    with pytest.raises(ValueError):
+        LennardJonesModelWrapper(0.01, 3.4, 8.5, switch_width=9.0)
 
 
 def test_adapt_output_stress_is_minus_virial_over_volume():

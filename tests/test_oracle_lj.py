@@ -164,3 +164,61 @@ def test_per_system_energy_is_fp64_sum_of_rounded_atomic_energies():
     out = oracle.lj_matrix(P, C, nm, sh, nn, bi, len(P), 1.0, 1.0, 2.5)
     exp = np.array([out["atomic_energies"][bi == s].astype(np.float64).sum() for s in range(3)]).astype(np.float32)
     assert np.array_equal(out["energy"], exp)
+
+
+def _dimer_switched(r, width, rc=7.5):
+    pos = np.array([[0.0, 0, 0], [r, 0, 0]], dtype=np.float32)
+    nm = np.array([[1, 2], [0, 2]], dtype=np.int32)
+    nn = np.array([1, 1], dtype=np.int32)
+    return oracle.lj_matrix(pos, np.eye(3)[None], nm, None, nn, [0, 0], 2, EPS, SIG, rc, switch_width=width)
+
+
+def test_switch_leaves_the_inner_region_alone_and_halves_the_energy_midway():
+    rc, w = 7.5, 1.5
+    for r in (2.6, 4.0, 5.99):  # below rc - w = 6.0
+        a, b = _dimer_switched(r, w), _dimer_switched(r, 0.0)
+        assert np.array_equal(a["forces"], b["forces"]) and np.array_equal(a["energy"], b["energy"])
+    mid = rc - w / 2  # 6.75: exactly representable
+    assert _dimer_switched(mid, w)["energy"][0] == pytest.approx(0.5 * _dimer_switched(mid, 0.0)["energy"][0], rel=1e-6)
+    # S falls monotonically from 1 to 0
+    ratios = [_dimer_switched(r, w)["energy"][0] / _dimer_switched(r, 0.0)["energy"][0]
+              for r in np.linspace(6.0, 7.49, 12)]
+    assert all(x > y for x, y in zip(ratios, ratios[1:])) and ratios[0] == pytest.approx(1.0) and ratios[-1] < 1e-4
+
+
+def test_switched_force_is_minus_energy_gradient():
+    rc, w, h = 7.5, 1.5, 2.0 ** -9
+    for r in (6.125, 6.5, 6.75, 7.0, 7.375):
+        ep = float(_dimer_switched(r + h, w)["energy"][0])
+        em = float(_dimer_switched(r - h, w)["energy"][0])
+        f1 = float(_dimer_switched(r, w)["forces"][1, 0])  # force on the atom at +x is -dE/dr
+        assert f1 == pytest.approx(-(ep - em) / (2 * h), rel=2e-3, abs=1e-9), r
+
+
+def test_switch_is_c2_at_both_ends():
+    """Energy, force and force derivative meet the unswitched potential at r_on and vanish at the
+    cutoff: with S ~ 1 - 10 t^3 near r_on and S ~ 10 (1 - t)^3 near the cutoff, the differences shrink
+    with the third, second and first power of the distance to the end."""
+    rc, w = 7.5, 1.5
+    for d in (2.0 ** -4, 2.0 ** -6):
+        t = d / w
+        near_on_sw, near_on = _dimer_switched(6.0 + d, w), _dimer_switched(6.0 + d, 0.0)
+        u = float(near_on["energy"][0])
+        assert abs(float(near_on_sw["energy"][0]) - u) < 11 * t ** 3 * abs(u)
+        f_sw, f = float(near_on_sw["forces"][1, 0]), float(near_on["forces"][1, 0])
+        # |u S'| <= 30 t^2 |u| / w on top of the unswitched force
+        assert abs(f_sw - f) < 31 * t ** 2 * abs(u) / w + 11 * t ** 3 * abs(f)
+        near_rc_sw, near_rc = _dimer_switched(7.5 - d, w), _dimer_switched(7.5 - d, 0.0)
+        u = float(near_rc["energy"][0])
+        assert abs(float(near_rc_sw["energy"][0])) < 11 * t ** 3 * abs(u)
+        assert abs(float(near_rc_sw["forces"][1, 0])) < 31 * t ** 2 * abs(u) / w + 11 * t ** 3 * abs(float(near_rc["forces"][1, 0]))
+    # the force derivative is continuous: slopes across r_on agree
+    h = 2.0 ** -7
+    f = lambda r: float(_dimer_switched(r, w)["forces"][1, 0])  # noqa: E731
+    slope_in = (f(6.0) - f(6.0 - h)) / h
+    slope_out = (f(6.0 + h) - f(6.0)) / h
+    g = lambda r: float(_dimer_switched(r, 0.0)["forces"][1, 0])  # noqa: E731
+    plain = (g(6.0 + h) - g(6.0)) / h
+    # (a switch that is only C1, such as 1 - 3 t^2 + 2 t^3, would add u S'' = 6 u / w^2: twice the slope itself)
+    assert slope_out == pytest.approx(plain, rel=0.1)
+    assert slope_in == pytest.approx(slope_out, rel=0.1)
