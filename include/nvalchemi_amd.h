@@ -228,6 +228,68 @@ int32_t nvamd_wrap_positions(float* positions, const float* cell, const uint8_t*
                              const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
                              void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Masked copy and in-place compaction of per-system rows and of per-system segments: replace the
+ * Warp launches of nvalchemi/data/buffer_kernels.py (the data movement of Batch.put / Batch.defrag,
+ * nvalchemi/data/batch.py:876-985).  Rows are opaque runs of row_bytes bytes (any dtype; source and
+ * destination share it); masks are one byte per system, 0 or 1.
+ * Workspace for all of them: nvamd_buffer_workspace_bytes(number of source systems, data bytes),
+ * where data bytes is the size of `source` for the two defrag calls and 0 for the others.
+ * ---------------------------------------------------------------------------------------- */
+int32_t nvamd_buffer_workspace_bytes(int64_t n_systems, int64_t data_bytes, size_t* bytes);
+
+/* put_masked_per_system (buffer_kernels.py:970-1079,1171-1220): of the rows with source_mask set,
+ * the first min(#masked, #empty destination slots) go to consecutive destination slots starting at
+ * the first empty one (dest_mask 0 = empty); dest_mask is set for the written slots and
+ * source_data_copied for the moved rows (neither is cleared elsewhere). */
+int32_t nvamd_put_masked_per_system(const void* source, const uint8_t* source_mask, void* dest,
+                                    uint8_t* dest_mask, uint8_t* source_data_copied, int32_t num_src,
+                                    int32_t num_dest, int64_t row_bytes, void* workspace,
+                                    size_t workspace_bytes, void* stream);
+
+/* compute_put_fit_mask_per_system (buffer_kernels.py:1081-1169): fit_mask[i] = the row would be
+ * moved by the call above.  Nothing is copied. */
+int32_t nvamd_put_fit_mask_per_system(const uint8_t* source_mask, const uint8_t* dest_mask,
+                                      uint8_t* fit_mask, int32_t num_src, int32_t num_dest,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* defrag_per_system (buffer_kernels.py:1222-1333): rows with source_data_copied 0 move to the
+ * front in their order, the rows behind them are zeroed, and source_data_copied[i] becomes
+ * (i >= number kept). */
+int32_t nvamd_defrag_per_system(void* source, uint8_t* source_data_copied, int32_t num_src,
+                                int64_t row_bytes, void* workspace, size_t workspace_bytes,
+                                void* stream);
+
+/* put_masked_segmented (buffer_kernels.py:1335-1527): segment i is rows
+ * [source_batch_ptr[i], source_batch_ptr[i+1]).  Masked segments are laid out one after another
+ * from dest_batch_ptr[num_dest_segments]; those that end at or before dest_capacity rows are
+ * copied, their ends appended to dest_batch_ptr (which must hold num_dest_segments + num_systems
+ * + 2 entries: one more copy of the last end follows the new ones), source_data_copied set for
+ * them, and *new_num_dest = num_dest_segments + number copied.  total_rows = rows of `source`. */
+int32_t nvamd_put_masked_segmented(const void* source, const int32_t* source_batch_ptr,
+                                   const uint8_t* source_mask, void* dest, int32_t* dest_batch_ptr,
+                                   int32_t num_dest_segments, int32_t dest_capacity,
+                                   uint8_t* source_data_copied, int32_t* new_num_dest,
+                                   int32_t num_systems, int32_t total_rows, int64_t row_bytes,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* compute_put_fit_mask_segmented (buffer_kernels.py:500-610): fit_mask[i] = segment i would be
+ * copied by the call above.  (The reference's host wrapper clears the mask instead when
+ * dest_batch_ptr is too short; that check stays with the caller.) */
+int32_t nvamd_put_fit_mask_segmented(const int32_t* source_batch_ptr, const uint8_t* source_mask,
+                                     const int32_t* dest_batch_ptr, int32_t num_dest_segments,
+                                     int32_t dest_capacity, uint8_t* fit_mask, int32_t num_systems,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* defrag_segmented (buffer_kernels.py:1529-1741): segments with source_data_copied 0 move to the
+ * front in their order, the rows behind them are zeroed; source_batch_ptr[0..kept] becomes the new
+ * boundaries and every later entry the number of rows kept; *num_kept = segments kept.  With
+ * num_systems == 0: source_batch_ptr[0] = 0 and *num_kept = 0. */
+int32_t nvamd_defrag_segmented(void* source, int32_t* source_batch_ptr,
+                               const uint8_t* source_data_copied, int32_t* num_kept,
+                               int32_t num_systems, int32_t total_rows, int64_t row_bytes,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

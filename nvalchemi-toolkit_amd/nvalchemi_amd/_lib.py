@@ -10,6 +10,7 @@ library, raises.
 from __future__ import annotations
 
 import ctypes
+import math
 from pathlib import Path
 
 import torch
@@ -47,6 +48,14 @@ _SIGNATURES = {
     "nvamd_kinetic_energy": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_buffer_workspace_bytes": (_i32, [_c.c_int64, _c.c_int64, _c.POINTER(_c.c_size_t)]),
+    "nvamd_put_masked_per_system": (_i32, [_vp] * 5 + [_i32, _i32, _c.c_int64, _vp, _c.c_size_t, _vp]),
+    "nvamd_put_fit_mask_per_system": (_i32, [_vp] * 3 + [_i32, _i32, _vp, _c.c_size_t, _vp]),
+    "nvamd_defrag_per_system": (_i32, [_vp, _vp, _i32, _c.c_int64, _vp, _c.c_size_t, _vp]),
+    "nvamd_put_masked_segmented": (_i32, [_vp] * 5 + [_i32, _i32, _vp, _vp, _i32, _i32, _c.c_int64, _vp,
+                                          _c.c_size_t, _vp]),
+    "nvamd_put_fit_mask_segmented": (_i32, [_vp] * 3 + [_i32, _i32, _vp, _i32, _vp, _c.c_size_t, _vp]),
+    "nvamd_defrag_segmented": (_i32, [_vp] * 4 + [_i32, _i32, _c.c_int64, _vp, _c.c_size_t, _vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -351,3 +360,104 @@ def kinetic_energy(velocities, masses, batch_idx, out) -> None:
         _dev(velocities, "velocities", torch.float32, (n, 3)), _dev(masses, "masses", torch.float32, (n,)),
         _dev(batch_idx, "batch_idx", torch.int32, (n,)), n, m, _dev(out, "kinetic_energy", torch.float32, (m,)),
         ws.data_ptr(), ws.numel(), _stream(velocities.device)), "nvamd_kinetic_energy")
+
+
+# --------------------------------------------------------------------------------------------
+# masked copy / compaction of rows and segments
+# --------------------------------------------------------------------------------------------
+BUFFER_DTYPES = (torch.bool, torch.float32, torch.float64, torch.int32, torch.int64)
+
+
+def _rows(t: torch.Tensor, name: str) -> tuple[int, int]:
+    """Device pointer and bytes per row of a contiguous (rows, ...) tensor of a supported dtype."""
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if t.device.type != "cuda":
+        raise KernelLibraryError(f"{name}: tensor is on {t.device}; the nvalchemi_amd kernels run on a ROCm device only")
+    if t.dtype not in BUFFER_DTYPES:
+        raise KeyError(t.dtype)
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: tensor must be contiguous")
+    return t.data_ptr(), math.prod(t.shape[1:]) * t.element_size()
+
+
+def _mask(t: torch.Tensor, name: str, n: int) -> int:
+    return _dev(_as_u8(t), name, torch.uint8, (n,))
+
+
+def _buffer_ws(device, n_systems: int, data_bytes: int = 0) -> torch.Tensor:
+    need = _size(library().nvamd_buffer_workspace_bytes, int(n_systems), int(data_bytes))
+    return workspaces.get(device, "buffers", need)
+
+
+def put_masked_per_system(source, source_mask, dest, dest_mask, source_data_copied) -> None:
+    n_src, n_dest = source.shape[0], dest.shape[0]
+    if source.dtype != dest.dtype:
+        raise TypeError(f"source {source.dtype} and dest {dest.dtype} differ")
+    sp, rb = _rows(source, "source")
+    dp, rb_d = _rows(dest, "dest")
+    if n_src and n_dest and rb != rb_d:
+        raise ValueError(f"source rows have {rb} bytes, dest rows {rb_d}")
+    ws = _buffer_ws(source.device, n_src)
+    _check(library().nvamd_put_masked_per_system(
+        sp, _mask(source_mask, "source_mask", n_src), dp, _mask(dest_mask, "dest_mask", n_dest),
+        _mask(source_data_copied, "source_data_copied", n_src), n_src, n_dest, rb, ws.data_ptr(), ws.numel(),
+        _stream(source.device)), "nvamd_put_masked_per_system")
+
+
+def put_fit_mask_per_system(source_mask, dest_mask, fit_mask) -> None:
+    n_src, n_dest = source_mask.shape[0], dest_mask.shape[0]
+    ws = _buffer_ws(source_mask.device, n_src)
+    _check(library().nvamd_put_fit_mask_per_system(
+        _mask(source_mask, "source_mask", n_src), _mask(dest_mask, "dest_mask", n_dest),
+        _mask(fit_mask, "fit_mask", n_src), n_src, n_dest, ws.data_ptr(), ws.numel(),
+        _stream(source_mask.device)), "nvamd_put_fit_mask_per_system")
+
+
+def defrag_per_system(source, source_data_copied) -> None:
+    n = source.shape[0]
+    sp, rb = _rows(source, "source")
+    ws = _buffer_ws(source.device, n, n * rb)
+    _check(library().nvamd_defrag_per_system(
+        sp, _mask(source_data_copied, "source_data_copied", n), n, rb, ws.data_ptr(), ws.numel(),
+        _stream(source.device)), "nvamd_defrag_per_system")
+
+
+def put_masked_segmented(source, source_batch_ptr, source_mask, dest, dest_batch_ptr, num_dest_segments: int,
+                         source_data_copied, new_num_dest) -> None:
+    n = source_batch_ptr.shape[0] - 1
+    if source.dtype != dest.dtype:
+        raise TypeError(f"source {source.dtype} and dest {dest.dtype} differ")
+    sp, rb = _rows(source, "source")
+    dp, rb_d = _rows(dest, "dest")
+    if source.shape[0] and dest.shape[0] and rb != rb_d:
+        raise ValueError(f"source rows have {rb} bytes, dest rows {rb_d}")
+    ws = _buffer_ws(source.device, n)
+    _check(library().nvamd_put_masked_segmented(
+        sp, _dev(source_batch_ptr, "source_batch_ptr", torch.int32, (n + 1,)), _mask(source_mask, "source_mask", n),
+        dp, _dev(dest_batch_ptr, "dest_batch_ptr", torch.int32), int(num_dest_segments), dest.shape[0],
+        _mask(source_data_copied, "source_data_copied", n), _dev(new_num_dest, "new_num_dest", torch.int32, (1,)),
+        n, source.shape[0], rb if source.shape[0] else rb_d, ws.data_ptr(), ws.numel(), _stream(source.device)),
+        "nvamd_put_masked_segmented")
+
+
+def put_fit_mask_segmented(source_batch_ptr, source_mask, dest_batch_ptr, num_dest_segments: int,
+                           dest_capacity: int, fit_mask) -> None:
+    n = source_batch_ptr.shape[0] - 1
+    ws = _buffer_ws(source_batch_ptr.device, n)
+    _check(library().nvamd_put_fit_mask_segmented(
+        _dev(source_batch_ptr, "source_batch_ptr", torch.int32, (n + 1,)), _mask(source_mask, "source_mask", n),
+        _dev(dest_batch_ptr, "dest_batch_ptr", torch.int32), int(num_dest_segments), int(dest_capacity),
+        _mask(fit_mask, "fit_mask", n), n, ws.data_ptr(), ws.numel(), _stream(source_batch_ptr.device)),
+        "nvamd_put_fit_mask_segmented")
+
+
+def defrag_segmented(source, source_batch_ptr, source_data_copied, num_kept) -> None:
+    n = source_batch_ptr.shape[0] - 1
+    sp, rb = _rows(source, "source")
+    rows = source.shape[0]
+    ws = _buffer_ws(source.device, n, rows * rb)
+    _check(library().nvamd_defrag_segmented(
+        sp, _dev(source_batch_ptr, "source_batch_ptr", torch.int32, (n + 1,)),
+        _mask(source_data_copied, "source_data_copied", n), _dev(num_kept, "num_kept", torch.int32, (1,)),
+        n, rows, rb, ws.data_ptr(), ws.numel(), _stream(source.device)), "nvamd_defrag_segmented")

@@ -297,3 +297,132 @@ def kinetic_energy(velocities, masses, batch_idx, n_systems: int) -> np.ndarray:
     acc = np.zeros(int(n_systems), dtype=np.float64)
     np.add.at(acc, _i32(batch_idx), per_atom)
     return acc.astype(np.float32)
+
+
+# ---------------------------------------------------------------------------------------------
+# masked copy / compaction of rows and segments (numpy, in place like the reference's functions)
+# nvalchemi/data/buffer_kernels.py; pinned by the reference's own cases
+# (test/data/test_buffer_kernels.py:49-535), restated in tests/test_oracle_buffers.py
+# ---------------------------------------------------------------------------------------------
+def _rows2d(a):
+    return a.reshape(a.shape[0], int(np.prod(a.shape[1:])))
+
+
+def _put_plan_per_system(source_mask, dest_mask):
+    """exclusive scan of the mask, number of rows that may move, first empty slot
+    (buffer_kernels.py:58-140)"""
+    m = np.asarray(source_mask, dtype=bool)
+    scan = np.cumsum(m) - m
+    count_empty = int((~np.asarray(dest_mask, dtype=bool)).sum())
+    max_copy = min(int(m.sum()), count_empty)
+    empty = np.flatnonzero(~np.asarray(dest_mask, dtype=bool))
+    first_empty = int(empty[0]) if len(empty) else len(dest_mask)
+    return m, scan, max_copy, first_empty
+
+
+def put_masked_per_system(source, source_mask, dest, dest_mask, source_data_copied):
+    """buffer_kernels.py:143-186, 970-1079"""
+    if source.shape[0] == 0:
+        return
+    src, dst = _rows2d(source), _rows2d(dest)
+    m, scan, max_copy, first_empty = _put_plan_per_system(source_mask, dest_mask)
+    for i in range(len(m)):
+        if not m[i] or scan[i] >= max_copy:
+            continue
+        k = first_empty + scan[i]
+        dst[k] = src[i]
+        dest_mask[k] = True
+        source_data_copied[i] = True
+
+
+def put_fit_mask_per_system(source_mask, dest_mask, fit_mask):
+    """buffer_kernels.py:612-622, 1081-1169"""
+    if len(source_mask) == 0:
+        return
+    m, scan, max_copy, _ = _put_plan_per_system(source_mask, dest_mask)
+    fit_mask[:] = m & (scan < max_copy)
+
+
+def defrag_per_system(source, source_data_copied):
+    """buffer_kernels.py:189-253, 1222-1333"""
+    if source.shape[0] == 0:
+        return
+    src = _rows2d(source)
+    keep = ~np.asarray(source_data_copied, dtype=bool)
+    kept = src[keep].copy()
+    src[:] = 0
+    src[: len(kept)] = kept
+    source_data_copied[:] = np.arange(len(keep)) >= len(kept)
+
+
+def _put_plan_segmented(source_batch_ptr, source_mask, dest_batch_ptr, num_dest_segments, dest_capacity):
+    """buffer_kernels.py:372-399, 454-497"""
+    ptr = np.asarray(source_batch_ptr, dtype=np.int64)
+    m = np.asarray(source_mask, dtype=bool)
+    lengths = np.where(m, ptr[1:] - ptr[:-1], 0)
+    offset = np.cumsum(lengths) - lengths
+    base = int(dest_batch_ptr[num_dest_segments])
+    fits = m & (base + offset + lengths <= dest_capacity)
+    return ptr, lengths, offset, base, fits
+
+
+def put_fit_mask_segmented(source_batch_ptr, source_mask, dest_batch_ptr, num_dest_segments, dest_capacity,
+                           fit_mask):
+    """buffer_kernels.py:500-610"""
+    n = len(source_batch_ptr) - 1
+    if n == 0:
+        return
+    if len(dest_batch_ptr) < num_dest_segments + n + 2:
+        fit_mask[:] = False
+        return
+    fit_mask[:] = _put_plan_segmented(source_batch_ptr, source_mask, dest_batch_ptr, num_dest_segments,
+                                      dest_capacity)[4]
+
+
+def put_masked_segmented(source, source_batch_ptr, source_mask, dest, dest_batch_ptr, num_dest_segments,
+                         source_data_copied):
+    """buffer_kernels.py:624-659, 1335-1527; returns the new number of destination segments"""
+    n = len(source_batch_ptr) - 1
+    if n == 0:
+        return None
+    need = num_dest_segments + n + 2
+    if len(dest_batch_ptr) < need:
+        raise ValueError(f"dest_batch_ptr must have size >= num_dest_segments + num_systems + 2 ({need}); "
+                         f"got {len(dest_batch_ptr)}")
+    src, dst = _rows2d(source), _rows2d(dest)
+    ptr, lengths, offset, base, fits = _put_plan_segmented(source_batch_ptr, source_mask, dest_batch_ptr,
+                                                           num_dest_segments, dst.shape[0])
+    fit_scan = np.cumsum(fits) - fits
+    n_fit = int(fits.sum())
+    for i in range(n):
+        if not fits[i]:
+            continue
+        a = base + offset[i]
+        dst[a: a + lengths[i]] = src[ptr[i]: ptr[i + 1]]
+        source_data_copied[i] = True
+        end = base + offset[i] + lengths[i]
+        dest_batch_ptr[num_dest_segments + 1 + fit_scan[i]] = end
+        if fit_scan[i] == n_fit - 1:
+            dest_batch_ptr[num_dest_segments + 1 + n_fit] = end
+    return num_dest_segments + n_fit
+
+
+def defrag_segmented(source, source_batch_ptr, source_data_copied):
+    """buffer_kernels.py:661-967, 1529-1741; returns the number of kept segments"""
+    n = len(source_batch_ptr) - 1
+    if n == 0:
+        source_batch_ptr[0] = 0
+        return 0
+    src = _rows2d(source)
+    ptr = np.asarray(source_batch_ptr, dtype=np.int64).copy()
+    keep = ~np.asarray(source_data_copied, dtype=bool)
+    pieces = [src[ptr[i]: ptr[i + 1]].copy() for i in range(n) if keep[i]]
+    lengths = [len(p) for p in pieces]
+    total = int(sum(lengths))
+    src[:] = 0
+    if total:
+        src[:total] = np.concatenate(pieces)
+    num_kept = len(pieces)
+    source_batch_ptr[: num_kept + 1] = np.concatenate([[0], np.cumsum(lengths)]) if num_kept else [0]
+    source_batch_ptr[num_kept + 1:] = total
+    return num_kept
