@@ -38,6 +38,20 @@ __device__ __forceinline__ double pair_d2_shifted(float xi, float yi, float zi, 
     return (d0 * d0 + d1 * d1) + d2 * d2;
 }
 
+// The same d for a cell without off-diagonal terms when the wanted image is the nearest one:
+// d_k = dd_k - rint(dd_k / h_kk) h_kk.  rint(.) is the negated shift, its product with h_kk is exact
+// in double, so the fused multiply-add rounds once, exactly like dd_k + (S . cell)_k above.
+__device__ __forceinline__ double pair_d2_nearest_diagonal(float xi, float yi, float zi, float xj, float yj,
+                                                           float zj, const double* h, const double* h_inv,
+                                                           double& d0, double& d1, double& d2) {
+#pragma clang fp contract(off)
+    const double e0 = (double)xj - (double)xi, e1 = (double)yj - (double)yi, e2 = (double)zj - (double)zi;
+    d0 = __builtin_fma(-__builtin_rint(e0 * h_inv[0]), h[0], e0);
+    d1 = __builtin_fma(-__builtin_rint(e1 * h_inv[1]), h[1], e1);
+    d2 = __builtin_fma(-__builtin_rint(e2 * h_inv[2]), h[2], e2);
+    return (d0 * d0 + d1 * d1) + d2 * d2;
+}
+
 __device__ __forceinline__ double pair_d2_exact(float xi, float yi, float zi, float xj, float yj,
                                                 float zj, int s0, int s1, int s2,
                                                 const double* __restrict__ h, double& d0,

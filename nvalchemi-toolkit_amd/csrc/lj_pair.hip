@@ -99,16 +99,60 @@ __device__ __forceinline__ double reciprocal(double x) {
 // perpendicular width of its cell, so the listed image is the nearest one and its shift is
 // -rint((r_j - r_i) . H^-1) (float32 is ample: the listed image's fractional components stay
 // below 0.49995 in magnitude).
-template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC, bool IMG, bool SWITCH>
+// energy, force and virial terms of one pair inside the cutoff
+template <bool VIRIAL, bool SWITCH>
+__device__ __forceinline__ void pair_terms(const LjArgs& a, double r2, double d0, double d1, double d2, double& e,
+                                           double& fx, double& fy, double& fz, double& w0, double& w1, double& w2,
+                                           double& w3, double& w4, double& w5) {
+    const double ir2 = reciprocal(r2);
+    double q2 = a.sig2 * ir2;
+    double q6 = q2 * q2 * q2;
+    double q12 = q6 * q6;
+    double uu = a.c4eps * (q12 - q6);
+    double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
+    if (SWITCH) apply_switch(a, r2, uu, gg);
+    e += 0.5 * uu;
+    fx += gg * d0;
+    fy += gg * d1;
+    fz += gg * d2;
+    if (VIRIAL) {
+        double hg = -0.5 * gg;
+        w0 += hg * d0 * d0;
+        w1 += hg * d0 * d1;
+        w2 += hg * d0 * d2;
+        w3 += hg * d1 * d1;
+        w4 += hg * d1 * d2;
+        w5 += hg * d2 * d2;
+    }
+}
+
+// IMG == 2: the same for a cell with zero off-diagonal terms, where each component stands alone:
+// d_k = dd_k - rint(dd_k / h_kk) h_kk in double (the product is exact, so the fused multiply-add
+// rounds exactly like the add of the tabulated shift . cell).
+__device__ __forceinline__ double uniform_double(const double* p) {
+    const int lo = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int*>(p)[0]);
+    const int hi = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int*>(p)[1]);
+    return __hiloint2double(hi, lo);
+}
+
+template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool LDS_POS, bool VEC, int IMG, bool SWITCH>
 __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, int sys_base,
                                         const float* __restrict__ s_pos, int span0, int span_n,
                                         const double (*s_shift)[3], int table_sys, const float* s_hinv,
-                                        double (*s_acc)[VIRIAL ? 7 : 1]) {
+                                        const double* s_diag, double (*s_acc)[VIRIAL ? 7 : 1]) {
     float hi[9];
-    if (IMG) {
+    double hd[3], hdi[3];
+    if (IMG == 1) {
 #pragma unroll
         for (int k = 0; k < 9; ++k)
             hi[k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_hinv[k])));
+    }
+    if (IMG == 2) {
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            hd[k] = uniform_double(s_diag + k);
+            hdi[k] = uniform_double(s_diag + 3 + k);
+        }
     }
     constexpr int G = kBlockFull / LPR;
     const int g = threadIdx.x / LPR;
@@ -146,7 +190,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                     const int kq = kv < last_quad ? kv : last_quad;  // never past the row's last used quad
                     const int4 j4 = *reinterpret_cast<const int4*>(row + kq);
                     jj[4 * v + 0] = j4.x; jj[4 * v + 1] = j4.y; jj[4 * v + 2] = j4.z; jj[4 * v + 3] = j4.w;
-                    if (SHIFTS && !IMG) {
+                    if (SHIFTS && IMG == 0) {
                         const int4* sp = reinterpret_cast<const int4*>(srow + 3 * kq);
                         const int4 sa = sp[0], sb = sp[1], sc = sp[2];
                         s0[4 * v + 0] = sa.x; s1[4 * v + 0] = sa.y; s2[4 * v + 0] = sa.z;
@@ -155,7 +199,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                         s0[4 * v + 3] = sc.y; s1[4 * v + 3] = sc.z; s2[4 * v + 3] = sc.w;
                     }
                 }
-                if (!SHIFTS || IMG) {
+                if (!SHIFTS || IMG != 0) {
 #pragma unroll
                     for (int u = 0; u < UNROLL; ++u) s0[u] = s1[u] = s2[u] = 0;
                 }
@@ -170,7 +214,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 const int kq = k < cnt ? k : cnt - 1;
                 jj[u] = row[kq];
                 s0[u] = s1[u] = s2[u] = 0;
-                if (SHIFTS && !IMG) {
+                if (SHIFTS && IMG == 0) {
                     s0[u] = srow[3 * kq + 0];
                     s1[u] = srow[3 * kq + 1];
                     s2[u] = srow[3 * kq + 2];
@@ -198,7 +242,14 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 double t0 = 0.0, t1 = 0.0, t2 = 0.0;
-                if (IMG) {
+                if (IMG == 2) {
+                    double d0, d1, d2;
+                    const double r2 = pair_d2_nearest_diagonal(xi, yi, zi, xj[u], yj[u], zj[u], hd, hdi, d0, d1, d2);
+                    if (jj[u] < 0 || !(r2 < a.rc2)) continue;
+                    pair_terms<VIRIAL, SWITCH>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
+                    continue;
+                }
+                if (IMG == 1) {
                     const float dx = xj[u] - xi, dy = yj[u] - yi, dz = zj[u] - zi;
                     s0[u] = -(int)__builtin_rintf(dx * hi[0] + dy * hi[3] + dz * hi[6]);
                     s1[u] = -(int)__builtin_rintf(dx * hi[1] + dy * hi[4] + dz * hi[7]);
@@ -218,26 +269,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 double d0, d1, d2;
                 double r2 = pair_d2_shifted(xi, yi, zi, xj[u], yj[u], zj[u], t0, t1, t2, d0, d1, d2);
                 if (jj[u] < 0 || !(r2 < a.rc2)) continue;
-                const double ir2 = reciprocal(r2);
-                double q2 = a.sig2 * ir2;
-                double q6 = q2 * q2 * q2;
-                double q12 = q6 * q6;
-                double uu = a.c4eps * (q12 - q6);
-                double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
-                if (SWITCH) apply_switch(a, r2, uu, gg);
-                e += 0.5 * uu;
-                fx += gg * d0;
-                fy += gg * d1;
-                fz += gg * d2;
-                if (VIRIAL) {
-                    double hg = -0.5 * gg;
-                    w0 += hg * d0 * d0;
-                    w1 += hg * d0 * d1;
-                    w2 += hg * d0 * d2;
-                    w3 += hg * d1 * d1;
-                    w4 += hg * d1 * d2;
-                    w5 += hg * d2 * d2;
-                }
+                pair_terms<VIRIAL, SWITCH>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
             }
         }
         e = group_sum<LPR>(e);
@@ -291,7 +323,8 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
     __shared__ float s_pos[3 * kLdsAtoms];
     __shared__ double s_shift[27][3];  // shift . cell of the system in hand, shifts -1..1 per axis
     __shared__ float s_hinv[9];        // its inverse cell
-    __shared__ int s_img;              // its pairs' shifts follow from the positions alone
+    __shared__ double s_diag[6];       // diagonal of the cell and of its inverse
+    __shared__ int s_img;              // its pairs' shifts follow from the positions alone (2: diagonal cell)
 
     // a workgroup owns rows_per_block consecutive rows; workgroups are numbered so that each
     // XCD walks one contiguous eighth of the atoms
@@ -342,27 +375,32 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
                         if (!(n2 < lim * lim)) ok = 0;
                     }
                     for (int k = 0; k < 9; ++k) s_hinv[k] = (float)hv[k];
+                    if (ok && h[1] == 0.0 && h[2] == 0.0 && h[3] == 0.0 && h[5] == 0.0 && h[6] == 0.0 && h[7] == 0.0) {
+                        ok = 2;
+                        for (int k = 0; k < 3; ++k) {
+                            s_diag[k] = h[4 * k];
+                            s_diag[3 + k] = hv[4 * k];
+                        }
+                    }
                 }
             }
             s_img = ok;
         }
         __syncthreads();
-        const bool img = SHIFTS && s_img != 0;
+        const int img = SHIFTS ? s_img : 0;
+#define NVAMD_LJ_ROWS(STAGED, IMG)                                                                              \
+    lj_rows<LPR, VIRIAL, SHIFTS, SYS, STAGED, VEC, (SHIFTS ? IMG : 0), SWITCH>(                                  \
+        a, r, seg_end, sys_lo, s_pos, STAGED ? span0 : 0, STAGED ? span_n : 0, s_shift, sys, s_hinv, s_diag, s_acc)
         if (staged) {
-            if (img)
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, SHIFTS, SWITCH>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
-                                                                     sys, s_hinv, s_acc);
-            else
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, true, VEC, false, SWITCH>(a, r, seg_end, sys_lo, s_pos, span0, span_n, s_shift,
-                                                                    sys, s_hinv, s_acc);
+            if (img == 2) NVAMD_LJ_ROWS(true, 2);
+            else if (img == 1) NVAMD_LJ_ROWS(true, 1);
+            else NVAMD_LJ_ROWS(true, 0);
         } else {
-            if (img)
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, SHIFTS, SWITCH>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
-                                                                      s_hinv, s_acc);
-            else
-                lj_rows<LPR, VIRIAL, SHIFTS, SYS, false, VEC, false, SWITCH>(a, r, seg_end, sys_lo, s_pos, 0, 0, s_shift, sys,
-                                                                     s_hinv, s_acc);
+            if (img == 2) NVAMD_LJ_ROWS(false, 2);
+            else if (img == 1) NVAMD_LJ_ROWS(false, 1);
+            else NVAMD_LJ_ROWS(false, 0);
         }
+#undef NVAMD_LJ_ROWS
         r = seg_end;
         if (r < row_end) __syncthreads();  // the stage is about to be overwritten
     }
