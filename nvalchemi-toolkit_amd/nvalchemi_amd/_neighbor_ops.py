@@ -29,6 +29,32 @@ def estimate_max_neighbors(cutoff: float, atomic_density: float = 0.2, safety_fa
     return max(16, ceil16(math.ceil(safety_factor * expected)))
 
 
+def suggest_neighbor_list_method(batch_ptr: torch.Tensor, cell: torch.Tensor, pbc: torch.Tensor, cutoff: float,
+                                 half_fill: bool = False, return_neighbor_list: bool = False,
+                                 positions_dtype: torch.dtype = torch.float32) -> str:
+    """Strategy name for the caller's bookkeeping (call site: nvalchemi/hooks/neighbor_list.py:737-747).
+    One cell-list kernel serves every input here, so the answer only says "batched cell list"; the
+    reference's cost model lives in its kernel library and picks among strategies this build does
+    not have.  Host-only, no synchronisation."""
+    if positions_dtype != torch.float32:
+        raise NotImplementedError("the HIP neighbor list takes float32 positions")
+    return "batch_cell_list"
+
+
+def neighbor_list_strategy_run_args(method: str) -> tuple[str, dict]:
+    """``(base method, extra keyword arguments)`` of a strategy name (call site:
+    nvalchemi/hooks/neighbor_list.py:757-760, which only uses element 0 to choose the scratch it
+    allocates).  No strategy of this build takes caller-side scratch: the base name is returned
+    with no arguments, and the scratch allocators the reference imports optionally
+    (``estimate_batch_cell_list_sizes``, ``allocate_cell_list``, ``compute_naive_num_shifts``,
+    ``allocate_batch_cluster_tile_list``, ``estimate_batch_max_tiles_per_group``) have no
+    counterpart -- the caller's ``except ImportError`` branches leave them ``None``."""
+    if method not in _METHODS or method is None:
+        raise ValueError(f"unknown neighbor list method {method!r}")
+    base = {"batch_cell_list_pair_centric": "batch_cell_list"}.get(method, method)
+    return base, {}
+
+
 def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | None = None,
                   pbc: torch.Tensor | None = None, max_neighbors: int | None = None,
                   half_fill: bool = False, batch_ptr: torch.Tensor | None = None,

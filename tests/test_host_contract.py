@@ -238,3 +238,21 @@ def test_estimate_max_neighbors_is_a_multiple_of_16_and_monotone():
     ks = [estimate_max_neighbors(rc) for rc in (1.0, 2.5, 5.0, 6.0, 8.5)]
     assert all(k % 16 == 0 and k >= 16 for k in ks) and ks == sorted(ks)
     assert ceil16(1) == 16 and ceil16(16) == 16 and ceil16(17) == 32
+
+
+def test_strategy_helpers_of_the_neighbor_hook():
+    """The two helpers the reference hook imports unconditionally
+    (nvalchemi/hooks/neighbor_list.py:63-65): a strategy name and its base method."""
+    from nvalchemi_amd._neighbor_ops import neighbor_list_strategy_run_args, suggest_neighbor_list_method
+
+    ptr = torch.tensor([0, 5, 9], dtype=torch.int32)
+    name = suggest_neighbor_list_method(ptr, torch.eye(3).repeat(2, 1, 1) * 10, torch.ones(2, 3, dtype=torch.bool), 3.0,
+                                        half_fill=False, return_neighbor_list=False, positions_dtype=torch.float32)
+    base, extra = neighbor_list_strategy_run_args(name)
+    assert base.endswith("cell_list") and extra == {}
+    assert neighbor_list_strategy_run_args("batch_cell_list_pair_centric")[0] == "batch_cell_list"
+    with pytest.raises(ValueError):
+        neighbor_list_strategy_run_args("no_such_strategy")
+    with pytest.raises(NotImplementedError):
+        suggest_neighbor_list_method(ptr, torch.eye(3).repeat(2, 1, 1), torch.ones(2, 3, dtype=torch.bool), 3.0,
+                                     positions_dtype=torch.float64)
