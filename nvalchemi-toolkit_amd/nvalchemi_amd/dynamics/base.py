@@ -351,6 +351,61 @@ class BaseDynamics(HookRegistryMixin):
         self.step_count += 1
         return batch, converged
 
+    # ---- updates of selected systems only (nvalchemi/dynamics/base.py:2085-2212) ---------------
+    def _run_masked(self, batch, mask: torch.Tensor, do_pre: bool, do_post: bool) -> None:
+        """``pre_update`` and/or ``post_update`` for the systems with ``mask`` set; the others keep
+        their mutable fields.  Integrators whose kernels take the mask get it; for the rest the
+        fields of the unselected systems are saved and restored, as in the reference."""
+        self._ensure_state_initialized(batch)
+        mask = mask.to(device=batch.device, dtype=torch.bool)
+        previous = self._active_mask
+        if self._honors_active_mask:
+            self._active_mask = mask
+            try:
+                if do_pre:
+                    self.pre_update(batch)
+                if do_post:
+                    self.post_update(batch)
+            finally:
+                self._active_mask = previous
+            return
+        node_mask = mask[batch.batch_idx.to(torch.long)]
+        sys_mask = ~mask
+        saved: dict[str, torch.Tensor] = {}
+        for field in self._mutable_fields:
+            val = getattr(batch, field, None)
+            if val is None:
+                continue
+            if val.shape[0] == batch.num_nodes:
+                saved[field] = val[~node_mask].clone()
+            elif val.shape[0] == batch.num_graphs:
+                saved[field] = val[sys_mask].clone()
+        self._active_mask = None
+        try:
+            if do_pre:
+                self.pre_update(batch)
+            if do_post:
+                self.post_update(batch)
+        finally:
+            self._active_mask = previous
+        with torch.no_grad():
+            for field, sv in saved.items():
+                val = getattr(batch, field)
+                if val.shape[0] == batch.num_nodes:
+                    val[~node_mask] = sv
+                else:
+                    val[sys_mask] = sv
+
+    def masked_update(self, batch, mask: torch.Tensor) -> None:
+        """``pre_update`` then ``post_update`` for the systems selected by ``mask (B,) bool``."""
+        self._run_masked(batch, mask, True, True)
+
+    def _masked_pre_update(self, batch, mask: torch.Tensor) -> None:
+        self._run_masked(batch, mask, True, False)
+
+    def _masked_post_update(self, batch, mask: torch.Tensor) -> None:
+        self._run_masked(batch, mask, False, True)
+
     def run(self, batch, n_steps: int | None = None):
         resolved = n_steps if n_steps is not None else self.n_steps
         if resolved is None:

@@ -339,3 +339,40 @@ def test_hook_leaves_the_cell_order_for_large_systems_and_the_model_uses_it():
     hook2 = model.make_neighbor_hooks()[0]
     hook2(HookContext(batch=small), None)
     assert getattr(small, "_neighbor_row_order", None) is None
+
+
+def test_masked_update_moves_only_the_selected_systems():
+    """``masked_update`` / ``_masked_pre_update`` / ``_masked_post_update``
+    (nvalchemi/dynamics/base.py:2085-2212): selected systems advance exactly as in an unmasked
+    update, the others keep positions and velocities -- through the kernels' own mask (NVE) and
+    through the save-and-restore route of integrators that do not take one."""
+    from nvalchemi_amd.dynamics import NVE
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = periodic_batch(seed=77, n_systems=5, n_lo=40, n_hi=90, density=0.5)
+    rng = np.random.default_rng(1)
+    V = rng.normal(0, 0.3, P.shape).astype(np.float32)
+    F = rng.normal(0, 1.0, P.shape).astype(np.float32)
+    Z = np.full(len(P), 18, dtype=np.int64)
+    M = np.full(len(P), 39.95, dtype=np.float32)
+    mask = torch.tensor([True, False, True, True, False], device=DEV)
+    node = mask[torch.repeat_interleave(torch.arange(5, device=DEV), torch.as_tensor(np.diff(ptr), device=DEV))]
+
+    class PlainNVE(NVE):
+        _honors_active_mask = False  # forces the save-and-restore route
+
+    for cls in (NVE, PlainNVE):
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=3.0, cutoff=6.0)
+        full, part, halves = (make_batch(P, Z, M, C, pb, ptr, V=V) for _ in range(3))
+        for b in (full, part, halves):
+            b.forces.copy_(torch.from_numpy(F))
+        dyn = cls(model, dt=1.0)
+        dyn.masked_update(full, torch.ones(5, dtype=torch.bool, device=DEV))
+        dyn.masked_update(part, mask)
+        dyn._masked_pre_update(halves, mask)
+        dyn._masked_post_update(halves, mask)
+        p0, v0 = torch.from_numpy(P).to(DEV), torch.from_numpy(V).to(DEV)
+        for b in (part, halves):
+            assert torch.equal(b.positions[node], full.positions[node]) and torch.equal(b.velocities[node], full.velocities[node])
+            assert torch.equal(b.positions[~node], p0[~node]) and torch.equal(b.velocities[~node], v0[~node])
+        assert not torch.equal(full.positions[~node], p0[~node])
