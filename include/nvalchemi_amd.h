@@ -290,6 +290,29 @@ int32_t nvamd_defrag_segmented(void* source, int32_t* source_batch_ptr,
                                int32_t num_systems, int32_t total_rows, int64_t row_bytes,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Filtering an existing list down to a tighter cutoff: the Torch code of
+ * nvalchemi/models/_ops/neighbor_filter.py (filter_neighbor_matrix :43-144; the distance test of
+ * filter_neighbor_list :147-224), used by prepare_neighbors_for_model (:286-430) when a model's
+ * cutoff is below the one the list was built with.  cells: (3,3) for all atoms
+ * (per_system_cells = 0) or (B,3,3) looked up through batch_idx (= 1); cells or shifts NULL: no
+ * shift is applied (shifts are still carried along).  The distance is evaluated in double on the
+ * float32 inputs (the reference: float32), strict <.
+ * nvamd_nl_filter_matrix: every slot with an index below fill_value and inside the cutoff is kept;
+ * kept entries move to the front of their row in order, the rest of the row becomes fill_value /
+ * zero shifts, out_num_neighbors (N) = number kept.  Outputs must not alias the inputs.
+ * nvamd_nl_filter_coo_flags: keep (E) bytes = 1 where edge e = (neighbor_list[e,0], [e,1]) is
+ * inside the cutoff. */
+int32_t nvamd_nl_filter_matrix(const float* positions, const float* cells, int32_t per_system_cells,
+                               const int32_t* neighbor_matrix, const int32_t* neighbor_matrix_shifts,
+                               const int32_t* batch_idx, int32_t n_atoms, int32_t max_neighbors,
+                               int32_t fill_value, double cutoff, int32_t* out_neighbor_matrix,
+                               int32_t* out_num_neighbors, int32_t* out_shifts, void* stream);
+int32_t nvamd_nl_filter_coo_flags(const float* positions, const float* cells, int32_t per_system_cells,
+                                  const int32_t* neighbor_list, const int32_t* neighbor_list_shifts,
+                                  const int32_t* batch_idx, int64_t n_edges, double cutoff,
+                                  uint8_t* keep, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,6 +48,8 @@ _SIGNATURES = {
     "nvamd_kinetic_energy": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_nl_filter_matrix": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _f64, _vp, _vp, _vp, _vp]),
+    "nvamd_nl_filter_coo_flags": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _c.c_int64, _f64, _vp, _vp]),
     "nvamd_buffer_workspace_bytes": (_i32, [_c.c_int64, _c.c_int64, _c.POINTER(_c.c_size_t)]),
     "nvamd_put_masked_per_system": (_i32, [_vp] * 5 + [_i32, _i32, _c.c_int64, _vp, _c.c_size_t, _vp]),
     "nvamd_put_fit_mask_per_system": (_i32, [_vp] * 3 + [_i32, _i32, _vp, _c.c_size_t, _vp]),
@@ -461,3 +463,39 @@ def defrag_segmented(source, source_batch_ptr, source_data_copied, num_kept) -> 
         sp, _dev(source_batch_ptr, "source_batch_ptr", torch.int32, (n + 1,)),
         _mask(source_data_copied, "source_data_copied", n), _dev(num_kept, "num_kept", torch.int32, (1,)),
         n, rows, rb, ws.data_ptr(), ws.numel(), _stream(source.device)), "nvamd_defrag_segmented")
+
+
+# --------------------------------------------------------------------------------------------
+# filtering a list to a tighter cutoff
+# --------------------------------------------------------------------------------------------
+def _cells_arg(cell, n_systems_hint=None):
+    if cell is None:
+        return None, 0
+    if cell.dim() == 2:
+        return _dev(cell, "cell", torch.float32, (3, 3)), 0
+    return _dev(cell, "cell", torch.float32, (None, 3, 3)), 1
+
+
+def nl_filter_matrix(positions, cell, neighbor_matrix, neighbor_matrix_shifts, batch_idx, fill_value: int,
+                     cutoff: float, out_matrix, out_counts, out_shifts) -> None:
+    N, K = neighbor_matrix.shape
+    cp, per_system = _cells_arg(cell)
+    _check(library().nvamd_nl_filter_matrix(
+        _dev(positions, "positions", torch.float32, (N, 3)), cp, per_system,
+        _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+        _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+        _opt(batch_idx, "batch_idx", torch.int32, (N,)), N, K, int(fill_value), float(cutoff),
+        _dev(out_matrix, "out_matrix", torch.int32, (N, K)), _dev(out_counts, "out_counts", torch.int32, (N,)),
+        _opt(out_shifts, "out_shifts", torch.int32, (N, K, 3)), _stream(positions.device)), "nvamd_nl_filter_matrix")
+
+
+def nl_filter_coo_flags(positions, cell, neighbor_list, neighbor_list_shifts, batch_idx, cutoff: float, keep) -> None:
+    N = positions.shape[0]
+    E = neighbor_list.shape[0]
+    cp, per_system = _cells_arg(cell)
+    _check(library().nvamd_nl_filter_coo_flags(
+        _dev(positions, "positions", torch.float32, (N, 3)), cp, per_system,
+        _dev(neighbor_list, "neighbor_list", torch.int32, (E, 2)),
+        _opt(neighbor_list_shifts, "neighbor_list_shifts", torch.int32, (E, 3)),
+        _opt(batch_idx, "batch_idx", torch.int32, (N,)), E, float(cutoff),
+        _dev(_as_u8(keep), "keep", torch.uint8, (E,)), _stream(positions.device)), "nvamd_nl_filter_coo_flags")

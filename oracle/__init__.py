@@ -426,3 +426,84 @@ def defrag_segmented(source, source_batch_ptr, source_data_copied):
     source_batch_ptr[: num_kept + 1] = np.concatenate([[0], np.cumsum(lengths)]) if num_kept else [0]
     source_batch_ptr[num_kept + 1:] = total
     return num_kept
+
+
+# ---------------------------------------------------------------------------------------------
+# filtering a list to a tighter cutoff (numpy restatement of the in-tree Torch code,
+# nvalchemi/models/_ops/neighbor_filter.py:43-283, with the distance in double on the float32
+# inputs as everywhere in this library; pinned by the reference's own cases,
+# test/models/test_neighbor_filter.py:49-760, restated in tests/test_oracle_filter.py)
+# ---------------------------------------------------------------------------------------------
+def _filter_d2(pos_i, pos_j, shifts, cells):
+    d = pos_j.astype(np.float64) - pos_i.astype(np.float64)
+    if shifts is not None and cells is not None:
+        s = shifts.astype(np.float64)
+        h = cells.astype(np.float64)
+        # (S0 a0 + S1 a1) + S2 a2 per component, as orc_pair_d2 does
+        t = (s[..., 0:1] * h[..., 0, :] + s[..., 1:2] * h[..., 1, :]) + s[..., 2:3] * h[..., 2, :]
+        d = d + t
+    return (d[..., 0] * d[..., 0] + d[..., 1] * d[..., 1]) + d[..., 2] * d[..., 2]
+
+
+def filter_neighbor_matrix(positions, cutoff, neighbor_matrix, num_neighbors, fill_value, cell=None,
+                           neighbor_matrix_shifts=None, batch_idx=None):
+    """neighbor_filter.py:43-144 -> (matrix, counts, shifts | None)"""
+    pos = _f32(positions)
+    nm = _i32(neighbor_matrix)
+    N, K = nm.shape
+    valid = nm < fill_value
+    j = np.clip(nm, 0, max(N - 1, 0))
+    cells = None
+    if cell is not None and neighbor_matrix_shifts is not None:
+        c = _f32(cell)
+        if c.ndim == 2:
+            cells = np.broadcast_to(c, (N, 1, 3, 3))
+        else:
+            if batch_idx is None:
+                raise ValueError("batch_idx is required when cell has shape (B, 3, 3).")
+            cells = c[_i32(batch_idx)][:, None]
+    d2 = _filter_d2(pos[:, None, :], pos[j], None if cells is None else _i32(neighbor_matrix_shifts), cells)
+    keep = valid & (d2 < float(cutoff) * float(cutoff))
+    order = np.argsort(~keep, axis=1, kind="stable")
+    keep_sorted = np.take_along_axis(keep, order, 1)
+    out_nm = np.where(keep_sorted, np.take_along_axis(nm, order, 1), fill_value).astype(np.int32)
+    out_nn = keep.sum(1).astype(np.asarray(num_neighbors).dtype)
+    out_sh = None
+    if neighbor_matrix_shifts is not None:
+        sh = np.take_along_axis(_i32(neighbor_matrix_shifts), order[..., None], 1)
+        out_sh = np.where(keep_sorted[..., None], sh, 0).astype(np.int32)
+    return out_nm, out_nn, out_sh
+
+
+def filter_neighbor_list(positions, cutoff, neighbor_list, neighbor_ptr, cell=None, neighbor_list_shifts=None,
+                         batch_idx=None):
+    """neighbor_filter.py:147-224 -> (edges, ptr, shifts | None)"""
+    pos = _f32(positions)
+    nl = _i32(neighbor_list)
+    N = pos.shape[0]
+    i, j = nl[:, 0], nl[:, 1]
+    cells = None
+    if cell is not None and neighbor_list_shifts is not None:
+        c = _f32(cell)
+        if c.ndim == 2:
+            cells = np.broadcast_to(c, (len(i), 3, 3))
+        else:
+            if batch_idx is None:
+                raise ValueError("batch_idx is required when cell has shape (B, 3, 3).")
+            cells = c[_i32(batch_idx)[i]]
+    d2 = _filter_d2(pos[i], pos[j], None if cells is None else _i32(neighbor_list_shifts), cells)
+    keep = d2 < float(cutoff) * float(cutoff)
+    ptr = np.zeros(N + 1, dtype=np.asarray(neighbor_ptr).dtype)
+    ptr[1:] = np.cumsum(np.bincount(i[keep], minlength=N))
+    return nl[keep], ptr, None if neighbor_list_shifts is None else _i32(neighbor_list_shifts)[keep]
+
+
+def neighbor_matrix_to_list(neighbor_matrix, num_neighbors, fill_value, neighbor_matrix_shifts=None):
+    """neighbor_filter.py:227-283 -> (edges (M,2), ptr (N+1), shifts | None)"""
+    nm = _i32(neighbor_matrix)
+    N, K = nm.shape
+    ii, kk = np.nonzero(nm < fill_value)
+    nl = np.stack([ii.astype(np.int32), nm[ii, kk]], axis=1)
+    ptr = np.zeros(N + 1, dtype=np.int32)
+    ptr[1:] = np.cumsum(_i32(num_neighbors))
+    return nl, ptr, None if neighbor_matrix_shifts is None else _i32(neighbor_matrix_shifts)[ii, kk]
