@@ -199,17 +199,23 @@ def main() -> int:
     stages = {}
     if timer:
         ms = timer.mean_ms()
-        # the pair kernel derives shifts from positions in cells wider than twice the search radius
-        # (this workload's are): it then reads the 4-byte index of a pair, not its 12-byte shift
+        # Algorithmic bytes are the compulsory traffic at the API's own I/O layout: a pair is its
+        # 4-byte index and its 12-byte shift.  The pair kernel derives shifts from positions in
+        # cells wider than twice the search radius (this workload's are) and then does not read
+        # them: the bytes it still has to touch are reported beside the API-level figure.
         stamp = getattr(batch, "_neighbor_search_cutoff", None)
         widths = 1.0 / torch.linalg.inv(batch.cell.double()).norm(dim=1)
         shifts_derived = bool(stamp) and bool((widths > 2.0002 * stamp[0]).all())
-        alg = {"nl": 20 * N + 16 * E, "lj": 36 * N + (4 if shifts_derived else 16) * E + 4 * B,
-               "vv_pre": 68 * N, "vv_post": 44 * N}
+        alg = {"nl": 20 * N + 16 * E, "lj": 36 * N + 16 * E + 4 * B, "vv_pre": 68 * N, "vv_post": 44 * N}
         for k, b in alg.items():
             gbps = b / (ms[k] * 1e-3) / 1e9
             stages[k] = {"ms": round(ms[k], 4), "alg_bytes": b, "GBps": round(gbps, 1),
                          "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+        if shifts_derived:
+            touched = 36 * N + 4 * E + 4 * B
+            stages["lj"]["shifts_derived_not_read"] = True
+            stages["lj"]["bytes_it_must_touch"] = touched
+            stages["lj"]["GBps_touched"] = round(touched / (ms["lj"] * 1e-3) / 1e9, 1)
         log("[bench] stage ms: " + ", ".join(f"{k}={v['ms']}" for k, v in stages.items())
             + f"; sum={sum(v['ms'] for v in stages.values()):.3f} vs wall/step={ms_per_step:.3f}")
     result = {
