@@ -1,5 +1,5 @@
-from .base import BaseDynamics, ConvergenceHook, DynamicsStage
+from .base import BaseDynamics, ConvergenceHook, DynamicsStage, FusedStage
 from .integrators.nve import NVE
 from .optimizers.fire import FIRE
 
-__all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "NVE", "FIRE"]
+__all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "FusedStage", "NVE", "FIRE"]

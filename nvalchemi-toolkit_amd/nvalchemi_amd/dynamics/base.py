@@ -189,6 +189,11 @@ class BaseDynamics(HookRegistryMixin):
     __provides_keys__: set[str] = set()
     _mutable_fields: tuple[str, ...] = ("positions", "velocities", "cell")
     _honors_active_mask: bool = False
+    #: graph-level fields that travel with a system (nvalchemi/dynamics/base.py:1336-1362)
+    _bookkeeping_keys: dict[str, Callable[[int, torch.device], torch.Tensor]] = {
+        "status": lambda n, dev: torch.zeros(n, 1, dtype=torch.long, device=dev),
+        "system_id": lambda n, dev: torch.full((n, 1), -1, dtype=torch.long, device=dev),
+    }
     _OUTPUT_KEY_TO_BATCH_ATTR: dict[str, str] = {"energy": "energy", "forces": "forces", "stress": "stress"}
 
     def __init__(self, model: BaseModelMixin, hooks: list | None = None, convergence_hook: Any = None,
@@ -211,6 +216,20 @@ class BaseDynamics(HookRegistryMixin):
         self._last_converged: torch.Tensor | None = None
         self._last_outputs: OrderedDict | None = None
         self._active_mask: torch.Tensor | None = None
+
+    @classmethod
+    def register_bookkeeping_key(cls, key: str, init_fn: Callable[[int, torch.device], torch.Tensor]) -> None:
+        """Register a graph-level field (``init_fn(n, device) -> (n, 1)`` tensor) that a fused stage
+        creates on the batch when it is absent."""
+        cls._bookkeeping_keys = {**cls._bookkeeping_keys, key: init_fn}
+
+    def __add__(self, other: "BaseDynamics") -> "FusedStage":
+        """``dyn_a + dyn_b``: a :class:`FusedStage` with status codes 0 and 1
+        (nvalchemi/dynamics/base.py:1210-1243)."""
+        if not isinstance(other, BaseDynamics):
+            raise TypeError("Both operands of + must be BaseDynamics instances. "
+                            f"other is {type(other).__name__}, not BaseDynamics.")
+        return FusedStage(sub_stages=[(0, self), (1, other)])
 
     # ---- hooks ---------------------------------------------------------------------------------
     def _call_hooks(self, stage: DynamicsStage, batch) -> None:
@@ -425,3 +444,241 @@ class BaseDynamics(HookRegistryMixin):
         return (f"{type(self).__name__}(model={type(self.model).__name__}, n_steps={self.n_steps}, "
                 f"step_count={self.step_count}, convergence_hook={self.convergence_hook!r}, "
                 f"hooks={len(self.hooks)})")
+
+
+class FusedStage(BaseDynamics):
+    """Several dynamics on one batch with one model evaluation per step: each sub-stage updates the
+    systems whose ``batch.status`` equals its code, convergence (or a per-system step budget,
+    ``n_steps`` of the sub-stage) moves a system on to the next code, ``exit_status`` (default: the
+    number of sub-stages) means done.  Mirror of nvalchemi/dynamics/base.py:2504-3337 for a batch
+    supplied by the caller; in-flight refill from a sampler and ``torch.compile`` of the step are
+    not available here.
+
+    One step (``_step_impl``, :2928-3079): BEFORE_STEP hooks; per sub-stage BEFORE_PRE_UPDATE and the
+    masked ``pre_update``; BEFORE_COMPUTE hooks of this stage (the neighbor list at the new
+    positions), one ``compute``, AFTER_COMPUTE; per sub-stage the masked ``post_update`` and
+    AFTER_POST_UPDATE; AFTER_STEP hooks (the convergence hooks migrate statuses there); step-budget
+    migration; ON_CONVERGE per sub-stage; counters.  Returns the indices of the systems that reached
+    ``exit_status`` during the step, or ``None``.  As in the reference, a sub-stage's step budget is
+    counted on the status after the migrations of the step (:3023-3028): the step in which a system
+    arrives in a sub-stage already counts towards that sub-stage's ``n_steps``.
+    """
+
+    def __init__(self, sub_stages: list[tuple[int, BaseDynamics]], *, entry_status: int = 0, exit_status: int = -1,
+                 compile_step: bool = False, compile_kwargs: dict[str, Any] | None = None,
+                 init_fn: Callable | None = None, **kwargs: Any) -> None:
+        if compile_step:
+            raise NotImplementedError("FusedStage(compile_step=True): the step is not compiled in this build")
+        if not sub_stages:
+            raise ValueError("FusedStage needs at least one sub-stage")
+        super().__init__(model=sub_stages[0][1].model, **kwargs)
+        self.sub_stages = list(sub_stages)
+        self.__needs_keys__ = set().union(*(dyn.__needs_keys__ for _, dyn in sub_stages))
+        self.__provides_keys__ = set().union(*(dyn.__provides_keys__ for _, dyn in sub_stages))
+        self.entry_status = entry_status
+        self.compile_kwargs = compile_kwargs if compile_kwargs is not None else {}
+        self.compile_step = False
+        self.exit_status = len(self.sub_stages) if exit_status == -1 else exit_status
+        self.convergence_check_frequency = 1
+        self.init_fn = init_fn
+        self.fused_hooks: list = []
+        # every sub-stage gets the convergence hook that moves its systems to the next code
+        for i, (source_code, source) in enumerate(self.sub_stages):
+            if i + 1 < len(self.sub_stages):
+                target_code = self.sub_stages[i + 1][0]
+            else:
+                if source.convergence_hook is None:
+                    continue
+                target_code = self.exit_status
+            source.hooks = [h for h in source.hooks
+                            if not (isinstance(h, ConvergenceHook) and getattr(h, "source_status", None) == source_code
+                                    and getattr(h, "target_status", None) == target_code)]
+            criteria = source.convergence_hook.criteria if source.convergence_hook is not None else None
+            source.register_hook(ConvergenceHook(criteria=criteria, source_status=source_code,
+                                                 target_status=target_code))
+        for code, dyn in self.sub_stages:
+            if dyn.n_steps is not None:
+                BaseDynamics.register_bookkeeping_key(
+                    f"n_steps_counter_{code}", lambda n, dev: torch.zeros(n, 1, dtype=torch.long, device=dev))
+
+    def __repr__(self) -> str:
+        stages = ", ".join(f"{code}:{type(dyn).__name__}" for code, dyn in self.sub_stages)
+        return (f"FusedStage(sub_stages=[{stages}], entry_status={self.entry_status}, "
+                f"exit_status={self.exit_status}, compiled=False, step_count={self.step_count})")
+
+    def __add__(self, other: BaseDynamics) -> "FusedStage":
+        if not isinstance(other, BaseDynamics):
+            raise TypeError("Cannot append stage: other must be a BaseDynamics instance. "
+                            f"Got {type(other).__name__} instead.")
+        return FusedStage(sub_stages=list(self.sub_stages) + [(len(self.sub_stages), other)],
+                          entry_status=self.entry_status, compile_kwargs=self.compile_kwargs)
+
+    # ---- hooks ---------------------------------------------------------------------------------
+    def register_fused_hook(self, hook) -> None:
+        """A hook that sees the whole batch at this stage's BEFORE_STEP / AFTER_STEP."""
+        if not isinstance(hook.frequency, int) or hook.frequency < 1:
+            raise ValueError(f"Hook {hook!r} has frequency={hook.frequency!r}. "
+                             "frequency must be a positive integer (>= 1).")
+        self.fused_hooks.append(hook)
+
+    def _call_fused_hooks(self, stage: DynamicsStage, batch) -> None:
+        ctx = self._build_context(batch)
+        for hook in self.fused_hooks:
+            runs_on_stage = getattr(hook, "_runs_on_stage", None)
+            if runs_on_stage is not None:
+                if not runs_on_stage(stage):
+                    continue
+            elif stage != hook.stage:
+                continue
+            if self.step_count % hook.frequency == 0:
+                hook(ctx, stage)
+
+    def _open_hooks(self) -> None:
+        super()._open_hooks()
+        seen: set[int] = set()
+        for hook in self.fused_hooks:
+            if id(hook) not in seen and hasattr(hook, "__enter__"):
+                seen.add(id(hook))
+                hook.__enter__()
+        for _, dyn in self.sub_stages:
+            dyn._open_hooks()
+
+    def _close_hooks(self) -> None:
+        super()._close_hooks()
+        seen: set[int] = set()
+        for hook in self.fused_hooks:
+            if id(hook) in seen:
+                continue
+            seen.add(id(hook))
+            if hasattr(hook, "__exit__"):
+                hook.__exit__(None, None, None)
+            elif hasattr(hook, "close"):
+                hook.close()
+        for _, dyn in self.sub_stages:
+            dyn._close_hooks()
+
+    def _ensure_bookkeeping_fields(self, batch) -> None:
+        for key, default_fn in self._bookkeeping_keys.items():
+            if getattr(batch, key, None) is None:
+                batch[key] = default_fn(batch.num_graphs, batch.device)
+
+    # ---- the step ------------------------------------------------------------------------------
+    @staticmethod
+    def _flat_status(batch) -> torch.Tensor:
+        status = batch.status
+        return status.squeeze(-1) if status.dim() == 2 else status
+
+    def _step_impl(self, batch):
+        self._ensure_bookkeeping_fields(batch)
+        self._call_fused_hooks(DynamicsStage.BEFORE_STEP, batch)
+        self._call_hooks(DynamicsStage.BEFORE_STEP, batch)
+        for _, dyn in self.sub_stages:
+            dyn._call_hooks(DynamicsStage.BEFORE_STEP, batch)
+
+        status = self._flat_status(batch)
+        masks: list[torch.Tensor] = []
+        for code, dyn in self.sub_stages:
+            mask = status == code
+            masks.append(mask)
+            dyn._call_hooks(DynamicsStage.BEFORE_PRE_UPDATE, batch)
+            if mask.any():
+                dyn._masked_pre_update(batch, mask)
+
+        self._call_hooks(DynamicsStage.BEFORE_COMPUTE, batch)
+        outputs = self.compute(batch)
+        for key, tensor in outputs.items():
+            if key not in ("forces", "energy"):
+                batch[key] = tensor
+        self._call_hooks(DynamicsStage.AFTER_COMPUTE, batch)
+        for _, dyn in self.sub_stages:
+            dyn._call_hooks(DynamicsStage.AFTER_COMPUTE, batch)
+
+        for (code, dyn), mask in zip(self.sub_stages, masks):
+            if mask.any():
+                dyn._masked_post_update(batch, mask)
+            dyn._call_hooks(DynamicsStage.AFTER_POST_UPDATE, batch)
+
+        before = self._flat_status(batch).clone()
+        for _, dyn in self.sub_stages:
+            dyn._call_hooks(DynamicsStage.AFTER_STEP, batch)
+        self._call_hooks(DynamicsStage.AFTER_STEP, batch)
+        self._call_fused_hooks(DynamicsStage.AFTER_STEP, batch)
+
+        # per-system step budgets of the sub-stages
+        for i, (code, dyn) in enumerate(self.sub_stages):
+            if dyn.n_steps is None:
+                continue
+            key = f"n_steps_counter_{code}"
+            if getattr(batch, key, None) is None:
+                batch[key] = torch.zeros(batch.num_graphs, 1, dtype=torch.long, device=batch.device)
+            counter = getattr(batch, key)
+            active = self._flat_status(batch) == code
+            counter[active] += 1
+            next_code = self.sub_stages[i + 1][0] if i + 1 < len(self.sub_stages) else self.exit_status
+            migrate = active & (counter.squeeze(-1) >= dyn.n_steps)
+            if migrate.any():
+                batch.status.view(-1)[migrate] = next_code
+                counter[migrate] = 0
+
+        for mask, (_, dyn) in zip(masks, self.sub_stages):
+            converged = dyn._check_convergence(batch)
+            dyn._last_converged = None
+            if converged is None:
+                continue
+            here = torch.zeros(batch.num_graphs, dtype=torch.bool, device=batch.device)
+            here[converged] = True
+            here &= mask
+            if not here.any():
+                continue
+            dyn._last_converged = torch.where(here)[0]
+            dyn._call_hooks(DynamicsStage.ON_CONVERGE, batch)
+
+        self.step_count += 1
+        for _, dyn in self.sub_stages:
+            dyn.step_count += 1
+        after = self._flat_status(batch)
+        graduated = (before < self.exit_status) & (after >= self.exit_status)
+        return batch, (torch.where(graduated)[0] if graduated.any() else None)
+
+    def step(self, batch):
+        return self._step_impl(batch)
+
+    def __call__(self, batch):
+        return self.step(batch)
+
+    @staticmethod
+    def all_complete(batch, exit_status: int) -> bool:
+        status = getattr(batch, "status", None)
+        if status is None:
+            return False
+        if status.dim() == 2:
+            status = status.squeeze(-1)
+        return bool((status == exit_status).all())
+
+    def run(self, batch=None, n_steps: int | None = None):
+        """Evaluate the model once (the first step integrates with real forces), then step until
+        every system has ``exit_status`` or ``n_steps`` steps are done
+        (nvalchemi/dynamics/base.py:3162-3265, the mode with a batch supplied by the caller)."""
+        if batch is None:
+            if self.sampler is None:
+                raise ValueError("No batch provided and no sampler configured.")
+            raise NotImplementedError("in-flight batching from a sampler is not available in this build")
+        self._ensure_bookkeeping_fields(batch)
+        resolved = n_steps if n_steps is not None else self.n_steps
+        self._open_hooks()
+        try:
+            self._call_hooks(DynamicsStage.BEFORE_COMPUTE, batch)
+            self.compute(batch)
+            self._call_hooks(DynamicsStage.AFTER_COMPUTE, batch)
+            step_num = 0
+            while True:
+                batch, _ = self.step(batch)
+                if (step_num + 1) % self.convergence_check_frequency == 0 \
+                        and self.all_complete(batch, self.exit_status):
+                    break
+                step_num += 1
+                if resolved is not None and step_num >= resolved:
+                    break
+            return batch
+        finally:
+            self._close_hooks()

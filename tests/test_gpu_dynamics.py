@@ -376,3 +376,85 @@ def test_masked_update_moves_only_the_selected_systems():
             assert torch.equal(b.positions[node], full.positions[node]) and torch.equal(b.velocities[node], full.velocities[node])
             assert torch.equal(b.positions[~node], p0[~node]) and torch.equal(b.velocities[~node], v0[~node])
         assert not torch.equal(full.positions[~node], p0[~node])
+
+
+def test_fused_stage_relax_then_md_equals_each_system_on_its_own():
+    """``FIRE + NVE`` as one ``FusedStage`` (nvalchemi/dynamics/base.py:2504-3337): every system
+    relaxes until its forces fall below the threshold, then runs its budget of MD steps, then
+    rests.  Systems do not interact, so the fused batch must reproduce each system taken through
+    the same two dynamics alone."""
+    from nvalchemi_amd.dynamics import FIRE, NVE, ConvergenceHook, FusedStage
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=5, n_boxes=4, reps=3, a=5.4, jitter=0.0)
+    rng = np.random.default_rng(3)
+    for s, amp in enumerate((0.02, 0.10, 0.25, 0.05)):  # different distances from the minimum
+        P[ptr[s]:ptr[s + 1]] += rng.normal(0, amp, (ptr[s + 1] - ptr[s], 3)).astype(np.float32)
+    Z = np.full(len(P), 18, dtype=np.int64)
+    M = np.full(len(P), 39.95, dtype=np.float32)
+    tol, md_steps, cap = 0.02, 5, 400
+
+    def dynamics():
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+        relax = FIRE(model, dt=1.0, convergence_hook=ConvergenceHook.from_fmax(tol))
+        md = NVE(model, dt=2.0, n_steps=md_steps)
+        return model, relax, md
+
+    model, relax, md = dynamics()
+    fused = relax + md
+    assert isinstance(fused, FusedStage) and fused.exit_status == 2 and [c for c, _ in fused.sub_stages] == [0, 1]
+    for h in model.make_neighbor_hooks():
+        fused.register_hook(h)
+    batch = make_batch(P, Z, M, C, pb, ptr, V=np.zeros_like(P))
+    graduated_at = {}
+    fused._ensure_bookkeeping_fields(batch)
+    fused._call_hooks(fused._stage_type.BEFORE_COMPUTE, batch)
+    fused.compute(batch)
+    for step in range(cap):
+        batch, done = fused.step(batch)
+        if done is not None:
+            for s in done.tolist():
+                graduated_at[s] = step
+        if FusedStage.all_complete(batch, fused.exit_status):
+            break
+    assert sorted(graduated_at) == [0, 1, 2, 3] and len(set(graduated_at.values())) > 1
+    assert batch.status.view(-1).tolist() == [2, 2, 2, 2]
+
+    for s in range(4):
+        a0, a1 = int(ptr[s]), int(ptr[s + 1])
+        one_ptr = np.array([0, a1 - a0], dtype=np.int32)
+        model, relax, md = dynamics()
+        b = make_batch(P[a0:a1], Z[a0:a1], M[a0:a1], C[s:s + 1], pb[s:s + 1], one_ptr, V=np.zeros((a1 - a0, 3), np.float32))
+        hooks = model.make_neighbor_hooks()
+        for h in hooks:
+            relax.register_hook(h)
+            md.register_hook(h)
+        relax._call_hooks(relax._stage_type.BEFORE_COMPUTE, b)
+        relax.compute(b)
+        steps = 0
+        while True:
+            _, conv = relax.step(b)
+            steps += 1
+            if conv is not None:
+                break
+            assert steps < cap
+        # the step budget of a sub-stage counts the step in which a system arrives
+        # (nvalchemi/dynamics/base.py:3023-3028 reads the status after the migration)
+        for _ in range(md_steps - 1):
+            md.step(b)
+        assert graduated_at[s] == steps + md_steps - 2, (s, graduated_at[s], steps)
+        close(batch.positions[a0:a1], b.positions.cpu().numpy(), f"positions of system {s}")
+        close(batch.velocities[a0:a1], b.velocities.cpu().numpy(), f"velocities of system {s}")
+
+    # run(): the same through the loop of the class, and a finished batch stays put
+    model, relax, md = dynamics()
+    fused2 = FusedStage([(0, relax), (1, md)], hooks=model.make_neighbor_hooks())
+    batch2 = fused2.run(make_batch(P, Z, M, C, pb, ptr, V=np.zeros_like(P)), n_steps=cap)
+    assert torch.equal(batch2.positions, batch.positions) and torch.equal(batch2.velocities, batch.velocities)
+    frozen = batch2.positions.clone()
+    fused2.step(batch2)
+    assert torch.equal(batch2.positions, frozen)
+    with pytest.raises(ValueError):
+        fused2.run(None)
+    with pytest.raises(TypeError):
+        fused2 + 3
