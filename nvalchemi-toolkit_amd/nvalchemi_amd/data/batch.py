@@ -79,6 +79,39 @@ class SegmentedGroup:
     def items(self):
         return self._tensors.items()
 
+    def select(self, idx: list[int]) -> "SegmentedGroup":
+        """The segments ``idx`` (any order, repeats allowed) as a new group: one gather per tensor
+        through an element index built from the boundaries."""
+        lengths_host = self.lengths_list()
+        new_lengths = [lengths_host[i] for i in idx]
+        total = sum(new_lengths)
+        sel = torch.tensor(idx, dtype=torch.long, device=self.device)
+        lens = self.segment_lengths[sel].to(torch.long)
+        starts = self.batch_ptr[sel].to(torch.long)
+        new_starts = torch.cumsum(lens, 0) - lens
+        rows = torch.repeat_interleave(starts - new_starts, lens, output_size=total) \
+            + torch.arange(total, dtype=torch.long, device=self.device)
+        out = SegmentedGroup({k: v.index_select(0, rows) for k, v in self._tensors.items()},
+                             torch.tensor(new_lengths, dtype=torch.int32), self.device)
+        out._lengths_host = new_lengths
+        return out
+
+    def concatenate(self, other: "SegmentedGroup") -> None:
+        """Append the segments of ``other`` in place; keys that only one side has are dropped
+        (derived data such as a neighbor matrix cannot be carried over a change of the batch)."""
+        common = [k for k in self._tensors if k in other._tensors]
+        self._tensors = {k: torch.cat([self._tensors[k], other._tensors[k].to(self.device)], 0) for k in common}
+        self.segment_lengths = torch.cat([self.segment_lengths, other.segment_lengths.to(self.device)])
+        self._batch_idx = self._batch_ptr = self._lengths_host = None
+        if hasattr(self, "_edge_ptr"):
+            del self._edge_ptr
+
+    def extend_for_appended_graphs(self, n: int) -> None:
+        """``n`` more systems without elements."""
+        self.segment_lengths = torch.cat([self.segment_lengths,
+                                          torch.zeros(n, dtype=torch.int32, device=self.device)])
+        self._batch_idx = self._batch_ptr = self._lengths_host = None
+
 
 class UniformGroup:
     """Tensors with exactly one leading row per system."""
@@ -109,6 +142,21 @@ class UniformGroup:
     def items(self):
         return self._tensors.items()
 
+    def select(self, idx: list[int]) -> "UniformGroup":
+        sel = torch.tensor(idx, dtype=torch.long, device=self.device)
+        return UniformGroup({k: v.index_select(0, sel) for k, v in self._tensors.items()}, len(idx), self.device)
+
+    def concatenate(self, other: "UniformGroup") -> None:
+        common = [k for k in self._tensors if k in other._tensors]
+        self._tensors = {k: torch.cat([self._tensors[k], other._tensors[k].to(self.device)], 0) for k in common}
+        self._n += len(other)
+
+    def extend_for_appended_graphs(self, n: int) -> None:
+        """``n`` more systems with zero rows (the other batch has no such group)."""
+        self._tensors = {k: torch.cat([v, torch.zeros((n,) + tuple(v.shape[1:]), dtype=v.dtype, device=v.device)], 0)
+                         for k, v in self._tensors.items()}
+        self._n += n
+
 
 class _Storage:
     def __init__(self, groups: dict[str, Any]) -> None:
@@ -123,7 +171,8 @@ class _Storage:
 
 
 _GROUP_ORDER = ("atoms", "edges", "system")
-_RESERVED = {"_storage", "device", "_neighbor_list_cutoff", "_neighbor_row_order", "_neighbor_search_cutoff"}
+_RESERVED = {"_storage", "device", "_neighbor_list_cutoff", "_neighbor_row_order", "_neighbor_search_cutoff",
+             "_copied_mask"}
 
 
 class Batch:
@@ -277,11 +326,106 @@ class Batch:
             return
         self[name] = value
 
-    def __getitem__(self, key: str) -> torch.Tensor:
+    def __getitem__(self, key):
+        """A tensor by key name, or -- for an int, slice, list or tensor -- the selected systems
+        (an ``AtomicData`` for an int, a ``Batch`` otherwise)."""
+        if not isinstance(key, str):
+            if isinstance(key, int):
+                return self.get_data(key if key >= 0 else self.num_graphs + key)
+            return self.index_select(key)
         g = self._find(key)
         if g is None:
             raise KeyError(key)
         return g[key]
+
+    # ---- selection and growth (nvalchemi/data/batch.py:816-874, 987-1072, 1138-1178) -----------
+    def _normalize_index(self, idx) -> list[int]:
+        import numpy as np
+
+        if isinstance(idx, bool):
+            raise IndexError("Unsupported index type: bool")
+        if isinstance(idx, int):
+            result = [idx]
+        elif isinstance(idx, slice):
+            result = list(range(self.num_graphs)[idx])
+        elif isinstance(idx, torch.Tensor):
+            if idx.dtype == torch.bool:
+                result = idx.flatten().nonzero(as_tuple=False).flatten().tolist()
+            elif idx.dtype.is_floating_point:
+                raise IndexError(f"Tensor index must be integer or bool, got {idx.dtype}")
+            else:
+                result = idx.flatten().tolist()
+        elif isinstance(idx, np.ndarray):
+            result = (idx.flatten().nonzero()[0] if idx.dtype == np.bool_ else idx.flatten()).tolist()
+        elif isinstance(idx, (list, tuple, range)):
+            result = list(idx)
+        else:
+            raise IndexError(f"Unsupported index type: {type(idx).__name__}")
+        if not result:
+            raise IndexError("Index is empty")
+        n = self.num_graphs
+        result = [n + i if i < 0 else i for i in result]
+        if any(i < 0 or i >= n for i in result):
+            raise IndexError(f"graph index out of range for a batch of {n}")
+        return result
+
+    def index_select(self, idx) -> "Batch":
+        """The systems ``idx`` as a new batch, gathered from the concatenated tensors; the atom
+        indices of ``neighbor_list`` are re-based.  Keys that hold global atom indices by value
+        (a neighbor matrix) are carried as they are and must be rebuilt, as in the reference."""
+        ids = self._normalize_index(idx)
+        groups: dict[str, Any] = {}
+        atoms = self._atoms_group
+        offset_diff = None
+        if atoms is not None:
+            new_atoms = atoms.select(ids)
+            sel = torch.tensor(ids, dtype=torch.long, device=self.device)
+            offset_diff = atoms.batch_ptr[sel] - new_atoms.batch_ptr[:-1]
+            groups["atoms"] = new_atoms
+        edges = self._edges_group
+        if edges is not None:
+            new_edges = edges.select(ids)
+            if "neighbor_list" in new_edges and offset_diff is not None:
+                corr = offset_diff[new_edges.batch_idx.to(torch.long)]
+                new_edges["neighbor_list"] = new_edges["neighbor_list"] - corr.unsqueeze(1).to(
+                    new_edges["neighbor_list"].dtype)
+            groups["edges"] = new_edges
+        system = self._system_group
+        if system is not None:
+            groups["system"] = system.select(ids)
+        return Batch(_Storage(groups), self.device)
+
+    def trim(self, copied_mask: torch.Tensor | None = None) -> "Batch | None":
+        """A new batch without the systems whose ``copied_mask`` is True; ``None`` if none is left."""
+        if copied_mask is None:
+            copied_mask = getattr(self, "_copied_mask", None)
+            if copied_mask is None:
+                raise ValueError("trim requires copied_mask or a prior put")
+        keep = ~copied_mask.to(device=self.device, dtype=torch.bool)
+        if not bool(keep.any()):
+            return None
+        return self.index_select(torch.where(keep)[0])
+
+    def append(self, other: "Batch") -> None:
+        """Append the systems of ``other`` in place.  A group that ``other`` lacks is extended with
+        empty segments (atoms, edges) or zero rows (system)."""
+        if other is self or other._storage is self._storage:
+            raise ValueError("Cannot append a Batch that shares storage with the receiver (would corrupt both).  "
+                             "Use batch.append(batch.clone()) instead.")
+        total_nodes = self.num_nodes
+        n_other = other.num_graphs
+        for name, group in self._storage.groups.items():
+            other_group = other._storage.groups.get(name)
+            if other_group is None:
+                group.extend_for_appended_graphs(n_other)
+                continue
+            if name == "edges" and "neighbor_list" in other_group and "neighbor_list" in group:
+                shifted = SegmentedGroup(dict(other_group.items()), other_group.segment_lengths, other_group.device)
+                shifted["neighbor_list"] = other_group["neighbor_list"] + total_nodes
+                other_group = shifted
+            group.concatenate(other_group)
+        for stamp in ("_neighbor_row_order", "_neighbor_search_cutoff"):
+            object.__setattr__(self, stamp, None)
 
     def __setitem__(self, key: str, value: torch.Tensor) -> None:
         g = self._find(key)

@@ -210,7 +210,10 @@ class BaseDynamics(HookRegistryMixin):
         self.exit_status = exit_status
         self.model_config = model.model_config
         self.current_hook_stage: DynamicsStage | None = None
-        self.sampler = None
+        self.sampler = kwargs.pop("sampler", None)
+        self.refill_frequency: int = kwargs.pop("refill_frequency", 1)
+        self.done = False
+        self.active_batch = None
         self.global_rank = 0
         self._init_hooks(hooks)
         self._last_converged: torch.Tensor | None = None
@@ -369,6 +372,83 @@ class BaseDynamics(HookRegistryMixin):
             self._call_hooks(DynamicsStage.ON_CONVERGE, batch)
         self.step_count += 1
         return batch, converged
+
+    # ---- replacing finished systems (nvalchemi/dynamics/base.py:1628-1680, 1957-2083) ------------
+    def _sync_state_to_batch(self, remaining_indices: torch.Tensor, n_new: int, template_batch) -> None:
+        """Keep ``self._state`` aligned with a batch whose systems were replaced: the rows of the
+        remaining systems in order, then fresh default rows (``_make_new_state``) for the new ones."""
+        if not hasattr(self, "_state"):
+            return
+        remaining = self._state.index_select(remaining_indices) if remaining_indices.numel() > 0 else None
+        fresh = self._make_new_state(n_new, template_batch) if n_new > 0 else None
+        if remaining is not None and fresh is not None:
+            remaining.append(fresh)
+            self._state = remaining
+        elif remaining is not None:
+            self._state = remaining
+        elif fresh is not None:
+            self._state = fresh
+        else:
+            del self._state
+            self._state_ready = False
+
+    def refill_check(self, batch, exit_status: int):
+        """Drop the systems with ``status >= exit_status`` and append replacements from
+        ``self.sampler`` (an object with ``max_atoms``, ``max_edges``, ``max_batch_size``,
+        ``exhausted`` and ``request_replacements_budget(atom_budget=, edge_budget=, max_count=)``
+        returning a list of ``AtomicData``).  Returns the batch itself when nothing graduated, a new
+        batch otherwise, or ``None`` when no system is left (``self.done`` is set once the sampler
+        is exhausted too).  Bookkeeping fields of the remaining systems are carried over, those of
+        the new ones take their defaults; per-system integrator state follows."""
+        if self.sampler is None:
+            raise RuntimeError("refill_check requires a sampler to be configured.")
+        status = batch.status
+        if status.dim() == 2:
+            status = status.squeeze(-1)
+        graduated = status >= exit_status
+        if not graduated.any():
+            return batch
+        remaining_indices = torch.where(~graduated)[0]
+        n_remaining = remaining_indices.numel()
+        result = batch.index_select(remaining_indices) if n_remaining > 0 else None
+        sampler = self.sampler
+        remaining_atoms = int(batch.num_nodes_per_graph[remaining_indices].sum()) if n_remaining > 0 else 0
+        atom_budget = sampler.max_atoms - remaining_atoms if sampler.max_atoms is not None else None
+        edges_per_graph = batch.num_edges_per_graph
+        remaining_edges = int(edges_per_graph[remaining_indices].sum()) \
+            if n_remaining > 0 and edges_per_graph.numel() > 0 else 0
+        edge_budget = sampler.max_edges - remaining_edges if sampler.max_edges is not None else None
+        max_new = sampler.max_batch_size - n_remaining if sampler.max_batch_size is not None else None
+        replacements = sampler.request_replacements_budget(atom_budget=atom_budget, edge_budget=edge_budget,
+                                                           max_count=max_new)
+        from ..data.batch import Batch
+
+        if result is not None and replacements:
+            result.append(Batch.from_data_list(replacements, device=batch.device))
+        elif result is None and replacements:
+            result = Batch.from_data_list(replacements, device=batch.device)
+        if result is not None:
+            n_total = result.num_graphs
+            for key, default_fn in self._bookkeeping_keys.items():
+                new_tensor = default_fn(n_total, result.device)
+                vals = getattr(result, key, None)
+                if vals is not None:
+                    vals = vals.unsqueeze(-1) if vals.dim() == 1 else vals
+                    if vals.shape != new_tensor.shape:
+                        raise RuntimeError(f"Bookkeeping key '{key}' has shape {vals.shape} after refill, "
+                                           f"expected {new_tensor.shape}.")
+                    new_tensor.copy_(vals)
+                old = getattr(batch, key, None)
+                if old is not None and n_remaining > 0:
+                    src = old[remaining_indices]
+                    new_tensor[:n_remaining] = src.unsqueeze(-1) if src.dim() == 1 else src
+                result[key] = new_tensor
+            self._sync_state_to_batch(remaining_indices, len(replacements), result)
+            return result
+        if sampler.exhausted:
+            self.done = True
+        self._sync_state_to_batch(remaining_indices, 0, batch)
+        return None
 
     # ---- updates of selected systems only (nvalchemi/dynamics/base.py:2085-2212) ---------------
     def _run_masked(self, batch, mask: torch.Tensor, do_pre: bool, do_post: bool) -> None:
@@ -557,6 +637,17 @@ class FusedStage(BaseDynamics):
         for _, dyn in self.sub_stages:
             dyn._close_hooks()
 
+    def _sync_state_to_batch(self, remaining_indices: torch.Tensor, n_new: int, template_batch) -> None:
+        for _, dyn in self.sub_stages:
+            dyn._sync_state_to_batch(remaining_indices, n_new, template_batch)
+
+    def refill_check(self, batch, exit_status: int):
+        result = super().refill_check(batch, exit_status)
+        self._last_converged = None
+        for _, dyn in self.sub_stages:
+            dyn._last_converged = None
+        return result
+
     def _ensure_bookkeeping_fields(self, batch) -> None:
         for key, default_fn in self._bookkeeping_keys.items():
             if getattr(batch, key, None) is None:
@@ -657,12 +748,18 @@ class FusedStage(BaseDynamics):
 
     def run(self, batch=None, n_steps: int | None = None):
         """Evaluate the model once (the first step integrates with real forces), then step until
-        every system has ``exit_status`` or ``n_steps`` steps are done
-        (nvalchemi/dynamics/base.py:3162-3265, the mode with a batch supplied by the caller)."""
+        every system has ``exit_status`` or ``n_steps`` steps are done.  With a sampler configured
+        (``FusedStage(..., sampler=, refill_frequency=)``) and ``batch=None``, the first batch comes
+        from ``sampler.build_initial_batch()`` and every ``refill_frequency`` steps finished systems
+        are replaced (:meth:`refill_check`); the run ends, returning ``None``, when no system is
+        left (nvalchemi/dynamics/base.py:3162-3265)."""
         if batch is None:
             if self.sampler is None:
                 raise ValueError("No batch provided and no sampler configured.")
-            raise NotImplementedError("in-flight batching from a sampler is not available in this build")
+            batch = self.sampler.build_initial_batch()
+            if self.init_fn is not None:
+                self.init_fn(batch)
+            self.active_batch = batch
         self._ensure_bookkeeping_fields(batch)
         resolved = n_steps if n_steps is not None else self.n_steps
         self._open_hooks()
@@ -673,7 +770,16 @@ class FusedStage(BaseDynamics):
             step_num = 0
             while True:
                 batch, _ = self.step(batch)
-                if (step_num + 1) % self.convergence_check_frequency == 0 \
+                if self.sampler is not None and (step_num + 1) % self.refill_frequency == 0:
+                    result = self.refill_check(batch, self.exit_status)
+                    if result is None:
+                        self.active_batch = None
+                        return None
+                    # (newcomers are first integrated with the forces they arrive with, as in the
+                    # reference: no evaluation is inserted here)
+                    batch = result
+                    self.active_batch = batch
+                elif self.sampler is None and (step_num + 1) % self.convergence_check_frequency == 0 \
                         and self.all_complete(batch, self.exit_status):
                     break
                 step_num += 1

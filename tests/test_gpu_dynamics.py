@@ -458,3 +458,112 @@ def test_fused_stage_relax_then_md_equals_each_system_on_its_own():
         fused2.run(None)
     with pytest.raises(TypeError):
         fused2 + 3
+
+
+class _ListSampler:
+    """The sampler protocol ``refill_check`` needs, over a list of systems
+    (nvalchemi/dynamics/sampler.py:261-516: initial batch, budgeted replacements, exhaustion)."""
+
+    def __init__(self, systems, batch_size):
+        self._systems = list(systems)
+        self.max_batch_size = batch_size
+        self.max_atoms = None
+        self.max_edges = None
+        self.handed_out = 0
+
+    def _take(self, n):
+        out = self._systems[:n]
+        self._systems = self._systems[n:]
+        self.handed_out += len(out)
+        return out
+
+    def build_initial_batch(self):
+        from nvalchemi_amd.data import Batch
+
+        return Batch.from_data_list(self._take(self.max_batch_size), device=DEV)
+
+    def request_replacements_budget(self, atom_budget=None, edge_budget=None, max_count=None):
+        return self._take(max_count if max_count is not None else 1)
+
+    @property
+    def exhausted(self):
+        return not self._systems
+
+
+def test_fused_stage_refills_finished_systems_from_a_sampler():
+    """In-flight batching (nvalchemi/dynamics/base.py:1957-2083, 3162-3265): seven systems go
+    through a batch of three slots; each is relaxed exactly as it would be alone, finished systems
+    are replaced, integrator state and bookkeeping fields follow their systems."""
+    from nvalchemi_amd.data import AtomicData
+    from nvalchemi_amd.dynamics import FIRE, ConvergenceHook, FusedStage
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=9, n_boxes=7, reps=3, a=5.4, jitter=0.0)
+    rng = np.random.default_rng(4)
+    amps = (0.02, 0.2, 0.05, 0.12, 0.03, 0.3, 0.08)
+    for s, amp in enumerate(amps):
+        P[ptr[s]:ptr[s + 1]] += rng.normal(0, amp, (ptr[s + 1] - ptr[s], 3)).astype(np.float32)
+    tol = 0.02
+
+    def system(s):
+        a0, a1 = int(ptr[s]), int(ptr[s + 1])
+        n = a1 - a0
+        return AtomicData(torch.from_numpy(P[a0:a1]), torch.full((n,), 18), atomic_masses=torch.full((n,), 39.95),
+                          forces=torch.zeros(n, 3), energy=torch.zeros(1, 1), velocities=torch.zeros(n, 3),
+                          cell=torch.from_numpy(C[s]), pbc=torch.from_numpy(pb[s]),
+                          system_id=torch.full((1, 1), s, dtype=torch.long))
+
+    def relaxer():
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+        return model, FIRE(model, dt=1.0, convergence_hook=ConvergenceHook.from_fmax(tol))
+
+    # each system alone: the steps it needs and where it ends
+    alone = {}
+    for s in range(7):
+        from nvalchemi_amd.data import Batch
+
+        model, relax = relaxer()
+        for h in model.make_neighbor_hooks():
+            relax.register_hook(h)
+        b = Batch.from_data_list([system(s)], device=DEV)
+        if s < 3:
+            # the first batch is evaluated before its first step; a newcomer is not: it takes its
+            # first step with the zero forces it arrives with (FIRE shortens its time step there)
+            relax._call_hooks(relax._stage_type.BEFORE_COMPUTE, b)
+            relax.compute(b)
+        steps = 0
+        while True:
+            _, conv = relax.step(b)
+            steps += 1
+            if conv is not None:
+                break
+            assert steps < 500
+        alone[s] = (steps, b.positions.cpu().numpy())
+    assert len({v[0] for v in alone.values()}) > 2
+
+    model, relax = relaxer()
+    sampler = _ListSampler([system(s) for s in range(7)], batch_size=3)
+    finished = {}
+
+    class Collect:
+        frequency = 1
+        stage = FusedStage._stage_type.AFTER_STEP
+
+        def __call__(self, ctx, stage):
+            b = ctx.batch
+            done = torch.where(b.status.view(-1) >= 1)[0].tolist()
+            for k in done:
+                sid = int(b.system_id.view(-1)[k])
+                if sid not in finished:
+                    a0, a1 = int(b.batch_ptr[k]), int(b.batch_ptr[k + 1])
+                    finished[sid] = b.positions[a0:a1].cpu().numpy()
+
+    fused = FusedStage([(0, relax)], hooks=model.make_neighbor_hooks(), sampler=sampler, refill_frequency=1)
+    fused.register_fused_hook(Collect())
+    out = fused.run(None, n_steps=2000)
+    assert out is None and fused.done and sampler.exhausted and sampler.handed_out == 7
+    assert sorted(finished) == list(range(7))
+    for s in range(7):
+        ref = alone[s][1]
+        err = np.abs(finished[s].astype(np.float64) - ref)
+        assert (err <= ATOL + RTOL * np.abs(ref)).all(), (s, float(err.max()))

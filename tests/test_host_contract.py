@@ -256,3 +256,39 @@ def test_strategy_helpers_of_the_neighbor_hook():
     with pytest.raises(NotImplementedError):
         suggest_neighbor_list_method(ptr, torch.eye(3).repeat(2, 1, 1), torch.ones(2, 3, dtype=torch.bool), 3.0,
                                      positions_dtype=torch.float64)
+
+
+def test_batch_index_select_append_and_trim():
+    """Selecting, appending and trimming systems (nvalchemi/data/batch.py:816-874, 987-1038,
+    1138-1178): segments gathered in the order asked, ``neighbor_list`` re-based, system rows
+    following, the receiver of ``append`` growing in place."""
+    from nvalchemi_amd.data import AtomicData, Batch
+
+    g = torch.Generator().manual_seed(0)
+    data = []
+    for n in (3, 5, 2, 4):
+        nl = torch.tensor([[0, 1], [1, 0], [n - 1, 0]], dtype=torch.int32)
+        data.append(AtomicData(torch.rand(n, 3, generator=g), torch.full((n,), n), cell=torch.eye(3) * n,
+                               pbc=torch.ones(3, dtype=torch.bool), neighbor_list=nl,
+                               energy=torch.full((1, 1), float(n))))
+    b = Batch.from_data_list(data)
+    s = b.index_select([2, 0])
+    assert s.num_graphs == 2 and s.batch_ptr.tolist() == [0, 2, 5] and s.atomic_numbers.tolist() == [2, 2, 3, 3, 3]
+    assert s.neighbor_list.tolist() == [[0, 1], [1, 0], [1, 0], [2, 3], [3, 2], [4, 2]]
+    assert s.energy.view(-1).tolist() == [2.0, 3.0] and s.num_edges_per_graph.tolist() == [3, 3]
+    assert torch.equal(s.positions[2:5], b.positions[0:3]) and torch.equal(s.cell[0], b.cell[2])
+    s.append(b.index_select([3]))
+    assert s.num_graphs == 3 and s.batch_ptr.tolist() == [0, 2, 5, 9] and s.neighbor_list[-3:].tolist() == [[5, 6], [6, 5], [8, 5]]
+    assert s.batch_idx.tolist() == [0, 0, 1, 1, 1, 2, 2, 2, 2]
+    assert b[1:3].num_nodes_list == [5, 2] and isinstance(b[0], AtomicData) and b[-1].num_nodes == 4
+    assert b[torch.tensor([True, False, False, True])].num_nodes_list == [3, 4]
+    assert b.trim(torch.tensor([True, True, False, False])).num_nodes_list == [2, 4]
+    assert b.trim(torch.ones(4, dtype=torch.bool)) is None
+    with pytest.raises(ValueError):
+        b.append(b)
+    with pytest.raises(IndexError):
+        b.index_select([])
+    with pytest.raises(IndexError):
+        b.index_select(torch.tensor([0.5]))
+    with pytest.raises(ValueError):
+        b.trim()
