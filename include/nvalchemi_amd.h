@@ -156,6 +156,19 @@ int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces
                         int32_t n_systems, void* workspace, size_t workspace_bytes,
                         void* stream);
 
+/* BAOAB Langevin pre-force half step B-A-O-A: replaces the Warp launch behind
+ * nvalchemi::langevin_half_step (nvalchemi/dynamics/_ops/langevin.py:52-117; called from
+ * nvalchemi/dynamics/integrators/nvt_langevin.py:160-181).  kT (M) f32 in energy units,
+ * friction (M) f32 in 1/time, dt (M) f32; positions and velocities updated in place; active (M)
+ * bytes or NULL as for velocity Verlet.  The normal deviates of atom i are a function of
+ * (random_seed, i) only (Philox4x32-10, Box-Muller): callers advance the seed every step, as the
+ * reference does (random_seed + step_count).  The final B step, nvalchemi::langevin_finalize
+ * (:134-170), is nvamd_vv_velocity_finalize. */
+int32_t nvamd_langevin_half_step(float* positions, float* velocities, const float* forces,
+                                 const float* masses, const float* dt, const float* kT,
+                                 const float* friction, uint64_t random_seed, const int32_t* batch_idx,
+                                 const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* stream);
+
 /* Per-system maximum atomic force norm (the default convergence criterion,
  * nvalchemi/dynamics/base.py:258-349: vector_norm over xyz, scatter amax over atoms).
  * fmax (M) f32; systems without atoms give -inf. */

@@ -48,6 +48,7 @@ _SIGNATURES = {
     "nvamd_kinetic_energy": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_langevin_half_step": (_i32, [_vp] * 7 + [_c.c_uint64, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_nl_filter_matrix": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _f64, _vp, _vp, _vp, _vp]),
     "nvamd_nl_filter_coo_flags": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _c.c_int64, _f64, _vp, _vp]),
     "nvamd_buffer_workspace_bytes": (_i32, [_c.c_int64, _c.c_int64, _c.POINTER(_c.c_size_t)]),
@@ -499,3 +500,19 @@ def nl_filter_coo_flags(positions, cell, neighbor_list, neighbor_list_shifts, ba
         _opt(neighbor_list_shifts, "neighbor_list_shifts", torch.int32, (E, 3)),
         _opt(batch_idx, "batch_idx", torch.int32, (N,)), E, float(cutoff),
         _dev(_as_u8(keep), "keep", torch.uint8, (E,)), _stream(positions.device)), "nvamd_nl_filter_coo_flags")
+
+
+# --------------------------------------------------------------------------------------------
+# Langevin
+# --------------------------------------------------------------------------------------------
+def langevin_half_step(positions, velocities, forces, masses, dt, kT, friction, random_seed: int, batch_idx,
+                       active=None) -> None:
+    N = positions.shape[0]
+    M = dt.shape[0]
+    _check(library().nvamd_langevin_half_step(
+        _dev(positions, "positions", torch.float32, (N, 3)), _dev(velocities, "velocities", torch.float32, (N, 3)),
+        _dev(forces, "forces", torch.float32, (N, 3)), _dev(masses, "masses", torch.float32, (N,)),
+        _dev(dt, "dt", torch.float32, (M,)), _dev(kT, "temperature", torch.float32, (M,)),
+        _dev(friction, "friction", torch.float32, (M,)), int(random_seed) & 0xFFFFFFFFFFFFFFFF,
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
+        N, M, _stream(positions.device)), "nvamd_langevin_half_step")

@@ -1,3 +1,4 @@
 from .nve import NVE
+from .nvt_langevin import NVTLangevin
 
-__all__ = ["NVE"]
+__all__ = ["NVE", "NVTLangevin"]

@@ -56,6 +56,15 @@ def lib() -> ctypes.CDLL:
                                              ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
                                              ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double,
                                              ctypes.c_int32, _f32p, _f32p, _f32p, _f32p]
+        _u32p = ctypes.POINTER(ctypes.c_uint32)
+        _f64p = ctypes.POINTER(ctypes.c_double)
+        L.orc_philox4x32_10.restype = None
+        L.orc_philox4x32_10.argtypes = [_u32p, _u32p, _u32p]
+        L.orc_langevin_normals.restype = None
+        L.orc_langevin_normals.argtypes = [ctypes.c_uint64, ctypes.c_int32, _f64p]
+        L.orc_langevin_half_step.restype = None
+        L.orc_langevin_half_step.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, ctypes.c_uint64,
+                                             _i32p, _u8p, ctypes.c_int32]
         L.orc_vv_pre.restype = None
         L.orc_vv_pre.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _i32p, _u8p, ctypes.c_int32]
         L.orc_vv_post.restype = None
@@ -507,3 +516,31 @@ def neighbor_matrix_to_list(neighbor_matrix, num_neighbors, fill_value, neighbor
     ptr = np.zeros(N + 1, dtype=np.int32)
     ptr[1:] = np.cumsum(_i32(num_neighbors))
     return nl, ptr, None if neighbor_matrix_shifts is None else _i32(neighbor_matrix_shifts)[ii, kk]
+
+
+# ---------------------------------------------------------------------------------------------
+# Langevin (BAOAB half step) and its generator
+# ---------------------------------------------------------------------------------------------
+def philox4x32_10(counter, key):
+    c = np.asarray(counter, dtype=np.uint32).copy()
+    k = np.asarray(key, dtype=np.uint32).copy()
+    out = np.zeros(4, dtype=np.uint32)
+    u32p = ctypes.POINTER(ctypes.c_uint32)
+    lib().orc_philox4x32_10(c.ctypes.data_as(u32p), k.ctypes.data_as(u32p), out.ctypes.data_as(u32p))
+    return out
+
+
+def langevin_normals(seed, atom):
+    xi = np.zeros(4, dtype=np.float64)
+    lib().orc_langevin_normals(int(seed), int(atom), xi.ctypes.data_as(ctypes.POINTER(ctypes.c_double)))
+    return xi
+
+
+def langevin_half_step(positions, velocities, forces, masses, dt, kT, friction, seed, batch_idx, active=None):
+    """In place on float32 ``positions`` / ``velocities``."""
+    assert positions.dtype == np.float32 and velocities.dtype == np.float32
+    act = None if active is None else np.ascontiguousarray(active, dtype=np.uint8)
+    lib().orc_langevin_half_step(_p(positions, _f32p), _p(velocities, _f32p), _p(_f32(forces), _f32p),
+                                 _p(_f32(masses), _f32p), _p(_f32(dt), _f32p), _p(_f32(kT), _f32p),
+                                 _p(_f32(friction), _f32p), int(seed), _p(_i32(batch_idx), _i32p),
+                                 None if act is None else _p(act, _u8p), positions.shape[0])

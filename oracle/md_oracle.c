@@ -18,6 +18,8 @@
  *   orc_lj_matrix                nvalchemi/models/_ops/lj.py:31-54,116-216,246-321 and
  *                                nvalchemi/models/lj.py:464-477 (fp64 per-system sum)
  *   orc_vv_pre / orc_vv_post     nvalchemi/dynamics/_ops/velocity_verlet.py:63-64,112
+ *   orc_langevin_half_step       nvalchemi/dynamics/_ops/langevin.py:52-117,
+ *                                nvalchemi/dynamics/integrators/nvt_langevin.py:103-196
  *   orc_fire_step                nvalchemi/dynamics/_ops/fire.py:245-362,
  *                                nvalchemi/dynamics/optimizers/fire.py:69-76,182-219,
  *                                nvalchemi/distributed/_dynamics_coordinator.py:296-322
@@ -49,6 +51,12 @@
  *                  follows Bitzek 2006 / ASE ordering, constrained by the reference's
  *                  notes (reductions at entry; mixing with the stored alpha; per-atom
  *                  maxstep clamp; vanilla branch only).  Checked by invariants only.
+ *   orc_langevin_half_step  PARITY UNPINNED against the reference: its random stream and the rounding
+ *                  of its kernel are inside the absent library.  Pinned as mathematics: the generator
+ *                  by the published Philox4x32-10 known answers, the deviates by their moments, the
+ *                  step by its limits (no friction: the two half drifts of velocity Verlet; infinite
+ *                  friction: velocities redrawn at kT/m) and by the invariance of the Maxwell-Boltzmann
+ *                  variance under the O step.
  *   orc_fmax       pinned: in-tree Torch definition is complete; literal cases.
  *   orc_rebuild_check  pinned by the reference's own cases (flags cleared on every call, 1.0 over a
  *                  threshold of 0.5 flags, 0.1 does not, per-system selectivity, reference refreshed
@@ -456,6 +464,71 @@ ORC_API int32_t orc_lj_matrix_switched(const float* pos, const float* cells, con
     }
     free(e); free(f); free(w);
     return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * BAOAB Langevin half step B-A-O-A (nvalchemi/dynamics/_ops/langevin.py:52-117 documents the
+ * splitting; the kernel and its random generator are in the absent library).  float32, one
+ * rounding per operation:
+ *   v += (F/m)(dt/2) ; r += v (dt/2) ; v = c1 v + c2 xi ; r += v (dt/2)
+ *   c1 = exp(-gamma dt), c2 = sqrt((kT/m)(1 - c1^2)) in double, rounded once
+ * xi: Philox4x32-10 (Salmon et al., SC'11), key = 64-bit seed, counter = (atom, 0, 0, 0), two
+ * Box-Muller pairs in double, the first three deviates used.
+ * ---------------------------------------------------------------------------------------- */
+ORC_API void orc_philox4x32_10(const uint32_t* counter, const uint32_t* key, uint32_t* out) {
+    const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+    uint32_t c0 = counter[0], c1 = counter[1], c2 = counter[2], c3 = counter[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)M0 * c0, p1 = (uint64_t)M1 * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += W0; k1 += W1;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+ORC_API void orc_langevin_normals(uint64_t seed, int32_t atom, double* xi /* 4 */) {
+    uint32_t ctr[4] = {(uint32_t)atom, 0u, 0u, 0u};
+    uint32_t key[2] = {(uint32_t)(seed & 0xffffffffu), (uint32_t)(seed >> 32)};
+    uint32_t w[4];
+    orc_philox4x32_10(ctr, key, w);
+    for (int p = 0; p < 2; ++p) {
+        double u1 = ((double)w[2 * p] + 1.0) * (1.0 / 4294967296.0);
+        double u2 = (double)w[2 * p + 1] * (1.0 / 4294967296.0);
+        double radius = sqrt(-2.0 * log(u1)), angle = 6.283185307179586476925286766559 * u2;
+        xi[2 * p] = radius * cos(angle);
+        xi[2 * p + 1] = radius * sin(angle);
+    }
+}
+
+ORC_API void orc_langevin_half_step(float* pos, float* vel, const float* forces, const float* masses,
+                                    const float* dt, const float* kT, const float* friction, uint64_t seed,
+                                    const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms) {
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float m = masses[i], h = dt[s], hh = 0.5f * h;
+        double c1d = exp(-(double)friction[s] * (double)h);
+        float c1 = (float)c1d;
+        float c2 = (float)sqrt(((double)kT[s] / (double)m) * (1.0 - c1d * c1d));
+        double xi[4];
+        orc_langevin_normals(seed, i, xi);
+        for (int a = 0; a < 3; ++a) {
+            float v = vel[3 * i + a], r = pos[3 * i + a];
+            float acc = forces[3 * i + a] / m;
+            float kick = acc * hh;
+            v = v + kick;
+            float drift = v * hh;
+            r = r + drift;
+            float damped = c1 * v, noise = c2 * (float)xi[a];
+            v = damped + noise;
+            drift = v * hh;
+            r = r + drift;
+            vel[3 * i + a] = v;
+            pos[3 * i + a] = r;
+        }
+    }
 }
 
 /* ------------------------------------------------------------------------------------------

@@ -567,3 +567,59 @@ def test_fused_stage_refills_finished_systems_from_a_sampler():
         ref = alone[s][1]
         err = np.abs(finished[s].astype(np.float64) - ref)
         assert (err <= ATOL + RTOL * np.abs(ref)).all(), (s, float(err.max()))
+
+
+def test_nvt_langevin_thermalises_an_lj_crystal():
+    """``NVTLangevin`` on 4 FCC argon boxes started at rest: the kinetic temperature settles at the
+    target (equipartition over 2000 atoms, a few per cent), different seeds give different
+    trajectories, the same seed the same one, and the run follows the oracle step loop."""
+    from nvalchemi_amd.dynamics import NVTLangevin
+    from nvalchemi_amd.dynamics.hooks import temperature_per_graph
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=2, n_boxes=4, reps=5, a=5.4, jitter=0.02)
+    N = len(P)
+    Z = np.full(N, 18, dtype=np.int64)
+    M = np.full(N, 39.95, dtype=np.float32)
+    T_target = 80.0
+
+    def run(seed, steps):
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+        dyn = NVTLangevin(model, dt=4.0, temperature=T_target, friction=0.02, random_seed=seed,
+                          hooks=model.make_neighbor_hooks())
+        batch = make_batch(P, Z, M, C, pb, ptr, V=np.zeros_like(P))
+        temps = []
+        for k in range(steps):
+            dyn.step(batch)
+            if k >= steps // 2:
+                temps.append(temperature_per_graph(batch.velocities, batch.atomic_masses, batch.batch_idx, 4,
+                                                   batch.num_nodes_per_graph).mean().item())
+        return batch, float(np.mean(temps))
+
+    b1, t1 = run(7, 400)
+    assert abs(t1 / T_target - 1) < 0.06, t1
+    b2, _ = run(7, 400)
+    assert torch.equal(b1.positions, b2.positions)
+    b3, _ = run(8, 400)
+    assert not torch.equal(b1.positions, b3.positions)
+
+    # a short run against the oracle loop (pre: half step; neighbor list + LJ; post: half kick)
+    from _reference_loop import FS_PER_INTERNAL_TIME, build_and_eval
+
+    model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+    dyn = NVTLangevin(model, dt=2.0, temperature=T_target, friction=0.05, random_seed=3, hooks=model.make_neighbor_hooks())
+    batch = make_batch(P, Z, M, C, pb, ptr, V=np.zeros_like(P))
+    p, v, f = P.copy(), np.zeros_like(P), np.zeros_like(P)
+    bi = oracle.batch_idx_from_ptr(ptr)
+    dt = np.full(4, np.float32(2.0 / FS_PER_INTERNAL_TIME), np.float32)
+    kT = np.full(4, np.float32(T_target * 8.617333262e-5), np.float32)
+    gamma = np.full(4, np.float32(0.05 * FS_PER_INTERNAL_TIME), np.float32)
+    K = 96
+    for step in range(10):
+        dyn.step(batch)
+        oracle.langevin_half_step(p, v, f, M, dt, kT, gamma, 3 + step, bi)
+        out, K = build_and_eval(p, C, pb, ptr, bi, 8.0, 0.0104, 3.4, K)
+        f = out["forces"]
+        oracle.vv_post(v, f, M, dt, bi)
+    close(batch.positions, p, "positions after 10 Langevin steps")
+    close(batch.velocities, v, "velocities after 10 Langevin steps")

@@ -415,3 +415,40 @@ def test_segmented_observables_match_oracle():
     temp = temperature_per_graph(T(vel), T(mass), T(idx), B, n_at).cpu().numpy()
     ok = np.array(counts) > 0
     assert np.allclose(temp[ok], 2 * want[ok] / (3 * np.array(counts)[ok] * KB_EV), rtol=2e-6)
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_langevin_half_step_matches_oracle(masked):
+    """B-A-O-A against the oracle with the same generator: positions and velocities to float32
+    rounding (the deviates pass through log / cos / sin of two different math libraries)."""
+    from nvalchemi_amd import _lib
+
+    rng = np.random.default_rng(12)
+    counts = np.array([5, 0, 300, 1, 64, 2000])
+    B = len(counts)
+    bi = np.repeat(np.arange(B), counts).astype(np.int32)
+    N = len(bi)
+    P = rng.normal(0, 3, (N, 3)).astype(np.float32)
+    V = rng.normal(0, 0.05, (N, 3)).astype(np.float32)
+    F = rng.normal(0, 0.3, (N, 3)).astype(np.float32)
+    M = rng.uniform(1, 60, N).astype(np.float32)
+    dt = rng.uniform(0.02, 0.2, B).astype(np.float32)
+    kT = rng.uniform(0.005, 0.05, B).astype(np.float32)
+    gamma = np.array([0.0, 1.0, 0.1, 5.0, 100.0, 0.5], np.float32)
+    active = np.array([1, 1, 0, 1, 1, 1], np.uint8) if masked else None
+    for seed in (0, 42, 2 ** 40 + 17):
+        p, v = P.copy(), V.copy()
+        oracle.langevin_half_step(p, v, F, M, dt, kT, gamma, seed, bi, active=active)
+        tp, tv = T(P), T(V)
+        _lib.langevin_half_step(tp, tv, T(F), T(M), T(dt), T(kT), T(gamma), seed, T(bi),
+                                None if active is None else T(active.astype(bool)))
+        assert np.allclose(tv.cpu().numpy(), v, rtol=2e-6, atol=1e-7)
+        assert np.allclose(tp.cpu().numpy(), p, rtol=2e-6, atol=1e-6)
+        if masked:
+            sel = bi == 2
+            assert np.array_equal(tp.cpu().numpy()[sel], P[sel]) and np.array_equal(tv.cpu().numpy()[sel], V[sel])
+    # another seed, other deviates
+    a, b = T(V), T(V)
+    _lib.langevin_half_step(T(P), a, T(F), T(M), T(dt), T(kT), T(gamma), 1, T(bi))
+    _lib.langevin_half_step(T(P), b, T(F), T(M), T(dt), T(kT), T(gamma), 2, T(bi))
+    assert not torch.equal(a, b)
