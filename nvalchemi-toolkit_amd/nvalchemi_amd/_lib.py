@@ -130,14 +130,14 @@ def _as_u8(t: torch.Tensor | None) -> torch.Tensor | None:
 
 
 class _Workspaces:
-    """One growing scratch buffer per (device, purpose); kernels of one purpose run in
-    stream order, so they can share it."""
+    """One growing scratch buffer per (device, stream, purpose): kernels of one purpose on one
+    stream run in order and can share it; another stream gets its own."""
 
     def __init__(self) -> None:
         self._bufs: dict[tuple, torch.Tensor] = {}
 
     def get(self, device: torch.device, purpose: str, nbytes: int) -> torch.Tensor:
-        key = (device.index, purpose)
+        key = (device.index, _stream(device), purpose)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
