@@ -1014,22 +1014,51 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         int nh = 0;                                         // entries in the hit list
                         unsigned short* my_hits = hits[wave];
 
-                        // The self entry (distance 0) is always accepted by the distance test; it is
-                        // dropped when the hit list is written out, which keeps that comparison out
-                        // of the per-candidate loop.
+                        // One step: 64 candidates against the centre atom, one comparison each: whatever
+                        // is inside the outer edge of the float32 uncertainty band goes to the wave's hit
+                        // list.  The list is a superset: it still holds the centre atom itself (distance 0)
+                        // and the few candidates inside the band.
+                        auto dist2 = [&](const float4& p) {
+                            const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
+                            return dx * dx + dy * dy + dz * dz;
+                        };
+                        auto accept = [&](const int k, const float4& p, const float d2) {
+                            const bool take = HALF ? (d2 < rc2_hi && i_atom <= __float_as_int(p.w)) : (d2 < rc2_hi);
+                            const unsigned long long m = __builtin_amdgcn_ballot_w64(take);
+                            if (take) {
+                                const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                             __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                my_hits[nh + before] = (unsigned short)k;
+                            }
+                            nh += __popcll(m);
+                        };
+                        // Writing the list out, 64 entries a step: the self entry is dropped, an entry
+                        // inside the band is decided by the exact expression (rare), the rest get their
+                        // shift and their slot.  This keeps everything but one comparison out of the
+                        // per-candidate loop.
                         auto flush = [&]() {
-                            int removed = 0;  // 1 once the self entry has been passed
                             for (int l0 = 0; l0 < nh; l0 += kWave) {
                                 const int l = l0 + lane;
-                                const bool live = l < nh;
-                                const int k = live ? my_hits[l] : -2;
-                                const unsigned long long ms = __builtin_amdgcn_ballot_w64(live && k == k_self);
-                                const int self_l = ms ? l0 + (int)__builtin_ctzll(ms) : 0x7fffffff;
-                                if (live && k != k_self) {
-                                    const int j = __float_as_int(c_pos[k].w);
-                                    int s0, s1, s2;
+                                const int k = l < nh ? my_hits[l] : k_self;
+                                bool in = l < nh && k != k_self;
+                                int j = 0, s0 = 0, s1 = 0, s2 = 0;
+                                if (in) {
+                                    const float4 p = c_pos[k];
+                                    j = __float_as_int(p.w);
                                     candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
-                                    const int slot = base + l - removed - (l > self_l ? 1 : 0);
+                                    if (!(dist2(p) < rc2_lo)) {  // inside the band: decide exactly
+                                        const float* pi = a.pos + 3 * (size_t)i_atom;
+                                        const float* pj = a.pos + 3 * (size_t)j;
+                                        double e0, e1d, e2d;
+                                        in = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1, s2,
+                                                           ws.sys[sidx].h, e0, e1d, e2d) < a.rc2;
+                                    }
+                                    if (HALF && in) in = half_keep(i_atom, j, s0, s1, s2);
+                                }
+                                const unsigned long long m = __builtin_amdgcn_ballot_w64(in);
+                                if (in) {
+                                    const int slot = base + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                                      __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
                                     if (slot < a.K) {
                                         row[slot] = j;
                                         if (srow) {
@@ -1039,61 +1068,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                         }
                                     }
                                 }
-                                if (ms) removed = 1;
+                                base += __popcll(m);
                             }
-                            base += nh - removed;
                             nh = 0;
-                        };
-
-                        // One step: 64 candidates against the centre atom.  Accepted candidates are
-                        // appended to the wave's hit list; the rare step that has a candidate inside the
-                        // float32 uncertainty band (or, for half lists, an image of the centre atom
-                        // itself) takes a second, exact look at those candidates only.
-                        auto dist2 = [&](const float4& p) {
-                            const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
-                            return dx * dx + dy * dy + dz * dz;
-                        };
-                        auto accept = [&](const int k, const float4& p, const float d2) {
-                            const bool lo = d2 < rc2_lo, hi = d2 < rc2_hi;
-                            const bool take = HALF ? (lo && i_atom < __float_as_int(p.w)) : lo;
-                            const unsigned long long m = __builtin_amdgcn_ballot_w64(take);
-                            if (take) {
-                                const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
-                                                                             __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-                                my_hits[nh + before] = (unsigned short)k;
-                            }
-                            nh += __popcll(m);
-                            bool rare;
-                            if (HALF) {
-                                rare = __builtin_amdgcn_ballot_w64(hi && (!lo || __float_as_int(p.w) == i_atom)) != 0ull;
-                            } else {
-                                rare = __builtin_amdgcn_ballot_w64(hi) != m;
-                            }
-                            if (rare) {
-                                bool in = false;
-                                if (hi && (!lo || (HALF && __float_as_int(p.w) == i_atom)) && k != k_self) {
-                                    const int j = __float_as_int(p.w);
-                                    int s0, s1, s2;
-                                    candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
-                                    in = lo;
-                                    if (!lo) {  // inside the band: decide exactly
-                                        const float* pi = a.pos + 3 * (size_t)i_atom;
-                                        const float* pj = a.pos + 3 * (size_t)j;
-                                        double e0, e1d, e2d;
-                                        const double r2 = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1,
-                                                                        s2, ws.sys[sidx].h, e0, e1d, e2d);
-                                        in = r2 < a.rc2;
-                                    }
-                                    if (HALF && in) in = half_keep(i_atom, j, s0, s1, s2);
-                                }
-                                const unsigned long long me = __builtin_amdgcn_ballot_w64(in);
-                                if (in) {
-                                    const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(me >> 32),
-                                                                                 __builtin_amdgcn_mbcnt_lo((unsigned)me, 0));
-                                    my_hits[nh + before] = (unsigned short)k;
-                                }
-                                nh += __popcll(me);
-                            }
                         };
                         int k0 = k_lo;
                         for (; k0 + kWave < k_hi; k0 += 2 * kWave) {
