@@ -20,6 +20,9 @@
 #ifndef NVAMD_LJ_UNROLL
 #define NVAMD_LJ_UNROLL 4
 #endif
+#ifndef NVAMD_LJ_UNROLL_DERIVED
+#define NVAMD_LJ_UNROLL_DERIVED 8
+#endif
 namespace nvamd {
 namespace {
 
@@ -175,7 +178,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
         // UNROLL row entries per lane are in flight at once: first every index and shift of the
         // chunk, then every neighbor position, then the arithmetic (the loop is latency bound
         // otherwise: two dependent trips to memory per entry)
-        constexpr int UNROLL = NVAMD_LJ_UNROLL;
+        constexpr int UNROLL = (IMG == 2 && VEC) ? NVAMD_LJ_UNROLL_DERIVED : NVAMD_LJ_UNROLL;
         const int last_quad = cnt > 0 ? ((cnt - 1) & ~3) : 0;  // lanes beyond it re-read it: no extra lines
         for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
             int jj[UNROLL], s0[UNROLL], s1[UNROLL], s2[UNROLL];
