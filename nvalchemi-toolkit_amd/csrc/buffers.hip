@@ -374,6 +374,8 @@ NVAMD_EXPORT int32_t nvamd_put_masked_per_system(const void* source, const uint8
     int32_t rc = check_common("put_masked_per_system", num_src, row_bytes, workspace, workspace_bytes, 0, &s);
     if (rc != NVAMD_OK) return rc;
     if (num_dest < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "put_masked_per_system: negative num_dest");
+    if ((size_t)num_src * (size_t)row_bytes > kMaxBytes)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "put_masked_per_system: more than 2^38 bytes");
     if (num_src == 0) return NVAMD_OK;
     if (!source_mask || !source_data_copied || (num_dest > 0 && !dest_mask) ||
         (row_bytes > 0 && (!source || (num_dest > 0 && !dest))))
@@ -446,6 +448,8 @@ NVAMD_EXPORT int32_t nvamd_put_masked_segmented(const void* source, const int32_
     if (rc != NVAMD_OK) return rc;
     if (num_dest_segments < 0 || dest_capacity < 0 || total_rows < 0 || row_bytes <= 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "put_masked_segmented: bad size");
+    if ((size_t)total_rows * (size_t)row_bytes > kMaxBytes)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "put_masked_segmented: more than 2^38 bytes");
     if (num_systems == 0) return NVAMD_OK;
     if (!source_batch_ptr || !source_mask || !dest_batch_ptr || !source_data_copied || !new_num_dest ||
         (total_rows > 0 && !source) || (dest_capacity > 0 && !dest))
