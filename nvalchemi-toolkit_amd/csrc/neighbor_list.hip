@@ -1073,6 +1073,20 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             nh = 0;
                         };
                         int k0 = k_lo;
+                        // four steps' candidates are in flight at once (the registers are there: the
+                        // kernel's register count is set by its set-up phases, not by this loop)
+                        for (; k0 + 3 * kWave < k_hi; k0 += 4 * kWave) {
+                            const int k = k0 + lane;
+                            const float4 pa = c_pos[k], pb = c_pos[k + kWave], pc = c_pos[k + 2 * kWave],
+                                         pd = c_pos[k + 3 * kWave];
+                            const float da = dist2(pa), db = dist2(pb), dc = dist2(pc), dd = dist2(pd);
+                            accept(k, pa, da);
+                            accept(k + kWave, pb, db);
+                            if (nh > kHitCap - 3 * kWave) flush();
+                            accept(k + 2 * kWave, pc, dc);
+                            accept(k + 3 * kWave, pd, dd);
+                            if (nh > kHitCap - 3 * kWave) flush();
+                        }
                         for (; k0 + kWave < k_hi; k0 += 2 * kWave) {
                             const int k = k0 + lane;
                             const float4 pa = c_pos[k], pb = c_pos[k + kWave];
