@@ -1,0 +1,141 @@
+"""The reference's own behavioural cases for ``NeighborListHook``, restated against this package
+(test/hooks/test_neighbor_list_hook.py: ``TestShapeInvalidation`` :539-608, ``TestAdaptiveK``
+:946-1029, ``TestStaleCOOEntries`` :1031-1100, with its builders ``_line_batch`` :63-90 and
+``_pbc_wrap_batch`` :91-104).  Same inputs, same expected results; buffers that only the
+reference's implementation has (staging copies) are not asserted."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+CUTOFF = 2.5
+
+
+def cfg(cutoff=CUTOFF, fmt=None, half_list=False):
+    from nvalchemi_amd.models.base import NeighborConfig, NeighborListFormat
+
+    return NeighborConfig(cutoff=cutoff, format=fmt or NeighborListFormat.MATRIX, half_list=half_list)
+
+
+def ctx(batch):
+    from nvalchemi_amd.hooks._context import HookContext
+
+    return HookContext(batch=batch)
+
+
+def stage():
+    from nvalchemi_amd.dynamics import DynamicsStage
+
+    return DynamicsStage.BEFORE_COMPUTE
+
+
+def line_batch(pbc=False, n_graphs=1, cell_size=20.0):
+    from nvalchemi_amd.data import AtomicData, Batch
+
+    data = []
+    for _ in range(n_graphs):
+        kw = {}
+        if pbc:
+            kw["cell"] = torch.eye(3) * cell_size
+            kw["pbc"] = torch.tensor([True, True, True])
+        data.append(AtomicData(torch.tensor([[0.0, 0, 0], [1.5, 0, 0], [5.0, 0, 0]]), torch.tensor([1, 1, 1]), **kw))
+    return Batch.from_data_list(data, device=DEV)
+
+
+def random_batch(n):
+    from nvalchemi_amd.data import AtomicData, Batch
+
+    return Batch.from_data_list([AtomicData(torch.rand(n, 3), torch.ones(n, dtype=torch.long))], device=DEV)
+
+
+def hook(**kw):
+    from nvalchemi_amd.hooks import NeighborListHook
+
+    config = kw.pop("config", None) or cfg()
+    return NeighborListHook(config, stage=stage(), **kw)
+
+
+def is_neighbor(nm, nn, i, j):
+    return j in nm[i, : int(nn[i])].tolist()
+
+
+def test_line_and_wrap_batches_give_the_reference_topology():
+    from nvalchemi_amd.data import AtomicData, Batch
+
+    b = line_batch()
+    hook()(ctx(b), stage())
+    assert is_neighbor(b.neighbor_matrix, b.num_neighbors, 0, 1) and is_neighbor(b.neighbor_matrix, b.num_neighbors, 1, 0)
+    assert int(b.num_neighbors[2]) == 0 and "neighbor_matrix_shifts" not in b
+    two = line_batch(n_graphs=2)
+    hook()(ctx(two), stage())
+    assert is_neighbor(two.neighbor_matrix, two.num_neighbors, 3, 4) and not is_neighbor(two.neighbor_matrix, two.num_neighbors, 1, 3)
+    w = Batch.from_data_list([AtomicData(torch.tensor([[0.1, 0, 0], [2.9, 0, 0]]), torch.tensor([1, 1]),
+                                         cell=torch.eye(3) * 3.0, pbc=torch.tensor([True, True, True]))], device=DEV)
+    hook()(ctx(w), stage())
+    assert is_neighbor(w.neighbor_matrix, w.num_neighbors, 0, 1)
+    k = w.neighbor_matrix[0, : int(w.num_neighbors[0])].tolist().index(1)
+    assert w.neighbor_matrix_shifts[0, k].tolist() == [-1, 0, 0]
+    assert w._neighbor_list_cutoff == CUTOFF
+
+
+def test_shape_changes_reallocate_and_reset_the_skin_reference():
+    h = hook()
+    small = line_batch()
+    h(ctx(small), stage())
+    assert h._alloc_N == 3 and h._alloc_B == 1
+    matrix = h._neighbor_matrix
+    h(ctx(small), stage())
+    assert h._neighbor_matrix is matrix  # same shape: the same buffers
+    h(ctx(random_batch(5)), stage())
+    assert h._alloc_N == 5 and h._neighbor_matrix.shape[0] == 5
+    h(ctx(line_batch(n_graphs=2)), stage())
+    assert h._alloc_B == 2 and h._alloc_N == 6
+    s = hook(skin=0.5)
+    s(ctx(small), stage())
+    assert s._ref_positions is not None and s._ref_positions.shape == (3, 3)
+    s(ctx(random_batch(5)), stage())
+    assert s._ref_positions is not None and s._ref_positions.shape == (5, 3)
+
+
+def test_adaptive_k():
+    from nvalchemi_amd.data import AtomicData, Batch
+    from nvalchemi_amd.neighbors import compute_neighbors
+
+    three = Batch.from_data_list([AtomicData(torch.tensor([[0.0, 0, 0], [1.0, 0, 0], [2.0, 0, 0]]),
+                                             torch.tensor([1, 1, 1]))], device=DEV)
+    h = hook(config=cfg(cutoff=100.0))
+    h(ctx(three), stage())
+    assert h._max_neighbors <= 16  # non-periodic: capped at ceil16(largest system)
+    pair = Batch.from_data_list([AtomicData(torch.tensor([[0.0, 0, 0], [1.0, 0, 0]]), torch.tensor([1, 1]),
+                                            cell=torch.eye(3) * 3.0, pbc=torch.tensor([True, True, True]))], device=DEV)
+    h = hook(config=cfg(cutoff=6.0))
+    h(ctx(pair), stage())
+    assert h._max_neighbors > 1 and int(h._num_neighbors.max()) < h._max_neighbors  # images: no cap
+    four = Batch.from_data_list([AtomicData(torch.tensor([[0.0, 0, 0], [1.0, 0, 0], [2.0, 0, 0], [3.0, 0, 0]]),
+                                            torch.ones(4, dtype=torch.long))], device=DEV)
+    h = hook(config=cfg(cutoff=5.0), max_neighbors=100)
+    h(ctx(four), stage())
+    assert h._max_neighbors < 100 and h._neighbor_matrix.shape[1] == h._max_neighbors
+    assert int(h._num_neighbors.max()) <= 3
+    b = Batch.from_data_list([AtomicData(torch.tensor([[0.0, 0, 0], [1.0, 0, 0], [2.0, 0, 0]]), torch.tensor([1, 1, 1]),
+                                         forces=torch.zeros(3, 3), energy=torch.zeros(1, 1))], device=DEV)
+    compute_neighbors(b, cutoff=100.0)
+    assert b.neighbor_matrix.shape[1] <= 16
+
+
+def test_shrinking_neighbors_leave_no_stale_coo_edges():
+    from nvalchemi_amd.hooks import NeighborListHook
+    from nvalchemi_amd.models.base import NeighborListFormat
+
+    h = NeighborListHook(cfg(fmt=NeighborListFormat.COO), skin=1.0, stage=stage())
+    b = line_batch()
+    h(ctx(b), stage())
+    before = {tuple(r) for r in b.neighbor_list.cpu().tolist()}
+    b.positions[1, 0] = 4.0  # 4.0 from atom 0 (beyond cutoff + skin), 1.0 from atom 2; moved 2.5 > skin / 2
+    h(ctx(b), stage())
+    after = {tuple(r) for r in b.neighbor_list.cpu().tolist()}
+    assert (0, 1) in before and (1, 0) in before
+    assert (0, 1) not in after and (1, 0) not in after and (1, 2) in after and (2, 1) in after
+    counts = torch.bincount(b.neighbor_list[:, 0].cpu().long(), minlength=b.num_nodes)
+    assert torch.equal(counts, h._num_neighbors.cpu().long())
