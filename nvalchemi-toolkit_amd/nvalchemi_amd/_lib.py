@@ -389,6 +389,8 @@ def _mask(t: torch.Tensor, name: str, n: int) -> int:
 
 
 def _buffer_ws(device, n_systems: int, data_bytes: int = 0) -> torch.Tensor:
+    if torch.device(device).type != "cuda":
+        raise KernelLibraryError(f"tensors are on {device}; the nvalchemi_amd kernels run on a ROCm device only")
     need = _size(library().nvamd_buffer_workspace_bytes, int(n_systems), int(data_bytes))
     return workspaces.get(device, "buffers", need)
 

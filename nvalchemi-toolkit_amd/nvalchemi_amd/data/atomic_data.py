@@ -128,3 +128,8 @@ class AtomicData:
         out = object.__new__(AtomicData)
         out._data = {k: v.to(device) for k, v in self._data.items()}
         return out
+
+    def clone(self) -> "AtomicData":
+        out = object.__new__(AtomicData)
+        out._data = {k: v.clone() for k, v in self._data.items()}
+        return out

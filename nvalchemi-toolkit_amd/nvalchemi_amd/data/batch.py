@@ -16,7 +16,19 @@ from typing import Any, Iterator
 
 import torch
 
+from . import buffer_kernels
 from .atomic_data import EDGE_KEYS, NODE_KEYS, SYSTEM_KEYS, AtomicData
+
+
+_NEIGHBOR_MATRIX_KEYS = ("neighbor_matrix", "neighbor_matrix_shifts", "num_neighbors")
+_BUFFER_DTYPES = (torch.bool, torch.float32, torch.float64, torch.int32, torch.int64)
+
+
+def _bool_on(mask: torch.Tensor, device) -> torch.Tensor:
+    """``mask`` itself when it already is a bool tensor on ``device`` (so that in-place updates
+    reach the caller), else a converted copy."""
+    return mask if mask.dtype == torch.bool and mask.device == torch.device(device) else mask.to(
+        device=device, dtype=torch.bool)
 
 
 class SegmentedGroup:
@@ -27,16 +39,44 @@ class SegmentedGroup:
         self.segment_lengths = segment_lengths.to(device=device, dtype=torch.int32)
         self.device = torch.device(device)
         self._batch_idx: torch.Tensor | None = None
+        # boundaries; may hold more than len(self) + 1 entries (headroom for put)
         self._batch_ptr: torch.Tensor | None = None
         self._lengths_host: list[int] | None = None
+        # True when the tensors may hold more rows than the segments use (empty, put, defrag)
+        self._over_allocated = False
 
     def __len__(self) -> int:
         return int(self.segment_lengths.shape[0])
 
     def num_elements(self) -> int:
+        if not self._over_allocated:
+            for t in self._tensors.values():
+                return int(t.shape[0])
+        return int(sum(self.lengths_list()))
+
+    def capacity(self) -> int:
+        """Rows the tensors can hold."""
         for t in self._tensors.values():
             return int(t.shape[0])
-        return int(sum(self.lengths_list()))
+        return 0
+
+    def _ptr_store(self) -> torch.Tensor:
+        if self._batch_ptr is None:
+            ptr = torch.zeros(len(self) + 1, dtype=torch.int32, device=self.device)
+            ptr[1:] = torch.cumsum(self.segment_lengths, 0)
+            self._batch_ptr = ptr
+        return self._batch_ptr
+
+    def _invalidate(self) -> None:
+        self._batch_idx = self._lengths_host = None
+        if hasattr(self, "_edge_ptr"):
+            del self._edge_ptr
+
+    def _tight(self) -> dict[str, torch.Tensor]:
+        if not self._over_allocated:
+            return self._tensors
+        n = self.num_elements()
+        return {k: v[:n] for k, v in self._tensors.items()}
 
     def lengths_list(self) -> list[int]:
         if self._lengths_host is None:
@@ -45,11 +85,7 @@ class SegmentedGroup:
 
     @property
     def batch_ptr(self) -> torch.Tensor:
-        if self._batch_ptr is None:
-            ptr = torch.zeros(len(self) + 1, dtype=torch.int32, device=self.device)
-            ptr[1:] = torch.cumsum(self.segment_lengths, 0)
-            self._batch_ptr = ptr
-        return self._batch_ptr
+        return self._ptr_store()[: len(self) + 1]
 
     @property
     def batch_idx(self) -> torch.Tensor:
@@ -79,6 +115,14 @@ class SegmentedGroup:
     def items(self):
         return self._tensors.items()
 
+    def mapped(self, fn, device) -> "SegmentedGroup":
+        """A group over ``fn`` of every tensor (a copy or a move), bookkeeping included."""
+        out = SegmentedGroup({k: fn(v) for k, v in self._tensors.items()}, fn(self.segment_lengths), device)
+        out._over_allocated = self._over_allocated
+        if self._over_allocated and self._batch_ptr is not None:
+            out._batch_ptr = fn(self._batch_ptr)
+        return out
+
     def select(self, idx: list[int]) -> "SegmentedGroup":
         """The segments ``idx`` (any order, repeats allowed) as a new group: one gather per tensor
         through an element index built from the boundaries."""
@@ -100,17 +144,121 @@ class SegmentedGroup:
         """Append the segments of ``other`` in place; keys that only one side has are dropped
         (derived data such as a neighbor matrix cannot be carried over a change of the batch)."""
         common = [k for k in self._tensors if k in other._tensors]
-        self._tensors = {k: torch.cat([self._tensors[k], other._tensors[k].to(self.device)], 0) for k in common}
+        mine, theirs = self._tight(), other._tight()
+        self._tensors = {k: torch.cat([mine[k], theirs[k].to(self.device)], 0) for k in common}
         self.segment_lengths = torch.cat([self.segment_lengths, other.segment_lengths.to(self.device)])
-        self._batch_idx = self._batch_ptr = self._lengths_host = None
-        if hasattr(self, "_edge_ptr"):
-            del self._edge_ptr
+        self._over_allocated = False
+        self._batch_ptr = None
+        self._invalidate()
 
     def extend_for_appended_graphs(self, n: int) -> None:
         """``n`` more systems without elements."""
         self.segment_lengths = torch.cat([self.segment_lengths,
                                           torch.zeros(n, dtype=torch.int32, device=self.device)])
-        self._batch_idx = self._batch_ptr = self._lengths_host = None
+        self._batch_ptr = None
+        self._invalidate()
+
+    # ---- fixed-capacity use (nvalchemi/data/level_storage.py:1778-1960) -----------------------
+    def compute_put_per_system_fit_mask(self, source: "SegmentedGroup", source_mask: torch.Tensor,
+                                        dest_mask: torch.Tensor | None, fit_mask: torch.Tensor) -> None:
+        """``fit_mask[i]`` = segment ``i`` of ``source`` is masked and would fit behind this group's
+        segments; all False when the boundary tensor has no headroom for ``len(source)`` more
+        segments.  ``dest_mask`` is ignored.  Nothing is copied."""
+        n_seg = len(source)
+        if source_mask.shape[0] != n_seg:
+            raise ValueError(f"source_mask shape {source_mask.shape[0]} != len(source) {n_seg}")
+        if fit_mask.shape[0] != n_seg:
+            raise ValueError(f"fit_mask shape {fit_mask.shape[0]} != {n_seg}")
+        store = self._ptr_store()
+        if store.shape[0] < len(self) + n_seg + 2:
+            fit_mask.zero_()
+            return
+        buffer_kernels.compute_put_fit_mask_segmented(source.batch_ptr, _bool_on(source_mask, self.device), store,
+                                                      len(self), self.capacity(), fit_mask)
+
+    def put(self, src: "SegmentedGroup", mask: torch.Tensor, *, copied_mask: torch.Tensor | None = None) -> None:
+        """Copy the masked segments of ``src`` that fit behind this group's segments, for the keys
+        both sides have; ``copied_mask`` (or ``src._copied_mask``) receives which segments moved.
+        One host read afterwards, for the new segment count.  Without headroom in the boundary
+        tensor nothing is copied.  The boundary tensor is cut to the new count.
+
+        The reference moves the float32 keys only (level_storage.py:1879-1884) and leaves the
+        others zero in the destination; here every key of a supported dtype moves, except the
+        per-atom neighbor data (matrix, its shifts, counts), which names atoms by their index in
+        the source batch and has to be rebuilt.  ``neighbor_list`` moves as it is: ``Batch.put``
+        re-bases it."""
+        if not self._tensors or not src._tensors:
+            raise ValueError("put requires non-empty source and dest")
+        common = [k for k in self._tensors if k in src._tensors]
+        if not common:
+            raise ValueError("put requires at least one common attribute")
+        n_seg = len(src)
+        if mask.shape[0] != n_seg:
+            raise ValueError(f"mask shape {mask.shape[0]} != num segments {n_seg}")
+        mask = _bool_on(mask, self.device)
+        if copied_mask is not None:
+            if copied_mask.shape[0] != n_seg:
+                raise ValueError(f"copied_mask shape {copied_mask.shape[0]} != {n_seg}")
+            out_mask = _bool_on(copied_mask, self.device)
+        else:
+            out_mask = torch.zeros(n_seg, device=self.device, dtype=torch.bool)
+            src._copied_mask = out_mask
+        store = self._ptr_store()
+        n_dest = len(self)
+        if store.shape[0] < n_dest + n_seg + 2:
+            return
+        src_ptr = src.batch_ptr
+        new_num_dest = None
+        for key in common:
+            src_t, dest_t = src._tensors[key], self._tensors[key]
+            if key in _NEIGHBOR_MATRIX_KEYS or src_t.dtype != dest_t.dtype or src_t.dtype not in _BUFFER_DTYPES:
+                continue
+            new_num_dest = buffer_kernels.put_masked_segmented(src_t, src_ptr, mask, dest_t, store, n_dest, out_mask)
+        if new_num_dest is not None:
+            new_n = int(new_num_dest.item())
+            self._batch_ptr = store[: new_n + 1].clone()
+            self.segment_lengths = self._batch_ptr[1:] - self._batch_ptr[:-1]
+            self._over_allocated = True
+            self._invalidate()
+
+    def defrag(self, copied_mask: torch.Tensor | None = None) -> "SegmentedGroup":
+        """Drop the segments whose ``copied_mask`` is True in place: the others move to the front,
+        the rows behind them are zeroed, the tensors keep their shape."""
+        if not self._tensors:
+            return self
+        n_seg = len(self)
+        if copied_mask is None:
+            copied_mask = getattr(self, "_copied_mask", None)
+            if copied_mask is None:
+                raise ValueError("defrag requires copied_mask or a prior put")
+        copied_mask = _bool_on(copied_mask, self.device)
+        if copied_mask.shape[0] != n_seg:
+            raise ValueError(f"copied_mask shape {copied_mask.shape[0]} != {n_seg}")
+        ptr = self.batch_ptr
+        original = ptr.clone()
+        num_kept = None
+        for key, t in self._tensors.items():
+            if num_kept is None:
+                num_kept = buffer_kernels.defrag_segmented(t, ptr, copied_mask)
+            else:
+                buffer_kernels.defrag_segmented(t, original.clone(), copied_mask)
+        n_kept = int(num_kept.item())
+        self.segment_lengths = (ptr[1:] - ptr[:-1])[:n_kept].clone()
+        self._over_allocated = True
+        self._invalidate()
+        if hasattr(self, "_copied_mask"):
+            del self._copied_mask
+        return self
+
+    def zero(self) -> None:
+        """No segments, all rows zero; tensors and boundary headroom are kept."""
+        for t in self._tensors.values():
+            t.zero_()
+        self.segment_lengths = torch.empty(0, dtype=torch.int32, device=self.device)
+        if self._batch_ptr is not None:
+            self._batch_ptr = torch.zeros(self._batch_ptr.shape[0], dtype=torch.int32, device=self.device)
+        self._over_allocated = True
+        self._invalidate()
 
 
 class UniformGroup:
@@ -120,9 +268,21 @@ class UniformGroup:
         self._tensors = dict(data)
         self._n = int(n)
         self.device = torch.device(device)
+        # True when the rows in use are counted apart from the tensors' shape (empty, defrag):
+        # then put adds to the count
+        self._counted = False
 
     def __len__(self) -> int:
         return self._n
+
+    def capacity(self) -> int:
+        """Rows the tensors can hold."""
+        for t in self._tensors.values():
+            return int(t.shape[0])
+        return self._n
+
+    def _tight(self) -> dict[str, torch.Tensor]:
+        return {k: v[: self._n] for k, v in self._tensors.items()} if self._counted else self._tensors
 
     def __getitem__(self, key):
         return self._tensors[key]
@@ -142,20 +302,114 @@ class UniformGroup:
     def items(self):
         return self._tensors.items()
 
+    def mapped(self, fn, device) -> "UniformGroup":
+        """A group over ``fn`` of every tensor (a copy or a move), bookkeeping included."""
+        out = UniformGroup({k: fn(v) for k, v in self._tensors.items()}, self._n, device)
+        out._counted = self._counted
+        return out
+
     def select(self, idx: list[int]) -> "UniformGroup":
         sel = torch.tensor(idx, dtype=torch.long, device=self.device)
         return UniformGroup({k: v.index_select(0, sel) for k, v in self._tensors.items()}, len(idx), self.device)
 
     def concatenate(self, other: "UniformGroup") -> None:
         common = [k for k in self._tensors if k in other._tensors]
-        self._tensors = {k: torch.cat([self._tensors[k], other._tensors[k].to(self.device)], 0) for k in common}
+        mine, theirs = self._tight(), other._tight()
+        self._tensors = {k: torch.cat([mine[k], theirs[k].to(self.device)], 0) for k in common}
         self._n += len(other)
+        self._counted = False
 
     def extend_for_appended_graphs(self, n: int) -> None:
         """``n`` more systems with zero rows (the other batch has no such group)."""
         self._tensors = {k: torch.cat([v, torch.zeros((n,) + tuple(v.shape[1:]), dtype=v.dtype, device=v.device)], 0)
-                         for k, v in self._tensors.items()}
+                         for k, v in self._tight().items()}
         self._n += n
+        self._counted = False
+
+    # ---- fixed-capacity use (nvalchemi/data/level_storage.py:1067-1228) -----------------------
+    def _dest_mask(self, dest_mask: torch.Tensor | None) -> torch.Tensor:
+        cap = self.capacity()
+        if dest_mask is None:
+            return torch.zeros(cap, device=self.device, dtype=torch.bool)
+        if dest_mask.shape[0] != cap:
+            raise ValueError(f"dest_mask shape {dest_mask.shape[0]} != dest capacity {cap}")
+        return _bool_on(dest_mask, self.device)
+
+    def compute_put_per_system_fit_mask(self, source: "UniformGroup", source_mask: torch.Tensor,
+                                        dest_mask: torch.Tensor | None, fit_mask: torch.Tensor) -> None:
+        """``fit_mask[i]`` = row ``i`` of ``source`` is masked and an empty slot is left for it
+        (``dest_mask`` True = occupied; None = every slot empty).  Nothing is copied."""
+        n_src = len(source)
+        if source_mask.shape[0] != n_src:
+            raise ValueError(f"source_mask shape {source_mask.shape[0]} != len(source) {n_src}")
+        if fit_mask.shape[0] != n_src:
+            raise ValueError(f"fit_mask shape {fit_mask.shape[0]} != {n_src}")
+        buffer_kernels.compute_put_fit_mask_per_system(_bool_on(source_mask, self.device), self._dest_mask(dest_mask),
+                                                       fit_mask)
+
+    def put(self, src: "UniformGroup", mask: torch.Tensor, *, copied_mask: torch.Tensor | None = None,
+            dest_mask: torch.Tensor | None = None) -> None:
+        """Copy the masked rows of ``src`` into the empty slots, for the keys both sides have;
+        ``dest_mask`` and ``copied_mask`` (or ``src._copied_mask``) are updated in place.
+
+        Every key fills the same slots.  (The reference hands the mask that the first key's copy
+        has already updated to the next key, level_storage.py:1170-1181, so that a second key's
+        rows land behind the first key's.)"""
+        if not self._tensors or not src._tensors:
+            raise ValueError("put requires non-empty source and dest")
+        common = [k for k in self._tensors if k in src._tensors]
+        if not common:
+            raise ValueError("put requires at least one common attribute")
+        n_src = len(src)
+        if mask.shape[0] != n_src:
+            raise ValueError(f"mask shape {mask.shape[0]} != len(src) {n_src}")
+        mask = _bool_on(mask, self.device)
+        if copied_mask is not None:
+            if copied_mask.shape[0] != n_src:
+                raise ValueError(f"copied_mask shape {copied_mask.shape[0]} != {n_src}")
+            out_mask = _bool_on(copied_mask, self.device)
+        else:
+            out_mask = torch.zeros(n_src, device=self.device, dtype=torch.bool)
+            src._copied_mask = out_mask
+        given = dest_mask
+        dest_mask = self._dest_mask(dest_mask)
+        before = dest_mask.clone()
+        for key in common:
+            # every key starts from the same occupancy: the kernel marks the slots it fills
+            slots = before.clone()
+            buffer_kernels.put_masked_per_system(src._tensors[key][:n_src], mask, self._tensors[key], slots, out_mask)
+            dest_mask.copy_(slots)
+        if given is not None and given is not dest_mask:
+            given.copy_(dest_mask)
+        if self._counted:
+            self._n += int(out_mask.sum().item())
+
+    def defrag(self, copied_mask: torch.Tensor | None = None) -> "UniformGroup":
+        """Drop the rows whose ``copied_mask`` is True in place: the others move to the front, the
+        rows behind them are zeroed, the tensors keep their shape."""
+        if not self._tensors:
+            return self
+        n_src = len(self)
+        if copied_mask is None:
+            copied_mask = getattr(self, "_copied_mask", None)
+            if copied_mask is None:
+                raise ValueError("defrag requires copied_mask or a prior put")
+        copied_mask = _bool_on(copied_mask, self.device)
+        if copied_mask.shape[0] != n_src:
+            raise ValueError(f"copied_mask shape {copied_mask.shape[0]} != {n_src}")
+        for t in self._tensors.values():
+            buffer_kernels.defrag_per_system(t[:n_src], copied_mask.clone())
+        self._n = int((~copied_mask).sum().item())
+        self._counted = True
+        if hasattr(self, "_copied_mask"):
+            del self._copied_mask
+        return self
+
+    def zero(self) -> None:
+        for t in self._tensors.values():
+            t.zero_()
+        self._n = 0
+        self._counted = True
 
 
 class _Storage:
@@ -219,6 +473,52 @@ class Batch:
     def _construct(cls, device, groups: dict[str, Any]) -> "Batch":
         return cls(_Storage(groups), device)
 
+    @classmethod
+    def empty(cls, *, num_systems: int, num_nodes: int, num_edges: int, template: "AtomicData | Batch | None" = None,
+              device="cpu") -> "Batch":
+        """A batch of zero systems over zeroed storage for ``num_systems`` systems, ``num_nodes``
+        atoms and ``num_edges`` edges in total, with the keys, trailing shapes and dtypes of
+        ``template`` (default: positions, atomic numbers and an energy).  Fill it with :meth:`put`
+        (nvalchemi/data/batch.py:569-687)."""
+        if num_systems < 0 or num_nodes < 0 or num_edges < 0:
+            raise ValueError("num_systems, num_nodes, and num_edges must be non-negative")
+        dev = torch.device(device)
+        if template is None:
+            template = AtomicData(torch.zeros(1, 3), torch.zeros(1, dtype=torch.long), energy=torch.tensor([[0.0]]))
+        ref = cls.from_data_list([template], device=dev) if isinstance(template, AtomicData) else template
+        groups: dict[str, Any] = {}
+        for name, group in ref._storage.groups.items():
+            keys = list(group.keys())
+            if not keys:
+                continue
+            rows = num_systems if name == "system" else num_nodes if name == "atoms" else num_edges
+            data = {k: torch.zeros((rows,) + tuple(group[k].shape[1:]), device=dev, dtype=group[k].dtype) for k in keys}
+            if name == "system":
+                g = UniformGroup(data, 0, dev)
+                g._counted = True
+            else:
+                g = SegmentedGroup(data, torch.empty(0, dtype=torch.int32), dev)
+                g._batch_ptr = torch.zeros(max(num_systems + 2, 2), dtype=torch.int32, device=dev)
+                g._over_allocated = True
+            groups[name] = g
+        return cls(_Storage(groups), dev)
+
+    @classmethod
+    def empty_like(cls, batch: "Batch", *, device=None) -> "Batch":
+        """A batch of zero systems and zero capacity with the keys of ``batch``."""
+        return cls.empty(num_systems=0, num_nodes=0, num_edges=0, template=batch,
+                         device=device if device is not None else batch.device)
+
+    def zero(self) -> None:
+        """Back to zero systems; the storage is zeroed and kept (nvalchemi/data/batch.py:690-737)."""
+        for group in self._storage.groups.values():
+            group.zero()
+        self._drop_neighbor_stamps()
+
+    def _drop_neighbor_stamps(self) -> None:
+        for stamp in ("_neighbor_row_order", "_neighbor_search_cutoff"):
+            object.__setattr__(self, stamp, None)
+
     # ---- sizes and index tensors ---------------------------------------------------------------
     @property
     def _atoms_group(self) -> SegmentedGroup | None:
@@ -247,6 +547,12 @@ class Batch:
     def num_edges(self) -> int:
         e = self._edges_group
         return e.num_elements() if e is not None else 0
+
+    @property
+    def system_capacity(self) -> int:
+        """Systems the storage can hold (for a batch from :meth:`empty`)."""
+        g = self._system_group
+        return g.capacity() if g is not None else 0
 
     @property
     def batch_idx(self) -> torch.Tensor:
@@ -282,6 +588,11 @@ class Batch:
     def num_nodes_list(self) -> list[int]:
         a = self._atoms_group
         return a.lengths_list() if a is not None else []
+
+    @property
+    def num_edges_list(self) -> list[int]:
+        e = self._edges_group
+        return e.lengths_list() if e is not None else []
 
     @property
     def num_nodes_per_graph(self) -> torch.Tensor:
@@ -406,6 +717,98 @@ class Batch:
             return None
         return self.index_select(torch.where(keep)[0])
 
+    # ---- fixed-capacity use (nvalchemi/data/batch.py:876-985) ------------------------------------
+    def put(self, src_batch: "Batch", mask: torch.Tensor, *, copied_mask: torch.Tensor | None = None,
+            dest_mask: torch.Tensor | None = None) -> None:
+        """Copy the systems of ``src_batch`` with ``mask`` set into this batch's free storage: the
+        systems that fit on every level (a free system slot, room for their atoms, room for their
+        edges) are copied, the others are not.  ``copied_mask`` -- or, without it,
+        ``src_batch._copied_mask`` -- receives which ones moved, for :meth:`defrag` or :meth:`trim`
+        of the source.  ``dest_mask`` (one flag per system slot, True = occupied) is updated in
+        place; None treats every slot as empty."""
+        device = self.device
+        n = src_batch.num_graphs
+        if mask.shape[0] != n:
+            raise ValueError(f"mask shape {mask.shape[0]} != num_graphs {n}")
+        mask = _bool_on(mask, device)
+        if copied_mask is not None:
+            if copied_mask.shape[0] != n:
+                raise ValueError(f"copied_mask shape {copied_mask.shape[0]} != {n}")
+            copy_mask = _bool_on(copied_mask, device)
+        else:
+            copy_mask = torch.zeros(n, device=device, dtype=torch.bool)
+            object.__setattr__(src_batch, "_copied_mask", copy_mask)
+        levels = []
+        for mine, theirs in ((self._system_group, src_batch._system_group),
+                             (self._atoms_group, src_batch._atoms_group),
+                             (self._edges_group, src_batch._edges_group)):
+            if mine is not None and theirs is not None and len(mine.keys()) and len(theirs.keys()):
+                levels.append((mine, theirs))
+        fit_mask = torch.ones(n, device=device, dtype=torch.bool)
+        for mine, theirs in levels:
+            level_fit = torch.empty(n, device=device, dtype=torch.bool)
+            mine.compute_put_per_system_fit_mask(theirs, mask, dest_mask if isinstance(mine, UniformGroup) else None,
+                                                 level_fit)
+            fit_mask.logical_and_(level_fit)
+        copy_mask.copy_(fit_mask)
+        if copied_mask is not None and copy_mask is not copied_mask:
+            copied_mask.copy_(copy_mask)
+        atoms, edges = self._atoms_group, self._edges_group
+        n_before = len(atoms) if atoms is not None else 0
+        for mine, theirs in levels:
+            if isinstance(mine, UniformGroup):
+                mine.put(theirs, copy_mask, copied_mask=copy_mask, dest_mask=dest_mask)
+            else:
+                mine.put(theirs, copy_mask, copied_mask=copy_mask)
+        # the copied edges name atoms by their index in the source: move them to where the atoms went
+        src_atoms, src_edges = src_batch._atoms_group, src_batch._edges_group
+        if atoms is not None and src_atoms is not None and edges is not None and src_edges is not None \
+                and "neighbor_list" in edges and "neighbor_list" in src_edges and len(atoms) > n_before \
+                and len(edges) == len(atoms):
+            moved = torch.where(copy_mask)[0]
+            new_ids = torch.arange(n_before, n_before + moved.numel(), device=device)
+            delta = atoms.batch_ptr[new_ids] - src_atoms.batch_ptr[moved]
+            eptr = edges.batch_ptr
+            lo, hi = int(eptr[n_before]), int(eptr[n_before + moved.numel()])
+            if hi > lo:
+                owner = edges.batch_idx[lo:hi].to(torch.long) - n_before
+                nl = edges["neighbor_list"]
+                nl[lo:hi] += delta[owner].unsqueeze(1).to(nl.dtype)
+        self._drop_neighbor_stamps()
+
+    def defrag(self, copied_mask: torch.Tensor | None = None) -> "Batch":
+        """Drop the systems whose ``copied_mask`` is True (default: the mask the last :meth:`put`
+        left on this batch) in place.  The kept systems move to the front of the storage, which
+        keeps its size; rows behind them are zeroed."""
+        if copied_mask is None:
+            copied_mask = getattr(self, "_copied_mask", None)
+            if copied_mask is None:
+                raise ValueError("defrag requires copied_mask or a prior put")
+        if copied_mask.shape[0] != self.num_graphs:
+            raise ValueError(f"copied_mask shape {copied_mask.shape[0]} != {self.num_graphs}")
+        atoms, edges = self._atoms_group, self._edges_group
+        rebase = atoms is not None and edges is not None and "neighbor_list" in edges and len(atoms.keys()) > 0
+        if rebase:
+            kept = torch.where(~_bool_on(copied_mask, self.device))[0]
+            old_starts = atoms.batch_ptr[kept].clone()
+        for group in (self._system_group, atoms, edges):
+            if group is not None:
+                group.defrag(copied_mask=copied_mask)
+        if rebase and kept.numel() and edges.num_elements():
+            # the kept systems' atoms moved forward: so do the indices their edges hold
+            delta = atoms.batch_ptr[: kept.numel()] - old_starts
+            nl = edges["neighbor_list"]
+            nl[: edges.num_elements()] += delta[edges.batch_idx.to(torch.long)].unsqueeze(1).to(nl.dtype)
+        if "_copied_mask" in self.__dict__:
+            object.__delattr__(self, "_copied_mask")
+        self._drop_neighbor_stamps()
+        return self
+
+    def append_data(self, data_list: list[AtomicData]) -> None:
+        if not data_list:
+            raise ValueError("No data provided to append.")
+        self.append(Batch.from_data_list(data_list, device=self.device))
+
     def append(self, other: "Batch") -> None:
         """Append the systems of ``other`` in place.  A group that ``other`` lacks is extended with
         empty segments (atoms, edges) or zero rows (system)."""
@@ -424,8 +827,7 @@ class Batch:
                 shifted["neighbor_list"] = other_group["neighbor_list"] + total_nodes
                 other_group = shifted
             group.concatenate(other_group)
-        for stamp in ("_neighbor_row_order", "_neighbor_search_cutoff"):
-            object.__setattr__(self, stamp, None)
+        self._drop_neighbor_stamps()
 
     def __setitem__(self, key: str, value: torch.Tensor) -> None:
         g = self._find(key)
@@ -465,38 +867,25 @@ class Batch:
         return f"Batch(num_graphs={self.num_graphs}, num_nodes={self.num_nodes}, keys={sorted(self.keys())})"
 
     # ---- movement ------------------------------------------------------------------------------
-    def to(self, device) -> "Batch":
-        dev = torch.device(device)
-        groups: dict[str, Any] = {}
-        for name, g in self._storage.groups.items():
-            data = {k: v.to(dev) for k, v in g.items()}
-            if isinstance(g, SegmentedGroup):
-                groups[name] = SegmentedGroup(data, g.segment_lengths, dev)
-            else:
-                groups[name] = UniformGroup(data, len(g), dev)
-        out = Batch(_Storage(groups), dev)
+    def _mapped(self, fn, device) -> "Batch":
+        groups = {name: g.mapped(fn, device) for name, g in self._storage.groups.items()}
+        out = Batch(_Storage(groups), device)
         if "_neighbor_list_cutoff" in self.__dict__:
             out._neighbor_list_cutoff = self._neighbor_list_cutoff
         return out
 
+    def to(self, device) -> "Batch":
+        dev = torch.device(device)
+        return self._mapped(lambda t: t.to(dev), dev)
+
     def clone(self) -> "Batch":
-        groups: dict[str, Any] = {}
-        for name, g in self._storage.groups.items():
-            data = {k: v.clone() for k, v in g.items()}
-            if isinstance(g, SegmentedGroup):
-                groups[name] = SegmentedGroup(data, g.segment_lengths.clone(), self.device)
-            else:
-                groups[name] = UniformGroup(data, len(g), self.device)
-        out = Batch(_Storage(groups), self.device)
-        if "_neighbor_list_cutoff" in self.__dict__:
-            out._neighbor_list_cutoff = self._neighbor_list_cutoff
-        return out
+        return self._mapped(lambda t: t.clone(), self.device)
 
     def cpu(self) -> "Batch":
         return self.to("cpu")
 
     def get_data(self, idx: int) -> AtomicData:
-        """One system back out of the batch (atoms and system keys)."""
+        """One system back out of the batch; ``neighbor_list`` is re-based to the system's atoms."""
         ptr = self.batch_ptr.tolist()
         a0, a1 = ptr[idx], ptr[idx + 1]
         fields = {}
@@ -504,6 +893,12 @@ class Batch:
             if k in ("neighbor_matrix", "neighbor_matrix_shifts", "num_neighbors"):
                 continue
             fields[k] = v[a0:a1]
+        edges = self._edges_group
+        if edges is not None and len(edges.keys()):
+            eptr = edges.batch_ptr.tolist()
+            e0, e1 = eptr[idx], eptr[idx + 1]
+            for k, v in edges.items():
+                fields[k] = v[e0:e1] - a0 if k == "neighbor_list" else v[e0:e1]
         sysg = self._system_group
         if sysg is not None:
             for k, v in sysg.items():
@@ -511,3 +906,6 @@ class Batch:
         pos = fields.pop("positions")
         z = fields.pop("atomic_numbers")
         return AtomicData(pos, z, **fields)
+
+    def to_data_list(self) -> list[AtomicData]:
+        return [self.get_data(i) for i in range(self.num_graphs)]

@@ -2,5 +2,7 @@ from .base import BaseDynamics, ConvergenceHook, DynamicsStage, FusedStage
 from .integrators.nve import NVE
 from .integrators.nvt_langevin import NVTLangevin
 from .optimizers.fire import FIRE
+from .sinks import DataSink, GPUBuffer, HostMemory
 
-__all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "FusedStage", "NVE", "NVTLangevin", "FIRE"]
+__all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "FusedStage", "NVE", "NVTLangevin", "FIRE",
+           "DataSink", "GPUBuffer", "HostMemory"]

@@ -211,6 +211,8 @@ class BaseDynamics(HookRegistryMixin):
         self.model_config = model.model_config
         self.current_hook_stage: DynamicsStage | None = None
         self.sampler = kwargs.pop("sampler", None)
+        sinks = kwargs.pop("sinks", None)
+        self.sinks = list(sinks) if sinks is not None else []
         self.refill_frequency: int = kwargs.pop("refill_frequency", 1)
         self.done = False
         self.active_batch = None
@@ -392,8 +394,18 @@ class BaseDynamics(HookRegistryMixin):
             del self._state
             self._state_ready = False
 
+    def _overflow_to_sinks(self, batch, mask: torch.Tensor | None = None) -> None:
+        """Write ``batch`` (its masked systems) to the first sink that is not full
+        (nvalchemi/dynamics/base.py:878-901)."""
+        for sink in self.sinks:
+            if not sink.is_full:
+                sink.write(batch, mask=mask)
+                return
+        raise RuntimeError(f"All sinks are full. Cannot store {batch.num_graphs} overflow samples.")
+
     def refill_check(self, batch, exit_status: int):
-        """Drop the systems with ``status >= exit_status`` and append replacements from
+        """Drop the systems with ``status >= exit_status`` (after writing them to the first sink with
+        room, when sinks are configured) and append replacements from
         ``self.sampler`` (an object with ``max_atoms``, ``max_edges``, ``max_batch_size``,
         ``exhausted`` and ``request_replacements_budget(atom_budget=, edge_budget=, max_count=)``
         returning a list of ``AtomicData``).  Returns the batch itself when nothing graduated, a new
@@ -409,6 +421,8 @@ class BaseDynamics(HookRegistryMixin):
         if not graduated.any():
             return batch
         remaining_indices = torch.where(~graduated)[0]
+        if self.sinks:
+            self._overflow_to_sinks(batch, mask=graduated)
         n_remaining = remaining_indices.numel()
         result = batch.index_select(remaining_indices) if n_remaining > 0 else None
         sampler = self.sampler

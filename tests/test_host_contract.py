@@ -292,3 +292,53 @@ def test_batch_index_select_append_and_trim():
         b.index_select(torch.tensor([0.5]))
     with pytest.raises(ValueError):
         b.trim()
+
+
+def test_fixed_capacity_batches_and_host_sink_on_the_host():
+    """The bookkeeping of ``Batch.empty`` / ``zero`` / ``empty_like`` (nvalchemi/data/batch.py:569-737,
+    1583-1616) and the ``HostMemory`` sink (nvalchemi/dynamics/sinks.py:537-670) need no kernel; the
+    masked copies do, and refuse host tensors instead of copying some other way."""
+    from nvalchemi_amd import _lib
+    from nvalchemi_amd.data import AtomicData, Batch
+    from nvalchemi_amd.dynamics import DataSink, GPUBuffer, HostMemory
+
+    g = torch.Generator().manual_seed(1)
+    data = [AtomicData(torch.rand(n, 3, generator=g), torch.full((n,), n), cell=torch.eye(3) * n,
+                       pbc=torch.ones(3, dtype=torch.bool), energy=torch.full((1, 1), float(n)),
+                       neighbor_list=torch.tensor([[0, n - 1], [n - 1, 0]])) for n in (3, 5, 2)]
+    b = Batch.from_data_list(data)
+    buf = Batch.empty(num_systems=4, num_nodes=20, num_edges=8, template=b)
+    assert buf.num_graphs == 0 and buf.system_capacity == 4 and buf.num_nodes == 0 and buf.num_edges == 0
+    assert buf.positions.shape == (20, 3) and buf.cell.shape == (4, 3, 3) and buf.neighbor_list.shape == (8, 2)
+    assert buf.atomic_numbers.dtype == b.atomic_numbers.dtype and buf.batch_ptr.tolist() == [0]
+    assert buf._atoms_group._ptr_store().shape[0] == 6 and buf.num_nodes_list == []
+    buf.zero()
+    assert buf.num_graphs == 0 and buf.system_capacity == 4
+    like = Batch.empty_like(b)
+    assert like.num_graphs == 0 and like.system_capacity == 0 and sorted(like.keys()) == sorted(b.keys())
+    with pytest.raises(_lib.KernelLibraryError):
+        buf.put(b, torch.ones(3, dtype=torch.bool))
+    with pytest.raises(_lib.KernelLibraryError):
+        b.defrag(copied_mask=torch.tensor([True, False, False]))
+    with pytest.raises(ValueError, match="defrag requires copied_mask or a prior put"):
+        Batch.from_data_list(data).defrag()
+
+    with pytest.raises(TypeError):
+        DataSink()
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="requires an available GPU"):
+            GPUBuffer(capacity=1, max_atoms=1, max_edges=0)
+    sink = HostMemory(capacity=3)
+    sink.write(b, mask=torch.tensor([False, True, True]))
+    assert len(sink) == 2 and not sink.is_full
+    with pytest.raises(RuntimeError, match="Buffer is full"):
+        sink.write(b)
+    out = sink.drain()
+    assert len(sink) == 0 and out.num_nodes_list == [5, 2] and out.neighbor_list.tolist() == [[0, 4], [4, 0], [5, 6], [6, 5]]
+    assert torch.equal(out.positions, b.positions[3:]) and out.energy.view(-1).tolist() == [5.0, 2.0]
+    got = b.to_data_list()
+    assert [d.num_nodes for d in got] == [3, 5, 2] and got[1].neighbor_list.tolist() == [[0, 4], [4, 0]]
+    b.append_data([data[0]])
+    assert b.num_nodes_list == [3, 5, 2, 3]
+    with pytest.raises(ValueError, match="No data provided"):
+        b.append_data([])
