@@ -67,6 +67,7 @@ class AtomicData:
         n = positions.shape[0]
         dtype = positions.dtype
         self._data: dict[str, torch.Tensor] = {"positions": positions, "atomic_numbers": atomic_numbers}
+        self._levels: dict[str, str] = {}
         for key, value in fields.items():
             if value is None:
                 continue
@@ -105,7 +106,10 @@ class AtomicData:
         return self._data.items()
 
     def level_of(self, key: str) -> str:
-        """``"atoms"``, ``"edges"`` or ``"system"`` (unknown keys: by leading dimension)."""
+        """``"atoms"``, ``"edges"`` or ``"system"`` (unknown keys: as declared by ``add_*_property``,
+        else by leading dimension)."""
+        if key in self._levels:
+            return self._levels[key]
         if key in NODE_KEYS:
             return "atoms"
         if key in EDGE_KEYS:
@@ -121,15 +125,42 @@ class AtomicData:
             return data[name]
         raise AttributeError(name)
 
+    def __setattr__(self, name: str, value: Any) -> None:
+        """A tensor assigned to a public name becomes a key of the system."""
+        if name.startswith("_") or not isinstance(value, torch.Tensor):
+            object.__setattr__(self, name, value)
+        else:
+            self._data[name] = value
+
     def __contains__(self, key: str) -> bool:
         return key in self._data
+
+    @property
+    def device(self) -> torch.device:
+        return self._data["positions"].device
+
+    def add_system_property(self, key: str, value: torch.Tensor) -> None:
+        """``value`` (leading dimension one) as a system-level key, whatever its name
+        (nvalchemi/data/atomic_data.py:667-670)."""
+        self._data[key] = torch.as_tensor(value)
+        self._levels[key] = "system"
+
+    def add_node_property(self, key: str, value: torch.Tensor) -> None:
+        self._data[key] = torch.as_tensor(value)
+        self._levels[key] = "atoms"
+
+    def add_edge_property(self, key: str, value: torch.Tensor) -> None:
+        self._data[key] = torch.as_tensor(value)
+        self._levels[key] = "edges"
 
     def to(self, device) -> "AtomicData":
         out = object.__new__(AtomicData)
         out._data = {k: v.to(device) for k, v in self._data.items()}
+        out._levels = dict(self._levels)
         return out
 
     def clone(self) -> "AtomicData":
         out = object.__new__(AtomicData)
         out._data = {k: v.clone() for k, v in self._data.items()}
+        out._levels = dict(self._levels)
         return out

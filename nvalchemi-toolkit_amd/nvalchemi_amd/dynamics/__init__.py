@@ -2,7 +2,8 @@ from .base import BaseDynamics, ConvergenceHook, DynamicsStage, FusedStage
 from .integrators.nve import NVE
 from .integrators.nvt_langevin import NVTLangevin
 from .optimizers.fire import FIRE
+from .sampler import SizeAwareSampler
 from .sinks import DataSink, GPUBuffer, HostMemory
 
 __all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "FusedStage", "NVE", "NVTLangevin", "FIRE",
-           "DataSink", "GPUBuffer", "HostMemory"]
+           "DataSink", "GPUBuffer", "HostMemory", "SizeAwareSampler"]

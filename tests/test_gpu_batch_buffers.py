@@ -263,10 +263,10 @@ def test_fused_stage_writes_finished_systems_to_its_sinks_in_order():
     (nvalchemi/dynamics/base.py:878-901, 1999-2000): what the sinks hold is what the step hook saw
     leave, bit for bit, whichever sink it went to."""
     from nvalchemi_amd.data import AtomicData
-    from nvalchemi_amd.dynamics import FIRE, ConvergenceHook, FusedStage, GPUBuffer, HostMemory
+    from nvalchemi_amd.dynamics import (FIRE, ConvergenceHook, FusedStage, GPUBuffer, HostMemory,
+                                        SizeAwareSampler)
     from nvalchemi_amd.models import LennardJonesModelWrapper
     from _systems import fcc_boxes
-    from test_gpu_dynamics import _ListSampler
 
     P, C, pb, ptr = fcc_boxes(seed=9, n_boxes=6, reps=2, a=5.4, jitter=0.0)
     rng = np.random.default_rng(4)
@@ -278,14 +278,26 @@ def test_fused_stage_writes_finished_systems_to_its_sinks_in_order():
         n = a1 - a0
         return AtomicData(torch.from_numpy(P[a0:a1]), torch.full((n,), 18), atomic_masses=torch.full((n,), 39.95),
                           forces=torch.zeros(n, 3), energy=torch.zeros(1, 1), velocities=torch.zeros(n, 3),
-                          cell=torch.from_numpy(C[s]), pbc=torch.from_numpy(pb[s]),
-                          system_id=torch.full((1, 1), s, dtype=torch.long))
+                          cell=torch.from_numpy(C[s]), pbc=torch.from_numpy(pb[s])).to(DEV)
+
+    class Dataset:
+        """The dataset protocol of the sampler over a list of systems."""
+
+        def __len__(self):
+            return 6
+
+        def get_metadata(self, k):
+            return int(ptr[k + 1] - ptr[k]), 0
+
+        def __getitem__(self, k):
+            return system(k), {}
 
     n_atoms = int(ptr[1] - ptr[0])
     model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=5.0)
     relax = FIRE(model, dt=1.0, convergence_hook=ConvergenceHook.from_fmax(0.02))
     sinks = [GPUBuffer(capacity=8, max_atoms=n_atoms, max_edges=0, device=DEV), HostMemory(capacity=10)]
-    sampler = _ListSampler([system(s) for s in range(6)], batch_size=3)
+    # room for three systems by atoms, four by count: the atom budget is what binds
+    sampler = SizeAwareSampler(Dataset(), max_atoms=3 * n_atoms + 5, max_batch_size=4)
     left = {}
 
     class Collect:
@@ -303,7 +315,7 @@ def test_fused_stage_writes_finished_systems_to_its_sinks_in_order():
                        sinks=sinks)
     fused.register_fused_hook(Collect())
     out = fused.run(None, n_steps=2000)
-    assert out is None and fused.done and sorted(left) == list(range(6))
+    assert out is None and fused.done and sampler.exhausted and sorted(left) == list(range(6))
     assert len(sinks[0]) == 6 and len(sinks[1]) == 0
     seen = []
     for sink in sinks[:1]:
