@@ -169,6 +169,32 @@ int32_t nvamd_langevin_half_step(float* positions, float* velocities, const floa
                                  const float* friction, uint64_t random_seed, const int32_t* batch_idx,
                                  const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* stream);
 
+/* Nose-Hoover chain thermostat, half-step propagator: replaces the Warp launch behind
+ * nvalchemi::nhc_chain_update (nvalchemi/dynamics/_ops/nose_hoover.py:143-246; called before and
+ * after the velocity-Verlet core of a step, nvalchemi/dynamics/integrators/nvt_nose_hoover.py:215-281).
+ * Per system: eta, eta_dot, chain_masses (M, chain_length) f32 row-major; kT (energy units), dt,
+ * ndof (M) f32; ke2 (M) f32 receives sum m v^2 (compute_ke != 0) or supplies it (compute_ke == 0, for a
+ * caller that holds the sum over more atoms than it passes); total_scale (M) f32 receives the factor
+ * the velocities were multiplied by.  velocities, eta, eta_dot are updated in place; active (M) bytes
+ * or NULL as for velocity Verlet.  chain_length 1..16; yoshida_order 1, 3 or 5 (the reference's
+ * integrator takes 3 or 5 and defaults to 3).  The propagator is the one of Martyna, Tuckerman, Tobias
+ * and Klein (1996) with one pass of the Suzuki-Yoshida weights; chain arithmetic in double.
+ * Workspace: nvamd_nhc_workspace_bytes(n_systems). */
+int32_t nvamd_nhc_workspace_bytes(int32_t n_systems, size_t* bytes);
+int32_t nvamd_nhc_chain_update(float* velocities, const float* masses, float* eta, float* eta_dot,
+                               const float* chain_masses, const float* kT, const float* dt,
+                               const float* ndof, float* ke2, float* total_scale,
+                               const int32_t* batch_idx, const uint8_t* active, int32_t compute_ke,
+                               int32_t chain_length, int32_t yoshida_order, int32_t n_atoms,
+                               int32_t n_systems, void* workspace, size_t workspace_bytes, void* stream);
+
+/* r += v dt with the system's dt: replaces the Warp launch behind nvalchemi::nhc_position_update
+ * (nvalchemi/dynamics/_ops/nose_hoover.py:291-325).  The third op of that integrator,
+ * nvalchemi::nhc_velocity_half_step (:248-289), v += (F/m) dt/2, is nvamd_vv_velocity_finalize. */
+int32_t nvamd_nhc_position_update(float* positions, const float* velocities, const float* dt,
+                                  const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms,
+                                  int32_t n_systems, void* stream);
+
 /* Per-system maximum atomic force norm (the default convergence criterion,
  * nvalchemi/dynamics/base.py:258-349: vector_norm over xyz, scatter amax over atoms).
  * fmax (M) f32; systems without atoms give -inf. */

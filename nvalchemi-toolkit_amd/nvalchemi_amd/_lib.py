@@ -49,6 +49,9 @@ _SIGNATURES = {
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_langevin_half_step": (_i32, [_vp] * 7 + [_c.c_uint64, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_nhc_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_nhc_chain_update": (_i32, [_vp] * 12 + [_i32] * 5 + [_vp, _c.c_size_t, _vp]),
+    "nvamd_nhc_position_update": (_i32, [_vp] * 5 + [_i32, _i32, _vp]),
     "nvamd_nl_filter_matrix": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _f64, _vp, _vp, _vp, _vp]),
     "nvamd_nl_filter_coo_flags": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _c.c_int64, _f64, _vp, _vp]),
     "nvamd_buffer_workspace_bytes": (_i32, [_c.c_int64, _c.c_int64, _c.POINTER(_c.c_size_t)]),
@@ -518,3 +521,33 @@ def langevin_half_step(positions, velocities, forces, masses, dt, kT, friction, 
         _dev(friction, "friction", torch.float32, (M,)), int(random_seed) & 0xFFFFFFFFFFFFFFFF,
         _dev(batch_idx, "batch_idx", torch.int32, (N,)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
         N, M, _stream(positions.device)), "nvamd_langevin_half_step")
+
+
+# --------------------------------------------------------------------------------------------
+# Nose-Hoover chain
+# --------------------------------------------------------------------------------------------
+def nhc_chain_update(velocities, masses, eta, eta_dot, chain_masses, kT, dt, ndof, ke2, total_scale, batch_idx,
+                     compute_ke: bool = True, yoshida_order: int = 3, active=None) -> None:
+    lib = library()
+    N = velocities.shape[0]
+    M, C = eta.shape
+    ws = workspaces.get(velocities.device, "nhc", _size(lib.nvamd_nhc_workspace_bytes, M))
+    _check(lib.nvamd_nhc_chain_update(
+        _dev(velocities, "velocities", torch.float32, (N, 3)), _dev(masses, "masses", torch.float32, (N,)),
+        _dev(eta, "eta", torch.float32, (M, C)), _dev(eta_dot, "eta_dot", torch.float32, (M, C)),
+        _dev(chain_masses, "Q", torch.float32, (M, C)), _dev(kT, "temperature", torch.float32, (M,)),
+        _dev(dt, "dt", torch.float32, (M,)), _dev(ndof, "ndof", torch.float32, (M,)),
+        _dev(ke2, "ke2", torch.float32, (M,)), _dev(total_scale, "total_scale", torch.float32, (M,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
+        1 if compute_ke else 0, C, int(yoshida_order), N, M, ws.data_ptr(), ws.numel(),
+        _stream(velocities.device)), "nvamd_nhc_chain_update")
+
+
+def nhc_position_update(positions, velocities, dt, batch_idx, active=None) -> None:
+    N = positions.shape[0]
+    M = dt.shape[0]
+    _check(library().nvamd_nhc_position_update(
+        _dev(positions, "positions", torch.float32, (N, 3)), _dev(velocities, "velocities", torch.float32, (N, 3)),
+        _dev(dt, "dt", torch.float32, (M,)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _opt(_as_u8(active), "active", torch.uint8, (M,)), N, M, _stream(positions.device)),
+        "nvamd_nhc_position_update")

@@ -1,9 +1,10 @@
 from .base import BaseDynamics, ConvergenceHook, DynamicsStage, FusedStage
 from .integrators.nve import NVE
 from .integrators.nvt_langevin import NVTLangevin
+from .integrators.nvt_nose_hoover import NVTNoseHoover
 from .optimizers.fire import FIRE
 from .sampler import SizeAwareSampler
 from .sinks import DataSink, GPUBuffer, HostMemory
 
-__all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "FusedStage", "NVE", "NVTLangevin", "FIRE",
+__all__ = ["BaseDynamics", "ConvergenceHook", "DynamicsStage", "FusedStage", "NVE", "NVTLangevin", "NVTNoseHoover", "FIRE",
            "DataSink", "GPUBuffer", "HostMemory", "SizeAwareSampler"]

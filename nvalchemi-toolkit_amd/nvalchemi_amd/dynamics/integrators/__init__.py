@@ -1,4 +1,5 @@
 from .nve import NVE
 from .nvt_langevin import NVTLangevin
+from .nvt_nose_hoover import NVTNoseHoover
 
-__all__ = ["NVE", "NVTLangevin"]
+__all__ = ["NVE", "NVTLangevin", "NVTNoseHoover"]

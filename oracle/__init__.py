@@ -65,6 +65,12 @@ def lib() -> ctypes.CDLL:
         L.orc_langevin_half_step.restype = None
         L.orc_langevin_half_step.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, ctypes.c_uint64,
                                              _i32p, _u8p, ctypes.c_int32]
+        L.orc_nhc_chain_update.restype = None
+        L.orc_nhc_chain_update.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
+                                           _i32p, _u8p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                                           ctypes.c_int32, ctypes.c_int32]
+        L.orc_nhc_position_update.restype = None
+        L.orc_nhc_position_update.argtypes = [_f32p, _f32p, _f32p, _i32p, _u8p, ctypes.c_int32]
         L.orc_vv_pre.restype = None
         L.orc_vv_pre.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _i32p, _u8p, ctypes.c_int32]
         L.orc_vv_post.restype = None
@@ -544,3 +550,42 @@ def langevin_half_step(positions, velocities, forces, masses, dt, kT, friction, 
                                  _p(_f32(masses), _f32p), _p(_f32(dt), _f32p), _p(_f32(kT), _f32p),
                                  _p(_f32(friction), _f32p), int(seed), _p(_i32(batch_idx), _i32p),
                                  None if act is None else _p(act, _u8p), positions.shape[0])
+
+
+# ---------------------------------------------------------------------------------------------
+# Nose-Hoover chain (md_oracle.c: orc_nhc_chain_update)
+# ---------------------------------------------------------------------------------------------
+def nhc_masses(kT, tau, ndof, chain_length):
+    """Q (M, C): Q_1 = N_f kT tau^2, Q_k = kT tau^2 (nvalchemi/dynamics/_ops/nose_hoover.py:67-70)."""
+    kT, tau, ndof = (np.asarray(a, dtype=np.float64) for a in (kT, tau, ndof))
+    q = np.repeat((kT * tau * tau)[:, None], chain_length, axis=1)
+    q[:, 0] *= ndof
+    return q.astype(np.float32)
+
+
+def nhc_chain_update(velocities, masses, eta, eta_dot, Q, kT, dt, ndof, batch_idx, ke2=None, active=None,
+                     yoshida_order=3):
+    """In place on float32 ``velocities (N,3)``, ``eta`` and ``eta_dot (M,C)``.  With ``ke2`` given it is
+    used as sum m v^2 per system instead of the velocities.  Returns ``(ke2, total_scale)``."""
+    assert velocities.dtype == np.float32 and eta.dtype == np.float32 and eta_dot.dtype == np.float32
+    assert eta.flags.c_contiguous and eta_dot.flags.c_contiguous and velocities.flags.c_contiguous
+    M, C = eta.shape
+    assert C <= 16
+    compute = ke2 is None
+    k2 = np.zeros(M, dtype=np.float32) if compute else np.ascontiguousarray(ke2, dtype=np.float32).copy()
+    scale = np.ones(M, dtype=np.float32)
+    act = None if active is None else np.ascontiguousarray(active, dtype=np.uint8)
+    lib().orc_nhc_chain_update(_p(velocities, _f32p), _p(_f32(masses), _f32p), _p(eta, _f32p), _p(eta_dot, _f32p),
+                               _p(_f32(Q), _f32p), _p(_f32(kT), _f32p), _p(_f32(dt), _f32p), _p(_f32(ndof), _f32p),
+                               _p(k2, _f32p), _p(scale, _f32p), _p(_i32(batch_idx), _i32p),
+                               None if act is None else _p(act, _u8p), int(compute), C, int(yoshida_order),
+                               velocities.shape[0], M)
+    return k2, scale
+
+
+def nhc_position_update(positions, velocities, dt, batch_idx, active=None):
+    assert positions.dtype == np.float32
+    act = None if active is None else np.ascontiguousarray(active, dtype=np.uint8)
+    lib().orc_nhc_position_update(_p(positions, _f32p), _p(_f32(velocities), _f32p), _p(_f32(dt), _f32p),
+                                  _p(_i32(batch_idx), _i32p), None if act is None else _p(act, _u8p),
+                                  positions.shape[0])

@@ -20,6 +20,9 @@
  *   orc_vv_pre / orc_vv_post     nvalchemi/dynamics/_ops/velocity_verlet.py:63-64,112
  *   orc_langevin_half_step       nvalchemi/dynamics/_ops/langevin.py:52-117,
  *                                nvalchemi/dynamics/integrators/nvt_langevin.py:103-196
+ *   orc_nhc_chain_update         nvalchemi/dynamics/_ops/nose_hoover.py:143-246 (arguments, what is
+ *                                updated in place), nvalchemi/dynamics/integrators/nvt_nose_hoover.py
+ *                                :215-281 (chain - kick - drift | kick - chain)
  *   orc_fire_step                nvalchemi/dynamics/_ops/fire.py:245-362,
  *                                nvalchemi/dynamics/optimizers/fire.py:69-76,182-219,
  *                                nvalchemi/distributed/_dynamics_coordinator.py:296-322
@@ -57,6 +60,14 @@
  *                  step by its limits (no friction: the two half drifts of velocity Verlet; infinite
  *                  friction: velocities redrawn at kT/m) and by the invariance of the Maxwell-Boltzmann
  *                  variance under the O step.
+ *   orc_nhc_chain_update  PARITY UNPINNED against the reference: the kernel is inside the absent
+ *                  library (the reference only names it: Martyna-Tobias-Klein equations, Yoshida-Suzuki
+ *                  factorisation, chain masses Q_1 = N_f kT tau^2, Q_k = kT tau^2).  The restatement is
+ *                  the published half-step propagator of Martyna, Tuckerman, Tobias and Klein (Mol. Phys.
+ *                  87, 1117 (1996)) with one pass of the 3- or 5-weight Suzuki-Yoshida scheme.  Pinned as
+ *                  mathematics: second-order convergence of the whole step to an adaptive integration of
+ *                  the Nose-Hoover chain equations of motion, the conserved extended energy, time
+ *                  reversal, weights summing to one.
  *   orc_fmax       pinned: in-tree Torch definition is complete; literal cases.
  *   orc_rebuild_check  pinned by the reference's own cases (flags cleared on every call, 1.0 over a
  *                  threshold of 0.5 flags, 0.1 does not, per-system selectivity, reference refreshed
@@ -527,6 +538,123 @@ ORC_API void orc_langevin_half_step(float* pos, float* vel, const float* forces,
             r = r + drift;
             vel[3 * i + a] = v;
             pos[3 * i + a] = r;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Nose-Hoover chain, half-step propagator of the thermostat (Martyna, Tuckerman, Tobias, Klein 1996).
+ * Per system, with KE2 = sum m v^2, N_f degrees of freedom, chain velocities u_k (eta_dot), chain
+ * positions eta_k, masses Q_k, and d = w dt for each Suzuki-Yoshida weight w in turn:
+ *   u_C   += G_C d/4                    G_1 = (KE2 - N_f kT) / Q_1,  G_k = (Q_{k-1} u_{k-1}^2 - kT) / Q_k
+ *   k = C-1 .. 1:  u_k *= exp(-u_{k+1} d/8);  u_k += G_k d/4;  u_k *= exp(-u_{k+1} d/8)
+ *   s = exp(-u_1 d/2);  scale *= s;  KE2 *= s^2
+ *   eta_k += u_k d/2                    (every k)
+ *   k = 1 .. C-1:  u_k *= exp(-u_{k+1} d/8);  u_k += G_k d/4;  u_k *= exp(-u_{k+1} d/8)
+ *   u_C   += G_C d/4
+ * and finally v *= scale.  Called once before and once after the velocity-Verlet core of a step with
+ * the full dt, it advances the thermostat by dt/2 each time.  Chain arithmetic in double on the
+ * float32 state, results rounded once when stored; velocities are multiplied by the float32 scale.
+ * ---------------------------------------------------------------------------------------- */
+static int orc_ys_weights(int order, double* w) {
+    if (order == 3) {
+        double a = 1.0 / (2.0 - cbrt(2.0));
+        w[0] = a; w[1] = 1.0 - 2.0 * a; w[2] = a;
+        return 3;
+    }
+    if (order == 5) {
+        double a = 1.0 / (4.0 - cbrt(4.0));
+        w[0] = a; w[1] = a; w[2] = 1.0 - 4.0 * a; w[3] = a; w[4] = a;
+        return 5;
+    }
+    w[0] = 1.0;
+    return 1;
+}
+
+ORC_API void orc_nhc_chain_update(float* vel, const float* masses, float* eta, float* eta_dot, const float* Q,
+                                  const float* kT, const float* dt, const float* ndof, float* ke2,
+                                  float* total_scale, const int32_t* batch_idx, const uint8_t* active,
+                                  int32_t compute_ke, int32_t chain_length, int32_t yoshida_order,
+                                  int32_t n_atoms, int32_t n_systems) {
+    const int C = chain_length;
+    double* sum = (double*)calloc((size_t)(n_systems > 0 ? n_systems : 1), sizeof(double));
+    if (compute_ke) {
+        for (int i = 0; i < n_atoms; ++i) {
+            double vx = vel[3 * i], vy = vel[3 * i + 1], vz = vel[3 * i + 2];
+            sum[batch_idx[i]] += (double)masses[i] * ((vx * vx + vy * vy) + vz * vz);
+        }
+    } else {
+        for (int s = 0; s < n_systems; ++s) sum[s] = (double)ke2[s];
+    }
+    double w[5];
+    const int nw = orc_ys_weights(yoshida_order, w);
+    for (int s = 0; s < n_systems; ++s) {
+        if (active && !active[s]) continue;
+        double u[16], x[16], q[16];
+        for (int k = 0; k < C; ++k) {
+            u[k] = eta_dot[s * C + k];
+            x[k] = eta[s * C + k];
+            q[k] = Q[s * C + k];
+        }
+        const double kt = kT[s], nf = ndof[s], h = dt[s];
+        double k2 = sum[s], scale = 1.0;
+        if (compute_ke) ke2[s] = (float)k2;
+        for (int iw = 0; iw < nw; ++iw) {
+            const double d = w[iw] * h, d2 = 0.5 * d, d4 = 0.25 * d, d8 = 0.125 * d;
+            /* from the end of the chain to the particles */
+            {
+                double g = (C > 1) ? (q[C - 2] * u[C - 2] * u[C - 2] - kt) / q[C - 1] : (k2 - nf * kt) / q[0];
+                u[C - 1] += g * d4;
+            }
+            for (int k = C - 2; k >= 0; --k) {
+                double aa = exp(-d8 * u[k + 1]);
+                double g = (k == 0) ? (k2 - nf * kt) / q[0] : (q[k - 1] * u[k - 1] * u[k - 1] - kt) / q[k];
+                u[k] = (u[k] * aa + g * d4) * aa;
+            }
+            {
+                double sc = exp(-d2 * u[0]);
+                scale *= sc;
+                k2 *= sc * sc;
+            }
+            for (int k = 0; k < C; ++k) x[k] += d2 * u[k];
+            /* and back */
+            for (int k = 0; k < C - 1; ++k) {
+                double aa = exp(-d8 * u[k + 1]);
+                double g = (k == 0) ? (k2 - nf * kt) / q[0] : (q[k - 1] * u[k - 1] * u[k - 1] - kt) / q[k];
+                u[k] = (u[k] * aa + g * d4) * aa;
+            }
+            {
+                double g = (C > 1) ? (q[C - 2] * u[C - 2] * u[C - 2] - kt) / q[C - 1] : (k2 - nf * kt) / q[0];
+                u[C - 1] += g * d4;
+            }
+        }
+        for (int k = 0; k < C; ++k) {
+            eta_dot[s * C + k] = (float)u[k];
+            eta[s * C + k] = (float)x[k];
+        }
+        total_scale[s] = (float)scale;
+    }
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float sc = total_scale[s];
+        vel[3 * i] *= sc;
+        vel[3 * i + 1] *= sc;
+        vel[3 * i + 2] *= sc;
+    }
+    free(sum);
+}
+
+/* r += v dt (nvalchemi/dynamics/_ops/nose_hoover.py:291-325) */
+ORC_API void orc_nhc_position_update(float* pos, const float* vel, const float* dt, const int32_t* batch_idx,
+                                     const uint8_t* active, int32_t n_atoms) {
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float h = dt[s];
+        for (int a = 0; a < 3; ++a) {
+            float step = vel[3 * i + a] * h;
+            pos[3 * i + a] = pos[3 * i + a] + step;
         }
     }
 }

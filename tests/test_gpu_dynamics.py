@@ -623,3 +623,83 @@ def test_nvt_langevin_thermalises_an_lj_crystal():
         oracle.vv_post(v, f, M, dt, bi)
     close(batch.positions, p, "positions after 10 Langevin steps")
     close(batch.velocities, v, "velocities after 10 Langevin steps")
+
+
+def test_nvt_nose_hoover_follows_the_oracle_loop_thermalises_and_conserves_its_energy():
+    """``NVTNoseHoover`` on 4 FCC argon boxes: 20 steps against the oracle step loop (chain - kick -
+    drift | neighbor list + LJ | kick - chain); over a longer run the extended energy
+    KE + PE + sum Q u^2/2 + N_f kT eta_1 + kT sum_{k>1} eta_k stays put while the thermostat moves
+    energy in and out, and the kinetic temperature settles at the target."""
+    from _reference_loop import FS_PER_INTERNAL_TIME, build_and_eval
+    from nvalchemi_amd.dynamics import NVTNoseHoover
+    from nvalchemi_amd.dynamics.hooks import kinetic_energy_per_graph, temperature_per_graph
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=2, n_boxes=4, reps=4, a=5.4, jitter=0.02)
+    N = len(P)
+    Z = np.full(N, 18, dtype=np.int64)
+    M = np.full(N, 39.95, dtype=np.float32)
+    rng = np.random.default_rng(5)
+    T_target = np.array([60.0, 80.0, 100.0, 120.0], np.float32)
+    kB = 8.617333262e-5
+    bi = oracle.batch_idx_from_ptr(ptr)
+    V0 = (rng.normal(0, 1, (N, 3)) * np.sqrt(kB * 40.0 / M)[:, None]).astype(np.float32)  # 40 K everywhere
+    chain = 3
+
+    model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+    dyn = NVTNoseHoover(model, dt=2.0, temperature=torch.from_numpy(T_target), thermostat_time=50.0,
+                        chain_length=chain, yoshida_order=5, hooks=model.make_neighbor_hooks())
+    batch = make_batch(P, Z, M, C, pb, ptr, V=V0)
+    p, v, f = P.copy(), V0.copy(), np.zeros_like(P)
+    dt = np.full(4, np.float32(2.0 / FS_PER_INTERNAL_TIME), np.float32)
+    kT = (T_target * np.float32(kB)).astype(np.float32)
+    tau = np.full(4, np.float32(50.0 / FS_PER_INTERNAL_TIME), np.float32)
+    ndof = (3 * np.diff(ptr)).astype(np.float32)
+    Q = oracle.nhc_masses(kT, tau, ndof, chain)
+    eta, u = np.zeros((4, chain), np.float32), np.zeros((4, chain), np.float32)
+    K = 96
+    for step in range(20):
+        dyn.step(batch)
+        oracle.nhc_chain_update(v, M, eta, u, Q, kT, dt, ndof, bi, yoshida_order=5)
+        oracle.vv_post(v, f, M, dt, bi)
+        oracle.nhc_position_update(p, v, dt, bi)
+        out, K = build_and_eval(p, C, pb, ptr, bi, 8.0, 0.0104, 3.4, K)
+        f = out["forces"]
+        oracle.vv_post(v, f, M, dt, bi)
+        oracle.nhc_chain_update(v, M, eta, u, Q, kT, dt, ndof, bi, yoshida_order=5)
+    close(batch.positions, p, "positions after 20 Nose-Hoover steps")
+    close(batch.velocities, v, "velocities after 20 Nose-Hoover steps")
+    close(dyn._state.nhc_eta, eta, "chain positions")
+    close(dyn._state.nhc_eta_dot, u, "chain velocities")
+    assert np.allclose(dyn._state.nhc_Q.cpu().numpy(), Q, rtol=1e-6)
+
+    # ---- a longer run: the conserved quantity and the temperature
+    def extended(b, d):
+        ke = kinetic_energy_per_graph(b.velocities, b.atomic_masses, b.batch_idx, 4).double().cpu().numpy().reshape(4)
+        pe = b.energy.double().cpu().numpy().reshape(4)
+        s = d._state
+        qu = 0.5 * (s.nhc_Q.double() * s.nhc_eta_dot.double() ** 2).sum(1).cpu().numpy()
+        e = s.nhc_eta.double().cpu().numpy()
+        return ke + pe + qu + ndof * kT.astype(np.float64) * e[:, 0] + kT.astype(np.float64) * e[:, 1:].sum(1), ke
+
+    model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+    dyn = NVTNoseHoover(model, dt=2.0, temperature=torch.from_numpy(T_target), thermostat_time=50.0,
+                        hooks=model.make_neighbor_hooks())
+    batch = make_batch(P, Z, M, C, pb, ptr, V=V0)
+    dyn.step(batch)
+    h0, ke0 = extended(batch, dyn)
+    temps, drift = [], 0.0
+    steps = 1500
+    for k in range(steps):
+        dyn.step(batch)
+        if k % 50 == 49:
+            h, _ = extended(batch, dyn)
+            drift = max(drift, float(np.abs(h - h0).max()))
+        if k >= steps // 2:
+            temps.append(temperature_per_graph(batch.velocities, batch.atomic_masses, batch.batch_idx, 4,
+                                               batch.num_nodes_per_graph).cpu().numpy().reshape(4))
+    mean_t = np.mean(temps, axis=0)
+    assert np.all(np.abs(mean_t / T_target - 1) < 0.08), mean_t
+    # the heat taken up is of the order of N_f k (T_target - 20 K) / 2 ~ 1 eV per box; the sum moves by far less
+    taken = np.abs(ndof * kT * dyn._state.nhc_eta[:, 0].double().cpu().numpy())
+    assert taken.min() > 0.2 and drift < 0.01 * taken.min(), (drift, taken)

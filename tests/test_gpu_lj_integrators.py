@@ -452,3 +452,71 @@ def test_langevin_half_step_matches_oracle(masked):
     _lib.langevin_half_step(T(P), a, T(F), T(M), T(dt), T(kT), T(gamma), 1, T(bi))
     _lib.langevin_half_step(T(P), b, T(F), T(M), T(dt), T(kT), T(gamma), 2, T(bi))
     assert not torch.equal(a, b)
+
+
+@pytest.mark.parametrize("chain,order", [(1, 3), (3, 3), (3, 5), (5, 1), (16, 3)])
+def test_nhc_chain_update_and_drift_match_oracle(chain, order):
+    """The chain propagator against the oracle over many systems of very different size: chain state
+    and scale to float32 rounding (double arithmetic on both sides; only the order of the sum m v^2
+    differs), velocities the scale times the old ones bit for bit; masked systems untouched; a
+    supplied sum m v^2 used in place of the velocities' own."""
+    from nvalchemi_amd import _lib
+
+    rng = np.random.default_rng(100 + chain)
+    counts = np.array([5, 0, 300, 1, 64, 2000, 7])
+    B = len(counts)
+    bi = np.repeat(np.arange(B), counts).astype(np.int32)
+    N = len(bi)
+    V = rng.normal(0, 0.05, (N, 3)).astype(np.float32)
+    P = rng.normal(0, 3, (N, 3)).astype(np.float32)
+    M = rng.uniform(1, 60, N).astype(np.float32)
+    dt = rng.uniform(0.02, 0.2, B).astype(np.float32)
+    kT = rng.uniform(0.005, 0.05, B).astype(np.float32)
+    tau = rng.uniform(0.5, 3.0, B).astype(np.float32)
+    ndof = (3 * np.maximum(counts, 1)).astype(np.float32)
+    Q = oracle.nhc_masses(kT, tau, ndof, chain)
+    eta0 = rng.normal(0, 0.2, (B, chain)).astype(np.float32)
+    u0 = rng.normal(0, 0.3 if chain <= 5 else 0.02, (B, chain)).astype(np.float32)  # (long chains: stay finite)
+    for active, supplied in ((None, False), (np.array([1, 1, 0, 1, 1, 1, 0], np.uint8), False), (None, True)):
+        v, eta, u = V.copy(), eta0.copy(), u0.copy()
+        ke2_in = rng.uniform(0.1, 5.0, B).astype(np.float32) if supplied else None
+        ke2, scale = oracle.nhc_chain_update(v, M, eta, u, Q, kT, dt, ndof, bi, ke2=ke2_in, active=active,
+                                             yoshida_order=order)
+        tv, teta, tu = T(V), T(eta0), T(u0)
+        tke2 = T(ke2_in) if supplied else torch.zeros(B, dtype=torch.float32, device=DEV)
+        tscale = torch.ones(B, dtype=torch.float32, device=DEV)
+        _lib.nhc_chain_update(tv, T(M), teta, tu, T(Q), T(kT), T(dt), T(ndof), tke2, tscale, T(bi),
+                              compute_ke=not supplied, yoshida_order=order,
+                              active=None if active is None else T(active.astype(bool)))
+        sel = np.ones(B, bool) if active is None else active.astype(bool)
+        gs = tscale.cpu().numpy()
+        assert np.allclose(gs[sel], scale[sel], rtol=3e-7, atol=0)
+        assert np.allclose(teta.cpu().numpy(), eta, rtol=1e-6, atol=1e-7)
+        assert np.allclose(tu.cpu().numpy(), u, rtol=1e-6, atol=1e-7)
+        assert np.allclose(tke2.cpu().numpy()[sel], ke2[sel], rtol=1e-6)
+        got_v = tv.cpu().numpy()
+        asel = sel[bi]
+        assert np.array_equal(got_v[asel], (V * gs[bi][:, None])[asel])
+        assert np.array_equal(got_v[~asel], V[~asel])
+        if active is not None:
+            assert np.array_equal(teta.cpu().numpy()[~sel], eta0[~sel]) and np.array_equal(tu.cpu().numpy()[~sel], u0[~sel])
+    # the drift: one multiplication and one addition per component, bit for bit
+    p = P.copy()
+    oracle.nhc_position_update(p, V, dt, bi, active=[1, 1, 1, 1, 0, 1, 1])
+    tp = T(P)
+    _lib.nhc_position_update(tp, T(V), T(dt), T(bi), T(np.array([1, 1, 1, 1, 0, 1, 1], bool)))
+    assert np.array_equal(tp.cpu().numpy(), p)
+
+
+def test_nhc_argument_errors_come_back_as_status_codes():
+    from nvalchemi_amd import _lib
+
+    z = lambda *s: torch.zeros(*s, dtype=torch.float32, device=DEV)
+    bi = torch.zeros(4, dtype=torch.int32, device=DEV)
+    with pytest.raises(_lib.KernelLibraryError, match="yoshida_order"):
+        _lib.nhc_chain_update(z(4, 3), z(4), z(1, 2), z(1, 2), z(1, 2), z(1), z(1), z(1), z(1), z(1), bi,
+                              yoshida_order=4)
+    with pytest.raises(_lib.KernelLibraryError, match="chain_length"):
+        _lib.nhc_chain_update(z(4, 3), z(4), z(1, 17), z(1, 17), z(1, 17), z(1), z(1), z(1), z(1), z(1), bi)
+    with pytest.raises(ValueError, match="eta_dot"):
+        _lib.nhc_chain_update(z(4, 3), z(4), z(1, 2), z(1, 3), z(1, 2), z(1), z(1), z(1), z(1), z(1), bi)
