@@ -156,6 +156,24 @@ int32_t nvamd_fire_step(float* positions, float* velocities, const float* forces
                         int32_t n_systems, void* workspace, size_t workspace_bytes,
                         void* stream);
 
+/* One FIRE 2.0 step on the forces of the current positions: replaces the call into the kernel library
+ * behind fire2_step_coord (nvalchemi/dynamics/_ops/fire.py:467-557; called from
+ * nvalchemi/dynamics/optimizers/fire2.py:218-251).  positions, velocities (N,3), alpha, dt (M) f32 and
+ * nsteps_inc (M) i32 are updated in place; vf, v_sumsq, f_sumsq (sum F.v, v.v, F.F per system) and
+ * max_norm (the largest atomic displacement the step would make before the maxstep limit) are outputs
+ * and may be NULL; the hyper-parameters are scalars as in the reference.  Unit masses (the reference's
+ * op takes none).  active (M) bytes or NULL as for velocity Verlet.  The algorithm is FIRE 2.0 as
+ * published with its LAMMPS implementation (Guenole et al. 2020): semi-implicit Euler, half step back
+ * on a reset.  Workspace: nvamd_fire2_workspace_bytes(n_systems). */
+int32_t nvamd_fire2_workspace_bytes(int32_t n_systems, size_t* bytes);
+int32_t nvamd_fire2_step(float* positions, float* velocities, const float* forces,
+                         const int32_t* batch_idx, float* alpha, float* dt, int32_t* nsteps_inc,
+                         float* vf, float* v_sumsq, float* f_sumsq, float* max_norm,
+                         int32_t delaystep, double dtgrow, double dtshrink, double alphashrink,
+                         double alpha0, double tmax, double tmin, double maxstep,
+                         const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
 /* BAOAB Langevin pre-force half step B-A-O-A: replaces the Warp launch behind
  * nvalchemi::langevin_half_step (nvalchemi/dynamics/_ops/langevin.py:52-117; called from
  * nvalchemi/dynamics/integrators/nvt_langevin.py:160-181).  kT (M) f32 in energy units,

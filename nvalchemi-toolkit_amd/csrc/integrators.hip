@@ -304,6 +304,146 @@ __global__ __launch_bounds__(kBlock) void fire_update_kernel(
     }
 }
 
+// ---- FIRE 2.0 -------------------------------------------------------------------------------
+// Reference interface: fire2_step_coord (nvalchemi/dynamics/_ops/fire.py:467-557), called by
+// FIRE2.pre_update (nvalchemi/dynamics/optimizers/fire2.py:218-251).  The reference's step is in its
+// kernel library; this is FIRE 2.0 as published with its LAMMPS implementation (Guenole et al.
+// 2020): semi-implicit Euler, half step back on a reset, unit masses, no initial delay:
+//   P > 0 :  a = 1 - alpha, b = alpha sqrt(VV / FF); count += 1; past delaystep: dt grows, alpha decays
+//   P <= 0:  count = 0; alpha = alpha0; r -= (dt/2) v; v = 0; dt shrinks while it stays >= tmin
+//   v += dt F;  P > 0: v = a v + b F;  dr = dt v, the whole system's step scaled so that its
+//   largest atomic displacement stays within maxstep.
+struct Fire2Scratch {
+    double* acc;   // (M,3): sum F.v, sum v.v, sum F.F
+    float* mix_a;  // (M) factor on the kicked v
+    float* mix_b;  // (M) factor on F
+    float* back;   // (M) length of the step back (0: none)
+    float* big;    // (M) largest |dr| of the system
+    int32_t* up;   // (M) P > 0
+};
+
+struct Fire2Params {
+    int delaystep;
+    float dtgrow, dtshrink, alphashrink, alpha0, tmax, tmin, maxstep;
+};
+
+__global__ __launch_bounds__(kBlock) void fire2_params_kernel(float* __restrict__ alpha, float* __restrict__ dt,
+                                                              int32_t* __restrict__ count, float* vf, float* vv,
+                                                              float* ff, const uint8_t* __restrict__ active,
+                                                              Fire2Scratch ws, Fire2Params p, int m) {
+    int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    const double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+    if (vf) vf[s] = (float)P;
+    if (vv) vv[s] = (float)VV;
+    if (ff) ff[s] = (float)FF;
+    float ma = 1.0f, mb = 0.0f, bk = 0.0f;
+    int up = 0;
+    if (!active || active[s]) {
+        if (P > 0.0) {
+            const float al = alpha[s];
+            up = 1;
+            ma = 1.0f - al;
+            mb = (FF > 1e-20) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
+            const int c = count[s] + 1;
+            count[s] = c;
+            if (c > p.delaystep) {
+                const float nd = dt[s] * p.dtgrow;
+                dt[s] = nd < p.tmax ? nd : p.tmax;
+                alpha[s] = al * p.alphashrink;
+            }
+        } else {
+            count[s] = 0;
+            alpha[s] = p.alpha0;
+            bk = 0.5f * dt[s];
+            const float nd = dt[s] * p.dtshrink;
+            if (nd >= p.tmin) dt[s] = nd;
+        }
+    }
+    ws.mix_a[s] = ma;
+    ws.mix_b[s] = mb;
+    ws.back[s] = bk;
+    ws.big[s] = 0.0f;
+    ws.up[s] = up;
+}
+
+// new velocities (and the step back), and the largest displacement they would give
+__global__ __launch_bounds__(kBlock) void fire2_kick_kernel(float* __restrict__ pos, float* __restrict__ vel,
+                                                            const float* __restrict__ frc,
+                                                            const float* __restrict__ dt,
+                                                            const int32_t* __restrict__ bidx,
+                                                            const uint8_t* __restrict__ active, Fire2Scratch ws,
+                                                            int n_atoms) {
+#pragma clang fp contract(off)
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    int seg = -1 - (i - n_atoms);
+    float nrm = 0.0f;
+    bool live = false;
+    if (i < n_atoms) {
+        const int s = bidx[i];
+        seg = s;
+        live = !active || active[s];
+        if (live) {
+            const float h = dt[s], ma = ws.mix_a[s], mb = ws.mix_b[s], bk = ws.back[s];
+            const bool up = ws.up[s] != 0;
+            const size_t b = 3 * (size_t)i;
+            float dr[3];
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                const float f = frc[b + a];
+                float v = vel[b + a];
+                if (!up) {
+                    const float undo = bk * v;
+                    pos[b + a] = pos[b + a] - undo;
+                    v = 0.0f;
+                }
+                const float kick = h * f;
+                v = v + kick;
+                if (up) {
+                    const float va = ma * v, fb = mb * f;
+                    v = va + fb;
+                }
+                v = fminf(fmaxf(v, -kFireVmax), kFireVmax);
+                vel[b + a] = v;
+                dr[a] = h * v;
+            }
+            const float top = fmaxf(fmaxf(fabsf(dr[0]), fabsf(dr[1])), fabsf(dr[2]));
+            if (top > 0.0f) {
+                const float a0 = dr[0] / top, a1 = dr[1] / top, a2 = dr[2] / top;
+                nrm = top * sqrtf((a0 * a0 + a1 * a1) + a2 * a2);
+            } else if (top != top) {
+                nrm = top;
+            }
+        }
+    }
+    const bool head = wave_segmented_max(seg, nrm);
+    // norms are >= 0 or NaN: their bit patterns order like signed integers, NaN above all
+    if (head && i < n_atoms && (!active || active[seg]))
+        atomicMax(reinterpret_cast<int*>(ws.big) + seg, __float_as_int(nrm));
+}
+
+__global__ __launch_bounds__(kBlock) void fire2_drift_kernel(float* __restrict__ pos, const float* __restrict__ vel,
+                                                             const float* __restrict__ dt,
+                                                             const int32_t* __restrict__ bidx,
+                                                             const uint8_t* __restrict__ active, Fire2Scratch ws,
+                                                             float maxstep, float* __restrict__ max_norm, int n_atoms) {
+#pragma clang fp contract(off)
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_atoms) return;
+    const int s = bidx[i];
+    if (active && !active[s]) return;
+    const float h = dt[s], big = ws.big[s];
+    const float sc = big > maxstep ? maxstep / big : 1.0f;
+    const size_t b = 3 * (size_t)i;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        float dr = h * vel[b + a];
+        dr = dr * sc;
+        pos[b + a] = pos[b + a] + dr;
+    }
+    if (max_norm && (i == 0 || bidx[i - 1] != s)) max_norm[s] = big;
+}
+
 // ---- per-system max force norm ------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void fmax_init_kernel(float* fmax, int m) {
     int s = blockIdx.x * kBlock + threadIdx.x;
@@ -413,6 +553,63 @@ NVAMD_EXPORT int32_t nvamd_fire_step(float* positions, float* velocities, const 
         hipLaunchKernelGGL(fire_update_kernel, grid_n, blk, 0, st, positions, velocities, forces, masses,
                            maxstep, batch_idx, active, ws, n_atoms);
     NVAMD_LAUNCH_CHECK("fire launch");
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_fire2_workspace_bytes(int32_t n_systems, size_t* bytes) {
+    if (!bytes || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2 workspace: bad argument");
+    size_t m = (size_t)(n_systems > 0 ? n_systems : 1);
+    *bytes = align_up(m * 3 * sizeof(double)) + 5 * align_up(m * sizeof(float));
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_fire2_step(float* positions, float* velocities, const float* forces,
+                                      const int32_t* batch_idx, float* alpha, float* dt, int32_t* nsteps_inc,
+                                      float* vf, float* v_sumsq, float* f_sumsq, float* max_norm,
+                                      int32_t delaystep, double dtgrow, double dtshrink, double alphashrink,
+                                      double alpha0, double tmax, double tmin, double maxstep,
+                                      const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2: negative size");
+    if (n_systems == 0) return NVAMD_OK;
+    if (!alpha || !dt || !nsteps_inc) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2: null per-system buffer");
+    if (n_atoms > 0 && (!positions || !velocities || !forces || !batch_idx))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2: null per-atom buffer");
+    size_t need = 0;
+    nvamd_fire2_workspace_bytes(n_systems, &need);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "fire2: workspace %zu < %zu bytes", workspace_bytes, need);
+    const size_t m = (size_t)n_systems;
+    char* w = static_cast<char*>(workspace);
+    Fire2Scratch ws;
+    ws.acc = reinterpret_cast<double*>(w);
+    w += align_up(m * 3 * sizeof(double));
+    ws.mix_a = reinterpret_cast<float*>(w);
+    w += align_up(m * sizeof(float));
+    ws.mix_b = reinterpret_cast<float*>(w);
+    w += align_up(m * sizeof(float));
+    ws.back = reinterpret_cast<float*>(w);
+    w += align_up(m * sizeof(float));
+    ws.big = reinterpret_cast<float*>(w);
+    w += align_up(m * sizeof(float));
+    ws.up = reinterpret_cast<int32_t*>(w);
+    const Fire2Params p{delaystep, (float)dtgrow, (float)dtshrink, (float)alphashrink, (float)alpha0,
+                        (float)tmax, (float)tmin, (float)maxstep};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 blk(kBlock), grid_m((n_systems + kBlock - 1) / kBlock), grid_n((n_atoms + kBlock - 1) / kBlock);
+    const int n3 = 3 * n_systems;
+    hipLaunchKernelGGL(fire_clear_kernel, dim3((n3 + kBlock - 1) / kBlock), blk, 0, st, ws.acc, n3);
+    if (n_atoms > 0)
+        hipLaunchKernelGGL(fire_reduce_kernel, grid_n, blk, 0, st, velocities, forces, batch_idx, ws.acc, n_atoms);
+    hipLaunchKernelGGL(fire2_params_kernel, grid_m, blk, 0, st, alpha, dt, nsteps_inc, vf, v_sumsq, f_sumsq, active,
+                       ws, p, n_systems);
+    if (n_atoms > 0) {
+        hipLaunchKernelGGL(fire2_kick_kernel, grid_n, blk, 0, st, positions, velocities, forces, dt, batch_idx,
+                           active, ws, n_atoms);
+        hipLaunchKernelGGL(fire2_drift_kernel, grid_n, blk, 0, st, positions, velocities, dt, batch_idx, active, ws,
+                           (float)maxstep, max_norm, n_atoms);
+    }
+    NVAMD_LAUNCH_CHECK("fire2 launch");
     return NVAMD_OK;
 }
 

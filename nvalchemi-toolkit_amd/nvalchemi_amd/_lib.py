@@ -49,6 +49,8 @@ _SIGNATURES = {
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_langevin_half_step": (_i32, [_vp] * 7 + [_c.c_uint64, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_fire2_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_fire2_step": (_i32, [_vp] * 11 + [_i32] + [_c.c_double] * 7 + [_vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
     "nvamd_nhc_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_nhc_chain_update": (_i32, [_vp] * 12 + [_i32] * 5 + [_vp, _c.c_size_t, _vp]),
     "nvamd_nhc_position_update": (_i32, [_vp] * 5 + [_i32, _i32, _vp]),
@@ -551,3 +553,25 @@ def nhc_position_update(positions, velocities, dt, batch_idx, active=None) -> No
         _dev(dt, "dt", torch.float32, (M,)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         _opt(_as_u8(active), "active", torch.uint8, (M,)), N, M, _stream(positions.device)),
         "nvamd_nhc_position_update")
+
+
+# --------------------------------------------------------------------------------------------
+# FIRE 2.0
+# --------------------------------------------------------------------------------------------
+def fire2_step(positions, velocities, forces, batch_idx, alpha, dt, nsteps_inc, vf=None, v_sumsq=None,
+               f_sumsq=None, max_norm=None, *, delaystep: int, dtgrow: float, dtshrink: float, alphashrink: float,
+               alpha0: float, tmax: float, tmin: float, maxstep: float, active=None) -> None:
+    lib = library()
+    N = positions.shape[0]
+    M = dt.shape[0]
+    ws = workspaces.get(positions.device, "fire2", _size(lib.nvamd_fire2_workspace_bytes, M))
+    _check(lib.nvamd_fire2_step(
+        _dev(positions, "positions", torch.float32, (N, 3)), _dev(velocities, "velocities", torch.float32, (N, 3)),
+        _dev(forces, "forces", torch.float32, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _dev(alpha, "alpha", torch.float32, (M,)), _dev(dt, "dt", torch.float32, (M,)),
+        _dev(nsteps_inc, "nsteps_inc", torch.int32, (M,)), _opt(vf, "vf", torch.float32, (M,)),
+        _opt(v_sumsq, "v_sumsq", torch.float32, (M,)), _opt(f_sumsq, "f_sumsq", torch.float32, (M,)),
+        _opt(max_norm, "max_norm", torch.float32, (M,)), int(delaystep), float(dtgrow), float(dtshrink),
+        float(alphashrink), float(alpha0), float(tmax), float(tmin), float(maxstep),
+        _opt(_as_u8(active), "active", torch.uint8, (M,)), N, M, ws.data_ptr(), ws.numel(),
+        _stream(positions.device)), "nvamd_fire2_step")

@@ -19,7 +19,7 @@ import torch
 
 from ... import _lib
 
-__all__ = ["fire_step"]
+__all__ = ["fire_step", "fire2_step_coord"]
 
 
 @torch.library.custom_op(
@@ -67,3 +67,28 @@ def fire_step(positions: torch.Tensor, velocities: torch.Tensor, forces: torch.T
     _lib.fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_alpha, dt_min, dt_max,
                    maxstep, n_steps_positive, n_min, f_dec, f_inc, uphill_flag, vf, vv, ff, batch_idx,
                    compute_reductions, active)
+
+
+def fire2_step_coord(positions: torch.Tensor, velocities: torch.Tensor, forces: torch.Tensor,
+                     batch_idx: torch.Tensor, alpha: torch.Tensor, dt: torch.Tensor, nsteps_inc: torch.Tensor, *,
+                     vf: torch.Tensor | None = None, v_sumsq: torch.Tensor | None = None,
+                     f_sumsq: torch.Tensor | None = None, max_norm: torch.Tensor | None = None,
+                     delaystep: int = 60, dtgrow: float = 1.05, dtshrink: float = 0.75, alphashrink: float = 0.985,
+                     alpha0: float = 0.09, tmax: float = 0.08, tmin: float = 0.005, maxstep: float = 0.1,
+                     active: torch.Tensor | None = None) -> None:
+    """One FIRE 2.0 step with fixed cells; same arguments and defaults as ``fire2_step_coord`` of
+    nvalchemi/dynamics/_ops/fire.py:467-557.  Mutates ``positions``, ``velocities``, ``alpha``, ``dt``,
+    ``nsteps_inc`` and, when given, the outputs ``vf``, ``v_sumsq``, ``f_sumsq`` (sum F.v, v.v, F.F per
+    system at entry) and ``max_norm`` (largest atomic displacement before the ``maxstep`` limit).
+    ``active [M] bool`` (extension): systems with ``False`` are left untouched.
+
+    The reference delegates the step to its kernel library; what runs here is FIRE 2.0 as published
+    with its LAMMPS implementation (Guenole et al. 2020), semi-implicit Euler with unit masses:
+    downhill (``sum F.v > 0``) the velocity is kicked, then mixed with the force direction; past
+    ``delaystep`` downhill steps in a row ``dt`` grows (up to ``tmax``) and ``alpha`` decays; otherwise
+    the positions go half a step back, the velocities restart from zero, ``alpha`` from ``alpha0`` and
+    ``dt`` shrinks (not below ``tmin``).  A system's step is scaled down so that no atom moves further
+    than ``maxstep``."""
+    _lib.fire2_step(positions, velocities, forces, batch_idx, alpha, dt, nsteps_inc, vf, v_sumsq, f_sumsq, max_norm,
+                    delaystep=delaystep, dtgrow=dtgrow, dtshrink=dtshrink, alphashrink=alphashrink, alpha0=alpha0,
+                    tmax=tmax, tmin=tmin, maxstep=maxstep, active=active)

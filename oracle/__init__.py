@@ -65,6 +65,9 @@ def lib() -> ctypes.CDLL:
         L.orc_langevin_half_step.restype = None
         L.orc_langevin_half_step.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, ctypes.c_uint64,
                                              _i32p, _u8p, ctypes.c_int32]
+        L.orc_fire2_step.restype = None
+        L.orc_fire2_step.argtypes = [_f32p, _f32p, _f32p, _i32p, _f32p, _f32p, _i32p, _f32p, _f32p, _f32p, _f32p,
+                                     ctypes.c_int32] + [ctypes.c_double] * 7 + [_u8p, ctypes.c_int32, ctypes.c_int32]
         L.orc_nhc_chain_update.restype = None
         L.orc_nhc_chain_update.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
                                            _i32p, _u8p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
@@ -589,3 +592,30 @@ def nhc_position_update(positions, velocities, dt, batch_idx, active=None):
     lib().orc_nhc_position_update(_p(positions, _f32p), _p(_f32(velocities), _f32p), _p(_f32(dt), _f32p),
                                   _p(_i32(batch_idx), _i32p), None if act is None else _p(act, _u8p),
                                   positions.shape[0])
+
+
+# ---------------------------------------------------------------------------------------------
+# FIRE 2.0 (md_oracle.c: orc_fire2_step)
+# ---------------------------------------------------------------------------------------------
+FIRE2_DEFAULTS = dict(delaystep=60, dtgrow=1.05, dtshrink=0.75, alphashrink=0.985, alpha0=0.09, tmax=0.08,
+                      tmin=0.005, maxstep=0.1)  # nvalchemi/dynamics/optimizers/fire2.py:54-63
+
+
+def fire2_step(positions, velocities, forces, batch_idx, alpha, dt, nsteps_inc, active=None, **params):
+    """In place on float32 ``positions``, ``velocities`` (N,3), ``alpha``, ``dt`` (M) and int32
+    ``nsteps_inc`` (M).  Returns ``dict(vf, v_sumsq, f_sumsq, max_norm)`` (M each)."""
+    for a in (positions, velocities, alpha, dt):
+        assert a.dtype == np.float32 and a.flags.c_contiguous
+    assert nsteps_inc.dtype == np.int32
+    p = dict(FIRE2_DEFAULTS)
+    p.update(params)
+    M = alpha.shape[0]
+    out = {k: np.zeros(M, dtype=np.float32) for k in ("vf", "v_sumsq", "f_sumsq", "max_norm")}
+    act = None if active is None else np.ascontiguousarray(active, dtype=np.uint8)
+    lib().orc_fire2_step(_p(positions, _f32p), _p(velocities, _f32p), _p(_f32(forces), _f32p),
+                         _p(_i32(batch_idx), _i32p), _p(alpha, _f32p), _p(dt, _f32p), _p(nsteps_inc, _i32p),
+                         _p(out["vf"], _f32p), _p(out["v_sumsq"], _f32p), _p(out["f_sumsq"], _f32p),
+                         _p(out["max_norm"], _f32p), int(p["delaystep"]), float(p["dtgrow"]), float(p["dtshrink"]),
+                         float(p["alphashrink"]), float(p["alpha0"]), float(p["tmax"]), float(p["tmin"]),
+                         float(p["maxstep"]), None if act is None else _p(act, _u8p), positions.shape[0], M)
+    return out

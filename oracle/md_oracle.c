@@ -26,6 +26,9 @@
  *   orc_fire_step                nvalchemi/dynamics/_ops/fire.py:245-362,
  *                                nvalchemi/dynamics/optimizers/fire.py:69-76,182-219,
  *                                nvalchemi/distributed/_dynamics_coordinator.py:296-322
+ *   orc_fire2_step               nvalchemi/dynamics/_ops/fire.py:467-557 (arguments, defaults, what is
+ *                                updated in place), nvalchemi/dynamics/optimizers/fire2.py:18-27,218-251
+ *                                (the whole step before the forces, nothing after them)
  *   orc_fmax                     nvalchemi/dynamics/base.py:304-349
  *   orc_rebuild_check            nvalchemi/dynamics/_ops/neighbor_list_rebuild.py:37-139 (the
  *                                displacement kernel itself is in the absent wheel)
@@ -60,6 +63,17 @@
  *                  step by its limits (no friction: the two half drifts of velocity Verlet; infinite
  *                  friction: velocities redrawn at kT/m) and by the invariance of the Maxwell-Boltzmann
  *                  variance under the O step.
+ *   orc_fire2_step  PARITY UNPINNED against the reference: the step is inside the absent library.  The
+ *                  parameter names (delaystep, dtgrow, dtshrink, alphashrink, alpha0, tmax, tmin) are those of
+ *                  FIRE 2.0 as published with its LAMMPS implementation (Guenole et al., Comput. Mater. Sci.
+ *                  175, 109584 (2020)); the restatement follows that algorithm with the semi-implicit Euler
+ *                  integrator, the half step back on a reset, unit masses (the reference's op takes none) and
+ *                  no initial delay (its state holds no step count).  Taken without evidence: mixing factors
+ *                  from the alpha and |v| of the entry, applied after the kick; the half step back with the
+ *                  time step before its reduction; maxstep as a limit on the largest atomic displacement of
+ *                  a system, by scaling the whole system's step.  Checked by what the algorithm fixes (the
+ *                  Euler limit, the reset, the bounds on dt and on the displacement, the counter) and by
+ *                  reaching the minimum.
  *   orc_nhc_chain_update  PARITY UNPINNED against the reference: the kernel is inside the absent
  *                  library (the reference only names it: Martyna-Tobias-Klein equations, Yoshida-Suzuki
  *                  factorisation, chain masses Q_1 = N_f kT tau^2, Q_k = kT tau^2).  The restatement is
@@ -540,6 +554,109 @@ ORC_API void orc_langevin_half_step(float* pos, float* vel, const float* forces,
             pos[3 * i + a] = r;
         }
     }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * FIRE 2.0, one step on the forces of the current positions (unit masses):
+ *   P = sum F.v, VV = sum v.v, FF = sum F.F per system (double)
+ *   P > 0 :  a = 1 - alpha, b = alpha sqrt(VV / FF)  (0 when FF <= 1e-20);  count += 1;
+ *            count > delaystep:  dt = min(dt dtgrow, tmax), alpha *= alphashrink
+ *   P <= 0:  count = 0; alpha = alpha0; back = dt / 2; dt dtshrink >= tmin: dt *= dtshrink;
+ *            r -= back v; v = 0
+ *   v += dt F;   P > 0: v = a v + b F;   dr = dt v
+ *   m = largest |dr_i| of the system;  m > maxstep: dr *= maxstep / m;   r += dr
+ * float32 per-atom arithmetic, one rounding per operation; the sums in double.
+ * ---------------------------------------------------------------------------------------- */
+ORC_API void orc_fire2_step(float* pos, float* vel, const float* forces, const int32_t* batch_idx, float* alpha,
+                            float* dt, int32_t* nsteps_inc, float* vf, float* v_sumsq, float* f_sumsq,
+                            float* max_norm, int32_t delaystep, double dtgrow, double dtshrink, double alphashrink,
+                            double alpha0, double tmax, double tmin, double maxstep, const uint8_t* active,
+                            int32_t n_atoms, int32_t n_systems) {
+    const size_t M = (size_t)(n_systems > 0 ? n_systems : 1);
+    double* acc = (double*)calloc(M * 3, sizeof(double));
+    float* mixa = (float*)malloc(sizeof(float) * M);
+    float* mixb = (float*)malloc(sizeof(float) * M);
+    float* back = (float*)malloc(sizeof(float) * M);
+    float* big = (float*)calloc(M, sizeof(float));
+    uint8_t* up = (uint8_t*)calloc(M, 1);
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        for (int a = 0; a < 3; ++a) {
+            double v = vel[3 * i + a], f = forces[3 * i + a];
+            acc[3 * s + 0] += f * v;
+            acc[3 * s + 1] += v * v;
+            acc[3 * s + 2] += f * f;
+        }
+    }
+    for (int s = 0; s < n_systems; ++s) {
+        double P = acc[3 * s], VV = acc[3 * s + 1], FF = acc[3 * s + 2];
+        if (vf) vf[s] = (float)P;
+        if (v_sumsq) v_sumsq[s] = (float)VV;
+        if (f_sumsq) f_sumsq[s] = (float)FF;
+        mixa[s] = 1.0f; mixb[s] = 0.0f; back[s] = 0.0f;
+        if (active && !active[s]) continue;
+        if (P > 0.0) {
+            float al = alpha[s];
+            up[s] = 1;
+            mixa[s] = 1.0f - al;
+            mixb[s] = (FF > 1e-20) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
+            nsteps_inc[s] += 1;
+            if (nsteps_inc[s] > delaystep) {
+                float nd = dt[s] * (float)dtgrow;
+                dt[s] = nd < (float)tmax ? nd : (float)tmax;
+                alpha[s] = al * (float)alphashrink;
+            }
+        } else {
+            nsteps_inc[s] = 0;
+            alpha[s] = (float)alpha0;
+            back[s] = 0.5f * dt[s];
+            float nd = dt[s] * (float)dtshrink;
+            if (nd >= (float)tmin) dt[s] = nd;
+        }
+    }
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float h = dt[s], dr[3];
+        for (int a = 0; a < 3; ++a) {
+            float f = forces[3 * i + a], v = vel[3 * i + a];
+            if (!up[s]) {
+                float undo = back[s] * v;
+                pos[3 * i + a] = pos[3 * i + a] - undo;
+                v = 0.0f;
+            }
+            float kick = h * f;
+            v = v + kick;
+            if (up[s]) {
+                float va = mixa[s] * v, fb = mixb[s] * f;
+                v = va + fb;
+            }
+            v = fminf(fmaxf(v, -ORC_VMAX), ORC_VMAX);
+            vel[3 * i + a] = v;
+            dr[a] = h * v;
+        }
+        float top = fmaxf(fmaxf(fabsf(dr[0]), fabsf(dr[1])), fabsf(dr[2]));
+        float nrm = 0.0f;
+        if (top > 0.0f) {
+            float a0 = dr[0] / top, a1 = dr[1] / top, a2 = dr[2] / top;
+            nrm = top * sqrtf((a0 * a0 + a1 * a1) + a2 * a2);
+        }
+        if (nrm > big[s] || nrm != nrm) big[s] = nrm;
+    }
+    for (int s = 0; s < n_systems; ++s)
+        if (max_norm && !(active && !active[s])) max_norm[s] = big[s];
+    for (int i = 0; i < n_atoms; ++i) {
+        int s = batch_idx[i];
+        if (active && !active[s]) continue;
+        float h = dt[s];
+        float sc = big[s] > (float)maxstep ? (float)maxstep / big[s] : 1.0f;
+        for (int a = 0; a < 3; ++a) {
+            float dr = h * vel[3 * i + a];
+            dr = dr * sc;
+            pos[3 * i + a] = pos[3 * i + a] + dr;
+        }
+    }
+    free(acc); free(mixa); free(mixb); free(back); free(big); free(up);
 }
 
 /* ------------------------------------------------------------------------------------------

@@ -520,3 +520,54 @@ def test_nhc_argument_errors_come_back_as_status_codes():
         _lib.nhc_chain_update(z(4, 3), z(4), z(1, 17), z(1, 17), z(1, 17), z(1), z(1), z(1), z(1), z(1), bi)
     with pytest.raises(ValueError, match="eta_dot"):
         _lib.nhc_chain_update(z(4, 3), z(4), z(1, 2), z(1, 3), z(1, 2), z(1), z(1), z(1), z(1), z(1), bi)
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_fire2_step_matches_oracle_over_many_steps(masked):
+    """FIRE 2.0 against the oracle for 60 steps on harmonic wells of very different stiffness and size
+    (so that systems are downhill, uphill, limited by maxstep and past the delay at different times):
+    per-system state equal, positions and velocities to float32 rounding (the sums differ in order)."""
+    from nvalchemi_amd import _lib
+
+    rng = np.random.default_rng(21)
+    counts = np.array([5, 0, 300, 1, 64, 2000, 7])
+    B = len(counts)
+    bi = np.repeat(np.arange(B), counts).astype(np.int32)
+    N = len(bi)
+    k = (np.array([1.0, 1.0, 30.0, 5.0, 200.0, 0.5, 2000.0])[bi][:, None] * (0.5 + rng.random((N, 3)))).astype(np.float32)
+    P = rng.normal(0, 1.0, (N, 3)).astype(np.float32)
+    V = rng.normal(0, 0.5, (N, 3)).astype(np.float32)
+    active = np.array([1, 1, 0, 1, 1, 1, 1], np.uint8) if masked else None
+    params = dict(delaystep=4, dtgrow=1.1, dtshrink=0.5, alphashrink=0.99, alpha0=0.1, tmax=0.06, tmin=0.002,
+                  maxstep=0.05)
+    p, v = P.copy(), V.copy()
+    alpha, dt, cnt = np.full(B, 0.1, np.float32), np.full(B, 0.02, np.float32), np.zeros(B, np.int32)
+    tp, tv = T(P), T(V)
+    talpha, tdt, tcnt = T(alpha), T(dt), T(cnt)
+    outs = {n: torch.zeros(B, dtype=torch.float32, device=DEV) for n in ("vf", "v_sumsq", "f_sumsq", "max_norm")}
+    seen_up, seen_down, seen_limit = set(), set(), set()
+    for step in range(60):
+        f = (-k * p).astype(np.float32)
+        tf = -T(k) * tp
+        assert np.allclose(tf.cpu().numpy(), f, rtol=1e-4, atol=1e-5)
+        out = oracle.fire2_step(p, v, f, bi, alpha, dt, cnt, active=active, **params)
+        _lib.fire2_step(tp, tv, T(f), T(bi), talpha, tdt, tcnt, outs["vf"], outs["v_sumsq"], outs["f_sumsq"],
+                        outs["max_norm"], active=None if active is None else T(active.astype(bool)), **params)
+        # the trajectories are kept together: the next step starts from the oracle's state
+        assert np.allclose(tv.cpu().numpy(), v, rtol=2e-5, atol=1e-6), step
+        assert np.allclose(tp.cpu().numpy(), p, rtol=2e-5, atol=1e-6), step
+        assert np.array_equal(tcnt.cpu().numpy(), cnt) and np.array_equal(tdt.cpu().numpy(), dt), step
+        assert np.array_equal(talpha.cpu().numpy(), alpha), step
+        for n in ("vf", "v_sumsq", "f_sumsq"):
+            assert np.allclose(outs[n].cpu().numpy(), out[n], rtol=1e-5, atol=1e-7), (step, n)
+        live = (counts > 0) & (np.ones(B, bool) if active is None else active.astype(bool))
+        assert np.allclose(outs["max_norm"].cpu().numpy()[live], out["max_norm"][live], rtol=2e-5, atol=1e-8)
+        seen_up |= set(np.flatnonzero(out["vf"] > 0))
+        seen_down |= set(np.flatnonzero((out["vf"] <= 0) & live))
+        seen_limit |= set(np.flatnonzero(out["max_norm"] > params["maxstep"]))
+        tp.copy_(T(p)); tv.copy_(T(v))
+    assert len(seen_up) >= 4 and len(seen_down) >= 4 and len(seen_limit) >= 3 and cnt.max() > 4
+    if masked:
+        sel = bi == 2
+        assert np.array_equal(tp.cpu().numpy()[sel], P[sel]) and np.array_equal(tv.cpu().numpy()[sel], V[sel])
+        assert tdt.cpu().numpy()[2] == np.float32(0.02) and tcnt.cpu().numpy()[2] == 0
