@@ -85,7 +85,9 @@ class SegmentedGroup:
 
     @property
     def batch_ptr(self) -> torch.Tensor:
-        return self._ptr_store()[: len(self) + 1]
+        store = self._ptr_store()
+        n = len(self) + 1
+        return store if store.shape[0] == n else store[:n]
 
     @property
     def batch_idx(self) -> torch.Tensor:
@@ -488,7 +490,9 @@ class Batch:
         ref = cls.from_data_list([template], device=dev) if isinstance(template, AtomicData) else template
         groups: dict[str, Any] = {}
         for name, group in ref._storage.groups.items():
-            keys = list(group.keys())
+            # (the per-atom neighbor data of the template is left out: put never carries it, and at
+            # K entries per atom it would be most of the allocation)
+            keys = [k for k in group.keys() if k not in _NEIGHBOR_MATRIX_KEYS]
             if not keys:
                 continue
             rows = num_systems if name == "system" else num_nodes if name == "atoms" else num_edges

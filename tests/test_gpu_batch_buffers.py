@@ -317,6 +317,8 @@ def test_fused_stage_writes_finished_systems_to_its_sinks_in_order():
     out = fused.run(None, n_steps=2000)
     assert out is None and fused.done and sampler.exhausted and sorted(left) == list(range(6))
     assert len(sinks[0]) == 6 and len(sinks[1]) == 0
+    # the batch carried the hook's neighbor matrix; the buffer does not allocate room for it
+    assert "neighbor_matrix" not in sinks[0]._buffer and "positions" in sinks[0]._buffer
     seen = []
     for sink in sinks[:1]:
         stored = sink.read()
