@@ -142,6 +142,8 @@ class _Workspaces:
         self._bufs: dict[tuple, torch.Tensor] = {}
 
     def get(self, device: torch.device, purpose: str, nbytes: int) -> torch.Tensor:
+        if torch.device(device).type != "cuda":
+            raise KernelLibraryError(f"tensors are on {device}; the nvalchemi_amd kernels run on a ROCm device only")
         key = (device.index, _stream(device), purpose)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:

@@ -754,3 +754,88 @@ def test_fire2_relaxation_matches_oracle_and_reaches_the_minimum():
     assert np.ptp(per_atom) < 2e-6 * abs(per_atom.mean()) + 1e-7, per_atom
     fm = np.linalg.norm(batch.forces.cpu().numpy(), axis=1).max()
     assert fm < 1e-3
+
+
+def test_integrator_state_follows_its_systems_through_a_refill():
+    """Restating test/dynamics/test_state_management.py:633-849: after ``refill_check`` the per-system
+    state has one row per system of the new batch -- the rows of the systems that stay, in order and
+    unchanged, then fresh rows for the newcomers -- for a plain integrator and for every sub-stage of
+    a fused stage; when nothing is left the state is dropped and the run is done."""
+    from nvalchemi_amd.data import AtomicData, Batch
+    from nvalchemi_amd.dynamics import FIRE, NVE, FusedStage
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=3, n_boxes=5, reps=2, a=5.4, jitter=0.1)
+
+    def system(s):
+        a0, a1 = int(ptr[s]), int(ptr[s + 1])
+        n = a1 - a0
+        return AtomicData(torch.from_numpy(P[a0:a1]), torch.full((n,), 18), atomic_masses=torch.full((n,), 39.95),
+                          forces=torch.zeros(n, 3), energy=torch.zeros(1, 1), velocities=torch.zeros(n, 3),
+                          cell=torch.from_numpy(C[s]), pbc=torch.from_numpy(pb[s]))
+
+    def batch_of(ids):
+        b = Batch.from_data_list([system(s) for s in ids], device=DEV)
+        b["status"] = torch.zeros(len(ids), 1, dtype=torch.long, device=DEV)
+        return b
+
+    def fire_with(replacements):
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=5.0)
+        sampler = _ListSampler(replacements, batch_size=3)
+        return FIRE(model, dt=1.0, hooks=model.make_neighbor_hooks(), sampler=sampler)
+
+    # no replacement: a row less, the others as they were
+    dyn = fire_with([])
+    batch = batch_of([0, 1, 2])
+    for _ in range(6):
+        dyn.step(batch)
+    s = dyn._state
+    assert s.num_graphs == 3 and int(s.n_steps_positive.max()) > 0
+    before = {k: getattr(s, k)[1:].clone() for k in ("alpha", "dt", "n_steps_positive")}
+    batch.status[0] = 1
+    result = dyn.refill_check(batch, exit_status=1)
+    assert result.num_graphs == 2 and dyn._state.num_graphs == 2 and dyn.done is False
+    for k, v in before.items():
+        assert torch.equal(getattr(dyn._state, k), v), k
+    dyn.step(result)  # and the integrator goes on with it
+
+    # one replacement: same size; the newcomer starts from the defaults
+    dyn = fire_with([system(3)])
+    batch = batch_of([0, 1])
+    for _ in range(8):
+        dyn.step(batch)
+    kept_alpha = dyn._state.alpha[1].clone()
+    batch.status[0] = 1
+    result = dyn.refill_check(batch, exit_status=1)
+    assert result.num_graphs == 2 and dyn._state.num_graphs == 2
+    assert torch.equal(dyn._state.alpha[0], kept_alpha)
+    assert int(dyn._state.n_steps_positive[-1]) == 0 and float(dyn._state.alpha[-1]) == pytest.approx(dyn.alpha_start)
+    assert float(dyn._state.dt[-1]) == 1.0
+    dyn.step(result)
+
+    # everything leaves and nothing comes: no state, done
+    dyn = fire_with([])
+    batch = batch_of([0, 1])
+    dyn.step(batch)
+    batch.status[:] = 1
+    assert dyn.refill_check(batch, exit_status=1) is None and not hasattr(dyn, "_state") and dyn.done is True
+
+    # a fused stage keeps the state of each of its sub-stages in step
+    model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=5.0)
+    relax, md = FIRE(model, dt=1.0), NVE(model, dt=1.0)
+    fused = FusedStage([(0, relax), (1, md)], hooks=model.make_neighbor_hooks(),
+                       sampler=_ListSampler([system(3), system(4)], batch_size=3), exit_status=2)
+    batch = batch_of([0, 1, 2])
+    batch.status[1] = 1  # (a sub-stage makes its state the first time a system carries its code)
+    fused.step(batch)
+    assert relax._state.num_graphs == 3 and md._state.num_graphs == 3
+    batch.status[1] = 2
+    result = fused.refill_check(batch, exit_status=2)
+    assert result.num_graphs == 3 and relax._state.num_graphs == 3 and md._state.num_graphs == 3
+    fused.step(result)
+    result.status[:] = 2
+    result = fused.refill_check(result, exit_status=2)
+    assert result.num_graphs == 1 and relax._state.num_graphs == 1 and md._state.num_graphs == 1
+    result.status[:] = 2
+    assert fused.refill_check(result, exit_status=2) is None and fused.done
+    assert not hasattr(relax, "_state") and not hasattr(md, "_state")

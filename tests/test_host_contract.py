@@ -342,3 +342,54 @@ def test_fixed_capacity_batches_and_host_sink_on_the_host():
     assert b.num_nodes_list == [3, 5, 2, 3]
     with pytest.raises(ValueError, match="No data provided"):
         b.append_data([])
+
+
+def test_state_of_the_thermostats_and_of_fire2_and_the_rows_made_for_newcomers():
+    """Per-system state of the other integrators (restating test/dynamics/test_state_management.py:249-530):
+    shapes, dtypes, internal units, and ``_make_new_state`` for systems that join a running batch."""
+    from nvalchemi_amd.dynamics import FIRE2, NVTLangevin, NVTNoseHoover
+
+    b = two_systems()
+    FS = 10.180505710759414
+    kB = 8.617333262e-5
+    lang = NVTLangevin(FakeModel(), dt=1.0, temperature=300.0, friction=0.1)
+    lang._init_state(b)
+    s = lang._state
+    assert s.dt.shape == s.temperature.shape == s.friction.shape == (2,) and s.num_graphs == 2
+    assert torch.allclose(s.temperature, torch.tensor(300.0 * kB)) and torch.allclose(s.friction, torch.tensor(0.1 * FS))
+    assert lang._make_new_state(3, b).friction.shape == (3,)
+
+    for M_new, C in ((1, 3), (4, 5)):
+        nhc = NVTNoseHoover(FakeModel(), dt=1.0, temperature=torch.tensor([100.0, 300.0]), thermostat_time=50.0,
+                            chain_length=C)
+        nhc._init_state(b)
+        s = nhc._state
+        assert s.dt.shape == s.temperature.shape == s.nhc_ndof.shape == (2,)
+        assert s.nhc_eta.shape == s.nhc_eta_dot.shape == s.nhc_Q.shape == (2, C) and s.num_graphs == 2
+        assert s.nhc_ndof.tolist() == [9.0, 15.0] and not s.nhc_eta.any() and not s.nhc_eta_dot.any()
+        kT, tau = torch.tensor([100.0, 300.0]) * kB, 50.0 / FS
+        assert torch.allclose(s.nhc_Q[:, 1], kT * tau * tau) and torch.allclose(s.nhc_Q[:, 0], s.nhc_ndof * kT * tau * tau)
+        fresh = NVTNoseHoover(FakeModel(), dt=1.0, temperature=300.0, thermostat_time=50.0,
+                              chain_length=C)._make_new_state(M_new, b)
+        assert fresh.nhc_eta.shape == (M_new, C) and fresh.nhc_Q.shape == (M_new, C) and fresh.num_graphs == M_new
+        assert fresh.nhc_ndof.tolist() == [12.0] * M_new  # the batch's mean system size: 8 atoms in 2 systems
+    with pytest.raises(ValueError, match="yoshida_order"):
+        NVTNoseHoover(FakeModel(), dt=1.0, temperature=300.0, thermostat_time=50.0, yoshida_order=4)
+
+    f2 = FIRE2(FakeModel(), dt=0.05)
+    f2._init_state(b)
+    s = f2._state
+    assert s.dt.tolist() == pytest.approx([0.05, 0.05]) and s.alpha.tolist() == pytest.approx([0.09, 0.09])
+    assert s.nsteps_inc.dtype == torch.int32 and s.nsteps_inc.tolist() == [0, 0] and s.num_graphs == 2
+    for k in ("vf", "v_sumsq", "f_sumsq"):
+        assert getattr(s, k).shape == (2,)
+    assert (f2.delaystep, f2.dtgrow, f2.dtshrink, f2.alphashrink, f2.tmax, f2.tmin, f2.maxstep) == \
+        (60, 1.05, 0.75, 0.985, 0.08, 0.005, 0.1)
+    assert f2._make_new_state(3, b).alpha.tolist() == pytest.approx([0.09] * 3)
+    # the kernels behind them refuse host tensors
+    from nvalchemi_amd import _lib
+
+    b.velocities = torch.zeros(8, 3)
+    for dyn in (nhc, f2):
+        with pytest.raises(_lib.KernelLibraryError):
+            dyn.pre_update(b)
