@@ -166,11 +166,11 @@ class ConvergenceHook:
 
     def __call__(self, ctx: DynamicsContext, stage: Enum) -> None:
         batch = ctx.batch
+        mask = self.converged_mask(batch)  # (a missing key is an error whether or not anything migrates)
         if self.source_status is None or self.target_status is None:
             return
         if not hasattr(batch, "status") or batch.status is None:
             return
-        mask = self.converged_mask(batch)
         flat = batch.status.view(-1)
         migrate = mask & (flat[: mask.shape[0]] == self.source_status)
         flat[: mask.shape[0]] = torch.where(migrate, torch.full_like(flat[: mask.shape[0]], self.target_status),
