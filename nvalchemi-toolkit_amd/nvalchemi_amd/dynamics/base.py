@@ -217,10 +217,41 @@ class BaseDynamics(HookRegistryMixin):
         self.done = False
         self.active_batch = None
         self.global_rank = 0
+        device_type = kwargs.pop("device_type", None)
+        self.device_type: str = device_type if device_type else ("cuda" if torch.cuda.is_available() else "cpu")
+        self._stream: torch.cuda.Stream | None = None
+        self._stream_ctx: Any = None
         self._init_hooks(hooks)
         self._last_converged: torch.Tensor | None = None
         self._last_outputs: OrderedDict | None = None
         self._active_mask: torch.Tensor | None = None
+
+    # ---- a stream of its own (nvalchemi/dynamics/base.py:686-742) ----------------------------------
+    @property
+    def device(self) -> torch.device:
+        return torch.device(f"cuda:{torch.cuda.current_device()}") if self.device_type == "cuda" and \
+            torch.cuda.is_available() else torch.device("cpu")
+
+    @property
+    def stream(self) -> "torch.cuda.Stream | None":
+        """The stream made by ``with dynamics:`` (None outside the block or without a GPU)."""
+        return self._stream
+
+    def __enter__(self):
+        """``with dynamics:`` -- a new stream of default priority becomes the current one: every kernel
+        of the steps inside the block goes to it.  The caller orders it against the work that made
+        the batch, as with any stream."""
+        if self.device_type == "cuda" and torch.cuda.is_available():
+            self._stream = torch.cuda.Stream(device=self.device)
+            self._stream_ctx = torch.cuda.stream(self._stream)
+            self._stream_ctx.__enter__()
+        return self
+
+    def __exit__(self, exc_type, exc_val, exc_tb) -> None:
+        if self._stream_ctx is not None:
+            self._stream_ctx.__exit__(exc_type, exc_val, exc_tb)
+        self._stream = None
+        self._stream_ctx = None
 
     @classmethod
     def register_bookkeeping_key(cls, key: str, init_fn: Callable[[int, torch.device], torch.Tensor]) -> None:
@@ -565,6 +596,12 @@ class FusedStage(BaseDynamics):
             raise NotImplementedError("FusedStage(compile_step=True): the step is not compiled in this build")
         if not sub_stages:
             raise ValueError("FusedStage needs at least one sub-stage")
+        device_types = {dyn.device_type for _, dyn in sub_stages}
+        if len(device_types) > 1:
+            per_stage = {code: dyn.device_type for code, dyn in sub_stages}
+            raise ValueError(f"All sub-stages in a FusedStage must share the same device_type, but got: {per_stage}. "
+                             "A FusedStage runs on a single device.")
+        kwargs.setdefault("device_type", next(iter(device_types)))
         super().__init__(model=sub_stages[0][1].model, **kwargs)
         self.sub_stages = list(sub_stages)
         self.__needs_keys__ = set().union(*(dyn.__needs_keys__ for _, dyn in sub_stages))
@@ -626,6 +663,19 @@ class FusedStage(BaseDynamics):
                 continue
             if self.step_count % hook.frequency == 0:
                 hook(ctx, stage)
+
+    def __enter__(self):
+        """The fused stage's stream is also the one its sub-stages report
+        (nvalchemi/dynamics/base.py:2790-2840)."""
+        super().__enter__()
+        for _, dyn in self.sub_stages:
+            dyn._stream = self._stream
+        return self
+
+    def __exit__(self, exc_type, exc_val, exc_tb) -> None:
+        for _, dyn in self.sub_stages:
+            dyn._stream = None
+        super().__exit__(exc_type, exc_val, exc_tb)
 
     def _open_hooks(self) -> None:
         super()._open_hooks()

@@ -839,3 +839,47 @@ def test_integrator_state_follows_its_systems_through_a_refill():
     result.status[:] = 2
     assert fused.refill_check(result, exit_status=2) is None and fused.done
     assert not hasattr(relax, "_state") and not hasattr(md, "_state")
+
+
+def test_steps_inside_the_stream_context_run_on_its_stream_and_give_the_same_trajectory():
+    """``with dynamics:`` (nvalchemi/dynamics/base.py:686-742, 2790-2840): a stream of its own becomes
+    current, the kernels of the steps inside go to it (the library launches on the current stream),
+    sub-stages of a fused stage report the same stream, and the trajectory is the one of the default
+    stream bit for bit."""
+    from nvalchemi_amd.dynamics import NVE, FusedStage
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=8, n_boxes=3, reps=3, a=5.4, jitter=0.05)
+    N = len(P)
+    Z = np.full(N, 18, dtype=np.int64)
+    M = np.full(N, 39.95, dtype=np.float32)
+
+    def run(in_context):
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+        dyn = NVE(model, dt=2.0, hooks=model.make_neighbor_hooks())
+        batch = make_batch(P, Z, M, C, pb, ptr, V=np.zeros_like(P))
+        torch.cuda.synchronize()
+        if in_context:
+            default = torch.cuda.current_stream()
+            with dyn as entered:
+                assert entered is dyn and dyn.stream is not None
+                assert torch.cuda.current_stream() == dyn.stream and dyn.stream != default
+                for _ in range(10):
+                    dyn.step(batch)
+                dyn.stream.synchronize()
+            assert dyn.stream is None and torch.cuda.current_stream() == default
+        else:
+            for _ in range(10):
+                dyn.step(batch)
+            torch.cuda.synchronize()
+        return batch.positions.clone(), batch.velocities.clone()
+
+    p0, v0 = run(False)
+    p1, v1 = run(True)
+    assert torch.equal(p0, p1) and torch.equal(v0, v1)
+    model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.4, cutoff=8.0)
+    a, b = NVE(model, dt=1.0), NVE(model, dt=1.0)
+    fused = FusedStage([(0, a), (1, b)])
+    with fused:
+        assert fused.stream is not None and a.stream is fused.stream and b.stream is fused.stream
+    assert fused.stream is None and a.stream is None and b.stream is None

@@ -196,3 +196,23 @@ def test_hooks_of_the_sub_stages_fire_at_their_stages():
     assert [c[1] for c in every_other.calls] == [0, 2]
     # only the stage whose systems converged announces it
     assert len(hooks1[DynamicsStage.ON_CONVERGE].calls) == 4 and hooks0[DynamicsStage.ON_CONVERGE].calls == []
+
+
+def test_device_type_and_the_stream_context_on_the_host():
+    """``device_type`` follows what is available unless given; a fused stage wants one device type;
+    without a GPU the stream context does nothing (test/dynamics/test_single_loop.py:863-1228)."""
+    m = ConstantForces()
+    auto = BaseDynamics(model=m)
+    assert auto.device_type == ("cuda" if torch.cuda.is_available() else "cpu")
+    a, b, c = (BaseDynamics(model=m, device_type=t) for t in ("cpu", "cpu", "cuda"))
+    assert FusedStage(sub_stages=[(0, a), (1, b)]).device_type == "cpu"
+    with pytest.raises(ValueError, match="must share the same device_type"):
+        FusedStage(sub_stages=[(0, a), (1, c)])
+    with pytest.raises(ValueError, match="device_type"):
+        a + c
+    fused = FusedStage(sub_stages=[(0, a), (1, b)])
+    assert fused.stream is None
+    with fused as entered:
+        assert entered is fused and fused.stream is None and a.stream is None
+        fused.step(status_batch(2, [0, 1]))
+    assert fused.stream is None and fused._stream_ctx is None
