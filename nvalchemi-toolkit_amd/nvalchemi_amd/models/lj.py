@@ -62,6 +62,14 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
                                            half_list=self.half_list),
         )
         self._eye_cells: torch.Tensor | None = None
+        # per-system energies of the last evaluation, kept between calls of the same batch size
+        # (nvalchemi/models/lj.py:190-203); the pair kernel writes them, callers get a copy
+        self._energies_buf: torch.Tensor | None = None
+
+    def _ensure_compute_buffers(self, B: int, dtype: torch.dtype, device: torch.device) -> None:
+        buf = self._energies_buf
+        if buf is None or buf.shape[0] != B or buf.dtype != dtype or buf.device != torch.device(device):
+            self._energies_buf = torch.zeros(B, dtype=dtype, device=device)
 
     #: ``forward(batch, out={"forces": ..., "energy": ...})`` writes into the given tensors
     #: (used by the dynamics engine to fill the batch without a copy pass)
@@ -173,6 +181,10 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             if (isinstance(e_out, torch.Tensor) and e_out.numel() == B and e_out.dtype == positions.dtype
                     and e_out.is_contiguous() and e_out.device == positions.device):
                 bufs["system_energies"] = e_out.view(B)
+        own_energy = "system_energies" not in bufs
+        if own_energy:
+            self._ensure_compute_buffers(B, positions.dtype, positions.device)
+            bufs["system_energies"] = self._energies_buf
         neighbor_matrix = inp["neighbor_matrix"].contiguous()
         _, forces, sys_e, virials = lj_energy_forces_system_batch(
             positions.contiguous(), cells, neighbor_matrix,
@@ -181,6 +193,8 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs,
             row_order=self._row_order_of(data, N, positions.device),
             neighbor_list_cutoff=self._search_cutoff_of(data, neighbor_matrix))
+        if own_energy:
+            sys_e = sys_e.clone()  # a fresh tensor for the caller, as in the reference (:482)
         model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
         if virials is not None:
             model_output["virial"] = virials.view(B, 3, 3)
