@@ -34,9 +34,13 @@ def _bool_on(mask: torch.Tensor, device) -> torch.Tensor:
 class SegmentedGroup:
     """Tensors whose leading dimension is a concatenation of per-system segments."""
 
-    def __init__(self, data: dict[str, torch.Tensor], segment_lengths: torch.Tensor, device) -> None:
+    def __init__(self, data: dict[str, torch.Tensor], segment_lengths, device,
+                 batch_ptr_capacity: int | None = None) -> None:
+        """``batch_ptr_capacity``: entries to give the boundary tensor, so that ``put`` can append
+        segments (``len + len(source) + 2`` are needed); the tensors may then hold more rows than the
+        segments use (nvalchemi/data/level_storage.py:1289-1340)."""
         self._tensors = dict(data)
-        self.segment_lengths = segment_lengths.to(device=device, dtype=torch.int32)
+        self.segment_lengths = torch.as_tensor(segment_lengths).to(device=device, dtype=torch.int32)
         self.device = torch.device(device)
         self._batch_idx: torch.Tensor | None = None
         # boundaries; may hold more than len(self) + 1 entries (headroom for put)
@@ -44,6 +48,15 @@ class SegmentedGroup:
         self._lengths_host: list[int] | None = None
         # True when the tensors may hold more rows than the segments use (empty, put, defrag)
         self._over_allocated = False
+        if batch_ptr_capacity is not None:
+            n = int(self.segment_lengths.shape[0])
+            ends = torch.cumsum(self.segment_lengths, 0)
+            store = torch.zeros(max(int(batch_ptr_capacity), n + 1), dtype=torch.int32, device=self.device)
+            store[1: n + 1] = ends
+            if n:
+                store[n + 1:] = ends[-1]
+            self._batch_ptr = store
+            self._over_allocated = True
 
     def __len__(self) -> int:
         return int(self.segment_lengths.shape[0])

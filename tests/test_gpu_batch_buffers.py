@@ -351,3 +351,105 @@ def test_fused_stage_writes_finished_systems_to_its_sinks_in_order():
     order._overflow_to_sinks(stored, mask=pick(3))
     with pytest.raises(RuntimeError, match="All sinks are full"):
         order._overflow_to_sinks(stored, mask=pick(0))
+
+
+# ---- test_level_storage.py: put / defrag / fit mask of one storage group ----------------------------
+def _col(values):
+    return torch.tensor([[float(v)] for v in values], device=DEV)
+
+
+def test_uniform_group_put_defrag_and_fit_mask():
+    """test/data/test_level_storage.py:283-452 restated for ``UniformGroup``."""
+    from nvalchemi_amd.data import UniformGroup
+
+    src = UniformGroup({"a": _col([1, 2, 3, 4])}, 4, DEV)
+    dest = UniformGroup({"a": torch.zeros(4, 1, device=DEV)}, 4, DEV)
+    dest.put(src, torch.tensor([True, False, True, False], device=DEV))
+    assert dest["a"].view(-1).tolist() == [1.0, 3.0, 0.0, 0.0] and dest["a"].shape == (4, 1)
+    assert src._copied_mask.tolist() == [True, False, True, False]
+    src.defrag()
+    assert len(src) == 2 and src["a"].view(-1).tolist() == [2.0, 4.0, 0.0, 0.0] and not hasattr(src, "_copied_mask")
+
+    src = UniformGroup({"a": _col([1, 2])}, 2, DEV)
+    dest = UniformGroup({"a": torch.zeros(2, 1, device=DEV)}, 2, DEV)
+    copied = torch.zeros(2, dtype=torch.bool, device=DEV)
+    dest.put(src, torch.tensor([True, True], device=DEV), copied_mask=copied)
+    assert bool(copied.all()) and dest["a"].view(-1).tolist() == [1.0, 2.0]
+    src.defrag(copied_mask=copied)
+    assert len(src) == 0 and src["a"].shape == (2, 1)
+
+    # only what fits: one empty slot, the first masked row takes it
+    src = UniformGroup({"a": _col([1, 2, 3])}, 3, DEV)
+    dest = UniformGroup({"a": torch.zeros(3, 1, device=DEV)}, 3, DEV)
+    copied = torch.zeros(3, dtype=torch.bool, device=DEV)
+    slots = torch.tensor([True, True, False], device=DEV)
+    dest.put(src, torch.ones(3, dtype=torch.bool, device=DEV), copied_mask=copied, dest_mask=slots)
+    assert copied.tolist() == [True, False, False] and float(dest["a"][2]) == 1.0 and slots.tolist() == [True] * 3
+
+    # the fit mask says beforehand what put will move
+    src = UniformGroup({"a": _col([1, 2, 3, 4])}, 4, DEV)
+    dest = UniformGroup({"a": torch.zeros(4, 1, device=DEV)}, 4, DEV)
+    fit = torch.zeros(4, dtype=torch.bool, device=DEV)
+    dest.compute_put_per_system_fit_mask(src, torch.tensor([True, False, True, False], device=DEV), None, fit)
+    assert fit.tolist() == [True, False, True, False]
+    dest.put(src, fit)
+    assert dest["a"].view(-1).tolist()[:2] == [1.0, 3.0]
+    src = UniformGroup({"a": _col([1, 2, 3])}, 3, DEV)
+    dest = UniformGroup({"a": torch.zeros(3, 1, device=DEV)}, 3, DEV)
+    fit = torch.ones(3, dtype=torch.bool, device=DEV)
+    dest.compute_put_per_system_fit_mask(src, torch.ones(3, dtype=torch.bool, device=DEV),
+                                         torch.tensor([True, True, False], device=DEV), fit)
+    assert fit.tolist() == [True, False, False]
+    # several keys of one row land in one slot
+    src = UniformGroup({"a": _col([1, 2, 3]), "b": 10 * _col([1, 2, 3])}, 3, DEV)
+    dest = UniformGroup({"a": torch.zeros(3, 1, device=DEV), "b": torch.zeros(3, 1, device=DEV)}, 3, DEV)
+    dest.put(src, torch.tensor([False, True, True], device=DEV))
+    assert dest["a"].view(-1).tolist() == [2.0, 3.0, 0.0] and dest["b"].view(-1).tolist() == [20.0, 30.0, 0.0]
+    with pytest.raises(ValueError, match="at least one common attribute"):
+        dest.put(UniformGroup({"c": _col([1])}, 1, DEV), torch.tensor([True], device=DEV))
+
+
+def test_segmented_group_put_defrag_and_fit_mask():
+    """test/data/test_level_storage.py:737-930 restated for ``SegmentedGroup``."""
+    from nvalchemi_amd.data import SegmentedGroup
+
+    rows = lambda *v: torch.tensor([[float(x), 0.0] for x in v], device=DEV)  # noqa: E731
+    src = SegmentedGroup({"x": rows(1, 2, 3, 4, 5)}, [2, 3], DEV)
+    dest = SegmentedGroup({"x": torch.zeros(15, 2, device=DEV)}, [10], DEV, batch_ptr_capacity=5)
+    dest.put(src, torch.tensor([True, True], device=DEV))
+    assert len(dest) == 3 and dest.num_elements() == 15 and dest["x"].shape == (15, 2)
+    assert torch.equal(dest["x"][10:15], src["x"]) and not dest["x"][:10].any()
+    assert dest.batch_ptr.tolist() == [0, 10, 12, 15] and dest.lengths_list() == [10, 2, 3]
+    assert bool(src._copied_mask.all())
+    src.defrag()
+    assert len(src) == 0 and src.num_elements() == 0 and src["x"].shape == (5, 2) and not src["x"].any()
+
+    src = SegmentedGroup({"x": _col([1, 2, 3])}, [1, 2], DEV)
+    dest = SegmentedGroup({"x": torch.zeros(10, 1, device=DEV)}, [0], DEV, batch_ptr_capacity=5)
+    copied = torch.zeros(2, dtype=torch.bool, device=DEV)
+    dest.put(src, torch.tensor([True, False], device=DEV), copied_mask=copied)
+    assert copied.tolist() == [True, False] and len(dest) == 2 and float(dest["x"][0]) == 1.0
+    src.defrag(copied_mask=copied)
+    assert len(src) == 1 and src.num_elements() == 2 and src["x"].view(-1).tolist() == [2.0, 3.0, 0.0]
+    assert src.batch_idx.tolist() == [0, 0]
+
+    # the fit mask, with and without headroom in the boundaries
+    src = SegmentedGroup({"x": _col([1, 2, 3, 4, 5])}, [2, 3], DEV)
+    dest = SegmentedGroup({"x": torch.zeros(15, 1, device=DEV)}, [10], DEV, batch_ptr_capacity=5)
+    fit = torch.zeros(2, dtype=torch.bool, device=DEV)
+    dest.compute_put_per_system_fit_mask(src, torch.tensor([True, True], device=DEV), None, fit)
+    assert fit.tolist() == [True, True]
+    dest.put(src, fit)
+    assert len(dest) == 3 and torch.equal(dest["x"][10:15], src["x"])
+    tight = SegmentedGroup({"x": torch.zeros(10, 1, device=DEV)}, [0], DEV)
+    fit = torch.ones(1, dtype=torch.bool, device=DEV)
+    tight.compute_put_per_system_fit_mask(SegmentedGroup({"x": _col([1, 2])}, [2], DEV),
+                                          torch.tensor([True], device=DEV), None, fit)
+    assert fit.tolist() == [False]
+
+    # room for the first segment only
+    src = SegmentedGroup({"x": _col([1, 2, 3, 4, 5])}, [2, 3], DEV)
+    dest = SegmentedGroup({"x": torch.zeros(12, 1, device=DEV)}, [10], DEV, batch_ptr_capacity=5)
+    copied = torch.zeros(2, dtype=torch.bool, device=DEV)
+    dest.put(src, torch.tensor([True, True], device=DEV), copied_mask=copied)
+    assert copied.tolist() == [True, False] and dest["x"].view(-1).tolist()[10:] == [1.0, 2.0] and len(dest) == 2
