@@ -117,7 +117,9 @@ def cpu_baseline(pos, cell, pbc, n_per_box, n_boxes_sample, K, steps):
     M = np.ones(n, dtype=np.float32)
     dt = np.full(n_boxes_sample, 0.005, dtype=np.float32)
     out = {}
-    for label, threads in (("1", 1), ("all", os.cpu_count() or 1)):
+    # (the host share of a one-GPU box is 16 cores, whatever the machine reports)
+    share = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    for label, threads in (("1", 1), ("all", share)):
         oracle.set_threads(threads)
         Pc, V, F = P.copy(), np.zeros_like(P), np.zeros_like(P)
         t0 = time.perf_counter()
@@ -251,14 +253,15 @@ def main() -> int:
                               "alg_bytes_per_launch": nl["alg_bytes"], "ms_per_launch": nl["ms"]}
         result["stages"] = stages
     if not args.no_cpu_baseline:
-        sample_boxes = min(B, 16)
+        # about ten seconds of host work: 32 boxes, 20 steps on one thread, then on the box's share of cores
+        sample_boxes, cpu_steps = min(B, 32), 20
         cb, n_s = cpu_baseline(batch.positions.cpu().numpy(), batch.cell.cpu().numpy(), batch.pbc.cpu().numpy(),
-                               n_per_box, sample_boxes, K, steps=3)
+                               n_per_box, sample_boxes, K, steps=cpu_steps)
         v1, c1, t1 = cb["1"]
         va, ca, ta = cb["all"]
         log(f"[bench] cpu oracle: {v1:.3e} atom-steps/s on 1 thread ({t1:.1f}s), {va:.3e} on {ca} threads ({ta:.1f}s)")
         result["cpu_baseline"] = {"value": v1, "unit": "atom-steps/s", "cores": c1, "kind": "port",
-                                  "sample": f"first {sample_boxes} boxes ({n_s} atoms) of the same workload, 3 steps "
+                                  "sample": f"first {sample_boxes} boxes ({n_s} atoms) of the same workload, {cpu_steps} steps "
                                             "(VV + cell-list build + LJ + VV), C oracle -O3",
                                   "all_cores": {"value": va, "cores": ca,
                                                 "note": "OpenMP over systems in the neighbor build only"}}
