@@ -37,8 +37,9 @@ class HookRegistryMixin:
                             "Pass stage= to the hook constructor or to register_hook().")
         if (stage_type is not None and not has_custom_dispatch and hook.stage is not None
                 and not isinstance(hook.stage, stage_type)):
-            raise TypeError(f"Hook {hook!r} has stage={hook.stage!r}, but this engine only accepts "
-                            f"{getattr(stage_type, '__name__', stage_type)} stages.")
+            expected = stage_type.__name__ if isinstance(stage_type, type) else " | ".join(t.__name__ for t in stage_type)
+            raise TypeError(f"Hook {hook!r} has stage={hook.stage!r} (type {type(hook.stage).__name__}), "
+                            f"but this engine only accepts {expected} stages.")
         on_register = getattr(hook, "on_register", None)
         if on_register is not None:
             if not callable(on_register):
