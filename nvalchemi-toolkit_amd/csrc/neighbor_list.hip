@@ -31,7 +31,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kTile = 960;        // candidates staged in LDS at a time
+constexpr int kTile = 1088;       // candidates staged in LDS at a time
 constexpr int kStencilBatch = 64; // stencil cells enumerated at a time (one per lane of a wave)
 constexpr int kCenterChunk = 96;  // centre atoms of a run of cells handled per pass
 constexpr int kMaxRun = 4;        // a workgroup's unit of work: up to this many cells in a row along z
