@@ -822,8 +822,6 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         run_off[0] = 0;
 #pragma unroll
         for (int r = 1; r <= kMaxRun; ++r) run_off[r] = ws.cell_start[c0 + (r < run_len ? r : run_len)] - c_begin;
-        const int n_center = run_off[kMaxRun];
-        if (n_center == 0) continue;
         const int R0 = rper & 63, R1 = (rper >> 6) & 63, R2 = (rper >> 12) & 63;
         const int e1 = 2 * R1 + 1, e01 = (2 * R0 + 1) * e1;
         const int n_layers = run_len + 2 * R2;
@@ -834,6 +832,65 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
         // (square cells never have a stencil cell out of reach: the test is skipped for them)
         const bool may_cull = S.cull_far > cull_reach + 2.0f * S.half_diag;
+        // One batch of stencil cells: the last wave enumerates up to 64 of them, one per lane, and scans
+        // their sizes.  (The other waves load centre atoms meanwhile: the round trips to memory run
+        // side by side.)  The cells' ranges need nothing but the unit record.
+        auto enumerate_stencil = [&](const int sb) {
+            const int si = sb + lane;
+            int start = 0, count = 0, q0 = 0, q1 = 0, q2 = 0;
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f;
+            if (si < n_stencil) {
+                const int layer = si / e01, in_layer = si - layer * e01;
+                const int oz = layer - R2, oy = in_layer % e1 - R1, ox = in_layer / e1 - R0;
+                int gx = cx + ox, gy = cy + oy, gz = cz0 + oz;
+                bool ok = true;
+                if (per0) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
+                if (per1) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
+                if (per2) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
+                if (ok) {
+                    // the cell's range is asked for first: it needs nothing but the unit record,
+                    // so it does not wait for the system's constants
+                    const int c2 = cell_offset + (gx * nc1 + gy) * nc2 + gz;
+                    start = ws.cell_start[c2];
+                    const int end = ws.cell_start[c2 + 1];
+                    float fx = (float)ox, fy = (float)oy, fz = (float)oz;
+                    o0 = fx * S.step[0] + fy * S.step[3] + fz * S.step[6];
+                    o1 = fx * S.step[1] + fy * S.step[4] + fz * S.step[7];
+                    o2 = fx * S.step[2] + fy * S.step[5] + fz * S.step[8];
+                    // Skewed cells put far-away images into the stencil.  A cell whose centre is
+                    // further than the search radius plus two half-diagonals from the centre of
+                    // every cell of the run holds no neighbor (no two points of two cells are
+                    // closer than their centres minus the half-diagonals): it is left empty.
+                    float best = 0.f;
+                    if (may_cull) best = 3.0e38f;
+                    for (int r = 0; may_cull && r < run_len; ++r) {
+                        const float dx = o0 - (float)r * S.step[6], dy = o1 - (float)r * S.step[7],
+                                    dz = o2 - (float)r * S.step[8];
+                        const float d2 = dx * dx + dy * dy + dz * dz;
+                        best = d2 < best ? d2 : best;
+                    }
+                    const float lim = cull_reach + 2.0f * S.half_diag;
+                    count = (best <= lim * lim) ? end - start : 0;
+                    if (count == 0) start = 0;
+                }
+            }
+            int incl = count;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                int up = __shfl_up(incl, o, kWave);
+                if (lane >= o) incl += up;
+            }
+            st_start[lane] = start;
+            st_prefix[lane] = incl - count;
+            if (lane == kWave - 1) st_prefix[kStencilBatch] = incl;
+            st_q[lane][0] = q0; st_q[lane][1] = q1; st_q[lane][2] = q2;
+            st_off[lane][0] = o0; st_off[lane][1] = o1; st_off[lane][2] = o2;
+        };
+        // The first batch is enumerated before the run's own cell ranges have arrived.  (Nobody reads
+        // the tables of the previous unit any more: its last pass ended with a barrier.)
+        if (wave == kWavesPerBlock - 1) enumerate_stencil(0);
+        const int n_center = run_off[kMaxRun];
+        if (n_center == 0) continue;
 
         // the run's centre atoms, one pass at a time; or the one pass this unit stands for
         const int first_centre = __builtin_amdgcn_readfirstlane(grid.w);
@@ -864,56 +921,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
             }
 
             for (int sb = 0; sb < n_stencil; sb += kStencilBatch) {
-                // ---- wave 0 enumerates up to 64 stencil cells, one per lane, and scans their sizes
-                if (wave == 0) {
-                    const int si = sb + lane;
-                    int start = 0, count = 0, q0 = 0, q1 = 0, q2 = 0;
-                    float o0 = 0.f, o1 = 0.f, o2 = 0.f;
-                    if (si < n_stencil) {
-                        const int layer = si / e01, in_layer = si - layer * e01;
-                        const int oz = layer - R2, oy = in_layer % e1 - R1, ox = in_layer / e1 - R0;
-                        int gx = cx + ox, gy = cy + oy, gz = cz0 + oz;
-                        bool ok = true;
-                        if (per0) { q0 = floordiv(gx, nc0); gx -= q0 * nc0; } else ok = ok && gx >= 0 && gx < nc0;
-                        if (per1) { q1 = floordiv(gy, nc1); gy -= q1 * nc1; } else ok = ok && gy >= 0 && gy < nc1;
-                        if (per2) { q2 = floordiv(gz, nc2); gz -= q2 * nc2; } else ok = ok && gz >= 0 && gz < nc2;
-                        if (ok) {
-                            float fx = (float)ox, fy = (float)oy, fz = (float)oz;
-                            o0 = fx * S.step[0] + fy * S.step[3] + fz * S.step[6];
-                            o1 = fx * S.step[1] + fy * S.step[4] + fz * S.step[7];
-                            o2 = fx * S.step[2] + fy * S.step[5] + fz * S.step[8];
-                            // Skewed cells put far-away images into the stencil.  A cell whose centre is
-                            // further than the search radius plus two half-diagonals from the centre of
-                            // every cell of the run holds no neighbor (no two points of two cells are
-                            // closer than their centres minus the half-diagonals): it is left empty.
-                            float best = 0.f;
-                            if (may_cull) best = 3.0e38f;
-                            for (int r = 0; may_cull && r < run_len; ++r) {
-                                const float dx = o0 - (float)r * S.step[6], dy = o1 - (float)r * S.step[7],
-                                            dz = o2 - (float)r * S.step[8];
-                                const float d2 = dx * dx + dy * dy + dz * dz;
-                                best = d2 < best ? d2 : best;
-                            }
-                            const float lim = cull_reach + 2.0f * S.half_diag;
-                            if (best <= lim * lim) {
-                                int c2 = cell_offset + (gx * nc1 + gy) * nc2 + gz;
-                                start = ws.cell_start[c2];
-                                count = ws.cell_start[c2 + 1] - start;
-                            }
-                        }
-                    }
-                    int incl = count;
-#pragma unroll
-                    for (int o = 1; o < kWave; o <<= 1) {
-                        int up = __shfl_up(incl, o, kWave);
-                        if (lane >= o) incl += up;
-                    }
-                    st_start[lane] = start;
-                    st_prefix[lane] = incl - count;
-                    if (lane == kWave - 1) st_prefix[kStencilBatch] = incl;
-                    st_q[lane][0] = q0; st_q[lane][1] = q1; st_q[lane][2] = q2;
-                    st_off[lane][0] = o0; st_off[lane][1] = o1; st_off[lane][2] = o2;
-                }
+                if (wave == kWavesPerBlock - 1 && !(sb == 0 && cc0 == cc_begin)) enumerate_stencil(sb);
                 __syncthreads();
                 const int batch_total = st_prefix[kStencilBatch];
                 const int n_entries = (n_stencil - sb) < kStencilBatch ? (n_stencil - sb) : kStencilBatch;
