@@ -40,8 +40,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
 # bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
 MEASURED_TRAFFIC_BYTES = {
-    "nl": 1024 * (2 * (43403 + 6581) + (933658 + 63212)),   # search + per-system sort
-    "lj": 1024 * (2 * (185117 + 2448) + 78176 + 13),        # pair kernel + system ranges
+    "nl": 1024 * (2 * (45789 + 6581) + (933783 + 62136)),   # search + per-system sort
+    "lj": 1024 * (2 * (184874 + 2448) + 78189 + 13),        # pair kernel + system ranges
 }
 
 
