@@ -769,7 +769,14 @@ __device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, i
 // what a range picks up beyond its own layers (ranges are widened to multiples of 64) lies
 // further than the stencil radius away and can never pass the distance test.
 template <bool HALF>
-__global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorkspace ws) {
+// The tables that every lane of a workgroup reads at the same address (unit records, the per-system
+// constants, the run's cell ranges) come in as read-only arguments of their own besides the workspace:
+// nothing in the kernel can be seen to write them, so they are fetched through the scalar cache, which
+// answers sooner than the vector path and keeps these loads out of the order of the row stores.
+__global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorkspace ws,
+                                                              const NlUnit* __restrict__ units_ro,
+                                                              const NlSearchSys* __restrict__ ssys_ro,
+                                                              const int* __restrict__ cell_start_ro) {
     __shared__ float4 c_pos[kTile];           // candidate: xyz relative to the run's first cell + atom index
     __shared__ int c_pk[kTile];               // packed (image of its cell - its own wrap)
     __shared__ float4 ca_pos[kCenterChunk];   // centre atoms of this pass: same frame + atom index
@@ -800,7 +807,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         // NOTE: every thread of the workgroup takes the same path through this loop body
         const int round0 = (li / group) * 8 * group;  // first unit of this round of 8 groups
         const int u = round0 + xcd * group + li % group;
-        const int4* rec = reinterpret_cast<const int4*>(ws.units + (u < last_unit ? u : last_unit));
+        const int4* rec = reinterpret_cast<const int4*>(units_ro + (u < last_unit ? u : last_unit));
         const int4 unit = rec[0], grid = rec[1];  // (asked for before u is known to exist)
         if (round0 >= total_units) break;
         if (u >= total_units) continue;
@@ -812,16 +819,16 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         const int rper = __builtin_amdgcn_readfirstlane(grid.y);
         const int cell_offset = __builtin_amdgcn_readfirstlane(grid.z);
         if (a.rebuild && !a.rebuild[sidx]) continue;
-        const NlSearchSys S = ws.ssys[sidx];  // (the cell steps and the tolerance are taken from here)
+        const NlSearchSys S = ssys_ro[sidx];  // (the cell steps and the tolerance are taken from here)
         const int nc0 = (nc_pack & 1023) + 1, nc1 = ((nc_pack >> 10) & 1023) + 1, nc2 = ((nc_pack >> 20) & 1023) + 1;
         const int per0 = (rper >> 18) & 1, per1 = (rper >> 19) & 1, per2 = (rper >> 20) & 1;
         const int cz0 = cxyz & 1023, cy = (cxyz >> 10) & 1023, cx = cxyz >> 20;
-        const int c_begin = ws.cell_start[c0];
+        const int c_begin = cell_start_ro[c0];
         // first centre atom (relative to c_begin) of the run's cells 1, 2, 3 and the run's end
         int run_off[kMaxRun + 1];
         run_off[0] = 0;
 #pragma unroll
-        for (int r = 1; r <= kMaxRun; ++r) run_off[r] = ws.cell_start[c0 + (r < run_len ? r : run_len)] - c_begin;
+        for (int r = 1; r <= kMaxRun; ++r) run_off[r] = cell_start_ro[c0 + (r < run_len ? r : run_len)] - c_begin;
         const int R0 = rper & 63, R1 = (rper >> 6) & 63, R2 = (rper >> 12) & 63;
         const int e1 = 2 * R1 + 1, e01 = (2 * R0 + 1) * e1;
         const int n_layers = run_len + 2 * R2;
@@ -1263,8 +1270,8 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     unsigned n_search = 8u * 2048u;
     size_t cells_bound = max_cells_for(n_atoms, n_systems);
     if (cells_bound < n_search) n_search = (unsigned)((cells_bound + 7) / 8 * 8);
-    if (a.half) hipLaunchKernelGGL(nl_search_kernel<true>, dim3(n_search), blk, 0, st, a, ws);
-    else hipLaunchKernelGGL(nl_search_kernel<false>, dim3(n_search), blk, 0, st, a, ws);
+    if (a.half) hipLaunchKernelGGL(nl_search_kernel<true>, dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start);
+    else hipLaunchKernelGGL(nl_search_kernel<false>, dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start);
     NVAMD_LAUNCH_CHECK("neighbor list launch");
     return NVAMD_OK;
 }
