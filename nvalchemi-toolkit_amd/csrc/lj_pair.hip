@@ -320,7 +320,12 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
 
 template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool VEC, bool SWITCH>
 // (six waves per SIMD: three workgroups per CU; the virial variant needs more registers than that leaves)
-__global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_matrix_kernel(LjArgs a) {
+// What a whole workgroup reads at one address while it finds its system (batch index, walk order, the
+// system's range and cell) comes in as read-only arguments of their own: nothing in the kernel can be seen
+// to write them, so this chain of dependent loads goes through the scalar cache.
+__global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_matrix_kernel(
+    LjArgs a, const int32_t* __restrict__ bidx_ro, const int32_t* __restrict__ order_ro,
+    const int32_t* __restrict__ first_ro, const int32_t* __restrict__ last_ro, const float* __restrict__ cells_ro) {
     constexpr int NV = VIRIAL ? 7 : 1;
     __shared__ double s_acc[kSysSlots][NV];
     __shared__ float s_pos[3 * kLdsAtoms];
@@ -336,16 +341,16 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
     const int row0 = (int)lb * a.rows_per_block;
     const int row_end = (row0 + a.rows_per_block) < a.n_atoms ? (row0 + a.rows_per_block) : a.n_atoms;
     if (row0 >= row_end) return;
-    const int sys_lo = a.bidx[a.order ? a.order[row0] : row0];
+    const int sys_lo = bidx_ro[order_ro ? order_ro[row0] : row0];
     if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
 
     // Neighbors live in the system of their row: the rows are taken one system at a time, with
     // that system's positions staged in LDS when they fit (atom order carries no spatial
     // locality, so gathers through the caches move a whole line per 12 useful bytes).
     for (int r = row0; r < row_end;) {
-        const int sys = a.bidx[a.order ? a.order[r] : r];
-        const int span0 = a.sys_first[sys];
-        const int span_end = a.sys_last[sys];
+        const int sys = bidx_ro[order_ro ? order_ro[r] : r];
+        const int span0 = first_ro[sys];
+        const int span_end = last_ro[sys];
         const int span_n = span_end - span0;
         // rows of this system inside the block; a batch index that is not sorted (a system in
         // several pieces) makes the range meaningless: then the rest of the block goes unstaged
@@ -358,7 +363,7 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
         }
         if (SHIFTS && threadIdx.x < 27) {
             const int t = threadIdx.x;
-            shift_vector(a.cells + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
+            shift_vector(cells_ro + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
                          s_shift[t][2]);
         }
         if (SHIFTS && threadIdx.x == 32) {
@@ -366,7 +371,7 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
             // width of the cell (1 / |column of the inverse|): then no pair has two listed images
             int ok = 0;
             if (a.list_rc > 0.0) {
-                const float* c = a.cells + 9 * (size_t)sys;
+                const float* c = cells_ro + 9 * (size_t)sys;
                 double h[9], hv[9];
                 for (int k = 0; k < 9; ++k) h[k] = (double)c[k];
                 inv3(h, hv);  // (a singular cell gives infinities or NaNs: they fail the test below)
@@ -543,8 +548,8 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
     const bool sw = a.inv_sw > 0.0;
 #define NVAMD_LJ_LAUNCH(V, S, Y, W)                                                                  \
     {                                                                                                \
-        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true, W>), grid, blk, 0, st, b); \
-        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false, W>), grid, blk, 0, st, b);    \
+        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true, W>), grid, blk, 0, st, b, b.bidx, b.order, b.sys_first, b.sys_last, b.cells); \
+        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false, W>), grid, blk, 0, st, b, b.bidx, b.order, b.sys_first, b.sys_last, b.cells);    \
         return;                                                                                      \
     }
 #define NVAMD_LJ_CASE(V, S, Y)                                                                 \
