@@ -40,8 +40,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
 # bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
 MEASURED_TRAFFIC_BYTES = {
-    "nl": 1024 * (2 * (45789 + 6581) + (933783 + 62136)),   # search + per-system sort
-    "lj": 1024 * (2 * (184874 + 2448) + 78189 + 13),        # pair kernel + system ranges
+    "nl": 1024 * (2 * (31569 + 6576) + (845320 + 62277)),   # search + per-system sort
+    "lj": 1024 * (2 * (178661 + 2448) + 78193 + 13),        # pair kernel + system ranges
 }
 
 
