@@ -183,28 +183,55 @@ __global__ __launch_bounds__(kBlock) void fire_clear_kernel(double* acc, int n) 
     if (t < n) acc[t] = 0.0;
 }
 
+// A workgroup takes kFireChunks chunks of kBlock atoms.  Inside a wave the atoms of one system are summed
+// with shuffles; the sums of the first kFireSlots systems a workgroup meets are then collected in LDS and
+// go to memory once per workgroup (a system of a few thousand atoms otherwise receives one atomic per wave
+// on the same three addresses, which is what this kernel then waits for).
+constexpr int kFireChunks = 4;
+constexpr int kFireSlots = 8;
+
 __global__ __launch_bounds__(kBlock) void fire_reduce_kernel(const float* __restrict__ vel,
                                                              const float* __restrict__ frc,
                                                              const int32_t* __restrict__ bidx,
                                                              double* __restrict__ acc, int n_atoms) {
-    int i = blockIdx.x * kBlock + threadIdx.x;
-    double v[3] = {0.0, 0.0, 0.0};
-    int seg = -1 - (i - n_atoms);  // distinct negative ids past the end: never merged
-    if (i < n_atoms) {
-        seg = bidx[i];
+    __shared__ double s_acc[kFireSlots][3];
+    const int first = (int)blockIdx.x * (kFireChunks * kBlock);  // (below n_atoms: the grid is sized so)
+    if (threadIdx.x < kFireSlots * 3) (&s_acc[0][0])[threadIdx.x] = 0.0;
+    const int seg_lo = bidx[first];
+    __syncthreads();
+    for (int c = 0; c < kFireChunks; ++c) {  // (every lane takes every turn: the sums use shuffles)
+        const int i = first + c * kBlock + (int)threadIdx.x;
+        double v[3] = {0.0, 0.0, 0.0};
+        int seg = -1 - (i - n_atoms);  // distinct negative ids past the end: never merged
+        if (i < n_atoms) {
+            seg = bidx[i];
 #pragma unroll
-        for (int a = 0; a < 3; ++a) {
-            double vv = (double)vel[3 * (size_t)i + a], ff = (double)frc[3 * (size_t)i + a];
-            v[0] += ff * vv;
-            v[1] += vv * vv;
-            v[2] += ff * ff;
+            for (int a = 0; a < 3; ++a) {
+                double vv = (double)vel[3 * (size_t)i + a], ff = (double)frc[3 * (size_t)i + a];
+                v[0] += ff * vv;
+                v[1] += vv * vv;
+                v[2] += ff * ff;
+            }
+        }
+        const bool head = wave_segmented_sum<3>(seg, v);
+        if (head && i < n_atoms) {
+            const unsigned slot = (unsigned)(seg - seg_lo);
+            if (slot < (unsigned)kFireSlots) {
+                atomicAdd(&s_acc[slot][0], v[0]);
+                atomicAdd(&s_acc[slot][1], v[1]);
+                atomicAdd(&s_acc[slot][2], v[2]);
+            } else {
+                atomic_add_f64(acc + 3 * (size_t)seg + 0, v[0]);
+                atomic_add_f64(acc + 3 * (size_t)seg + 1, v[1]);
+                atomic_add_f64(acc + 3 * (size_t)seg + 2, v[2]);
+            }
         }
     }
-    bool head = wave_segmented_sum<3>(seg, v);
-    if (head && i < n_atoms) {
-        atomic_add_f64(acc + 3 * (size_t)seg + 0, v[0]);
-        atomic_add_f64(acc + 3 * (size_t)seg + 1, v[1]);
-        atomic_add_f64(acc + 3 * (size_t)seg + 2, v[2]);
+    __syncthreads();
+    if (threadIdx.x < kFireSlots * 3) {
+        // (a slot that no atom touched is still zero and names a system that may not exist)
+        const double v = (&s_acc[0][0])[threadIdx.x];
+        if (v != 0.0) atomic_add_f64(acc + 3 * (size_t)seg_lo + threadIdx.x, v);
     }
 }
 
@@ -541,8 +568,8 @@ NVAMD_EXPORT int32_t nvamd_fire_step(float* positions, float* velocities, const 
         int n3 = 3 * n_systems;
         hipLaunchKernelGGL(fire_clear_kernel, dim3((n3 + kBlock - 1) / kBlock), blk, 0, st, ws.acc, n3);
         if (n_atoms > 0)
-            hipLaunchKernelGGL(fire_reduce_kernel, grid_n, blk, 0, st, velocities, forces, batch_idx,
-                               ws.acc, n_atoms);
+            hipLaunchKernelGGL(fire_reduce_kernel, dim3((n_atoms + kFireChunks * kBlock - 1) / (kFireChunks * kBlock)), blk,
+                               0, st, velocities, forces, batch_idx, ws.acc, n_atoms);
     } else {
         hipLaunchKernelGGL(fire_import_kernel, grid_m, blk, 0, st, vf, vv, ff, ws.acc, n_systems);
     }
@@ -600,7 +627,8 @@ NVAMD_EXPORT int32_t nvamd_fire2_step(float* positions, float* velocities, const
     const int n3 = 3 * n_systems;
     hipLaunchKernelGGL(fire_clear_kernel, dim3((n3 + kBlock - 1) / kBlock), blk, 0, st, ws.acc, n3);
     if (n_atoms > 0)
-        hipLaunchKernelGGL(fire_reduce_kernel, grid_n, blk, 0, st, velocities, forces, batch_idx, ws.acc, n_atoms);
+        hipLaunchKernelGGL(fire_reduce_kernel, dim3((n_atoms + kFireChunks * kBlock - 1) / (kFireChunks * kBlock)), blk, 0, st,
+                           velocities, forces, batch_idx, ws.acc, n_atoms);
     hipLaunchKernelGGL(fire2_params_kernel, grid_m, blk, 0, st, alpha, dt, nsteps_inc, vf, v_sumsq, f_sumsq, active,
                        ws, p, n_systems);
     if (n_atoms > 0) {
