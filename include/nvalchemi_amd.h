@@ -74,6 +74,25 @@ int32_t nvamd_nl_build(const float* positions, const float* cell, const uint8_t*
                        int32_t* neighbor_matrix_shifts, void* workspace, size_t workspace_bytes,
                        void* stream);
 
+/* nvamd_nl_build with the way the atoms are brought into cell order chosen by the caller instead
+ * of by the library (no counterpart in the reference; the lists are the same sets either way):
+ *   NVAMD_NL_SORT_AUTO        what nvamd_nl_build does: per system up to 8192 atoms per system
+ *                             on average, global above
+ *   NVAMD_NL_SORT_PER_SYSTEM  one workgroup sorts one system (batches of many small systems)
+ *   NVAMD_NL_SORT_GLOBAL      one counting sort over all atoms (few, large systems)
+ * Either path handles any input; the choice only matters for speed.  The tests use it to run
+ * every case on both. */
+#define NVAMD_NL_SORT_AUTO 0
+#define NVAMD_NL_SORT_PER_SYSTEM 1
+#define NVAMD_NL_SORT_GLOBAL 2
+int32_t nvamd_nl_build_path(const float* positions, const float* cell, const uint8_t* pbc,
+                            const int32_t* batch_ptr, const int32_t* batch_idx,
+                            const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                            double cutoff, int32_t max_neighbors, int32_t half_fill,
+                            int32_t tail_mode, int32_t sort_path, int32_t* neighbor_matrix,
+                            int32_t* num_neighbors, int32_t* neighbor_matrix_shifts, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
 /* Dense -> COO compaction in row-major order (atom ascending, slot ascending).  Replaces
  * nvalchemiops.torch.neighbors.neighbor_utils.get_neighbor_list_from_neighbor_matrix as
  * called at nvalchemi/neighbors.py:92-103, in two steps so the caller can size the output:
@@ -140,8 +159,13 @@ int32_t nvamd_vv_velocity_finalize(float* velocities, const float* forces_new,
  * FIRE step.  Replaces nvalchemi::_fire_step_op (nvalchemi/dynamics/_ops/fire.py:79-140).
  *   All per-system arrays have M entries; alpha, dt, n_steps_positive, vf, vv, ff and
  *   positions, velocities are updated.  compute_reductions = 0 consumes vf/vv/ff as given.
- *   uphill_flag is accepted for signature parity; only the vanilla branch exists, entries
- *   other than 0 are ignored.  `active` as above.
+ *   Order (nvalchemi/dynamics/_ops/fire.py:270-272): reductions over the arrays as passed in,
+ *   then the MD integration with the stored dt (kick, drift limited to maxstep per atom), then
+ *   the mixing with the stored alpha (sum F.v >= 0) or the reset of the velocities (< 0),
+ *   then the update of dt, alpha and n_steps_positive.
+ *   Only the vanilla branch exists.  uphill_flag is a device array, so the library cannot look
+ *   at it without a synchronisation and does not: the caller must pass zeros (the Python
+ *   wrapper checks and raises for anything else).  `active` as above.
  *   workspace: nvamd_fire_workspace_bytes(n_systems).
  * ---------------------------------------------------------------------------------------- */
 int32_t nvamd_fire_workspace_bytes(int32_t n_systems, size_t* bytes);

@@ -260,10 +260,11 @@ __global__ __launch_bounds__(kBlock) void fire_params_kernel(
         vv[s] = (float)VV;
         ff[s] = (float)FF;
     }
-    float h = dt[s];
+    const float h_stored = dt[s];  // the MD sub-step integrates with the time step of before the update
+    float h = h_stored;
     float ma = 1.0f, mb = 0.0f;
     if (!active || active[s]) {
-        if (P > 0.0) {
+        if (P >= 0.0) {
             float al = alpha[s];
             ma = 1.0f - al;
             mb = (FF > 0.0) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(kBlock) void fire_params_kernel(
     }
     ws.mix_a[s] = ma;
     ws.mix_b[s] = mb;
-    ws.dt_use[s] = h;
+    ws.dt_use[s] = h_stored;
 }
 
 __global__ __launch_bounds__(kBlock) void fire_update_kernel(
@@ -302,13 +303,12 @@ __global__ __launch_bounds__(kBlock) void fire_update_kernel(
     if (active && !active[s]) return;
     float ma = ws.mix_a[s], mb = ws.mix_b[s], h = ws.dt_use[s], ms = maxstep[s], m = masses[i];
     size_t b = 3 * (size_t)i;
-    float v[3], dr[3];
+    float v[3], dr[3], f[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        float f = frc[b + a];
-        float vm = (ma * vel[b + a]) + (mb * f);
-        float acc = f / m;
-        v[a] = vm + (h * acc);
+        f[a] = frc[b + a];
+        float acc = f[a] / m;
+        v[a] = vel[b + a] + (h * acc);
         v[a] = fminf(fmaxf(v[a], -kFireVmax), kFireVmax);  // keep dr finite
         dr[a] = h * v[a];
     }
@@ -324,9 +324,10 @@ __global__ __launch_bounds__(kBlock) void fire_update_kernel(
 #pragma unroll
         for (int a = 0; a < 3; ++a) dr[a] = dr[a] * sc;
     }
+    // the mixing comes after the integration and acts on the kicked velocity
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        vel[b + a] = v[a];
+        vel[b + a] = (ma * v[a]) + (mb * f[a]);
         pos[b + a] = pos[b + a] + dr[a];
     }
 }

@@ -532,12 +532,8 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
     LjArgs b = a;
     // a workgroup owns a run of consecutive rows: long enough to amortise the staging of its
     // systems' positions and to keep per-system sums in LDS, short enough to fill the chip
-    static int forced_rows = [] {
-        const char* e = getenv("NVAMD_LJ_ROWS_PER_BLOCK");
-        return e ? atoi(e) : 0;
-    }();
-    int rows = forced_rows > 0 ? forced_rows : 512;
-    while (forced_rows <= 0 && rows > 4 * G && (a.n_atoms + rows - 1) / rows < 256 * 6) rows /= 2;
+    int rows = 512;
+    while (rows > 4 * G && (a.n_atoms + rows - 1) / rows < 256 * 6) rows /= 2;
     rows = (rows + G - 1) / G * G;
     b.rows_per_block = rows;
     b.n_blocks = (unsigned)((a.n_atoms + rows - 1) / rows);
@@ -567,11 +563,6 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
 }
 
 int lanes_per_row(int K) {
-    static int forced = [] {
-        const char* e = getenv("NVAMD_LJ_LANES_PER_ROW");
-        return e ? atoi(e) : 0;
-    }();
-    if (forced == 8 || forced == 16 || forced == 32 || forced == 64) return forced;
     if (K <= 192) return 8;
     if (K <= 512) return 16;
     return 32;
@@ -609,17 +600,15 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces(const float* positions, const float*
                                          system_energies, workspace, workspace_bytes, stream);
 }
 
-NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells,
-                                                    const int32_t* neighbor_matrix,
-                                                    const int32_t* neighbor_matrix_shifts,
-                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
-                                                    const int32_t* row_order, double neighbor_list_cutoff,
-                                                    int32_t n_atoms,
-                                                    int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
-                                                    double epsilon, double sigma, double cutoff,
-                                                    double switch_width, int32_t half_list, float* atomic_energies,
-                                                    float* forces, float* virials, float* system_energies,
-                                                    void* workspace, size_t workspace_bytes, void* stream) {
+// The one implementation behind the three entry points; `workspace` is device memory of at least
+// nvamd_lj_workspace_bytes(n_atoms, n_systems, half_list) bytes, wherever it comes from.
+static int32_t lj_energy_forces_impl(const float* positions, const float* cells, const int32_t* neighbor_matrix,
+                                     const int32_t* neighbor_matrix_shifts, const int32_t* num_neighbors,
+                                     const int32_t* batch_idx, const int32_t* row_order, double neighbor_list_cutoff,
+                                     int32_t n_atoms, int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
+                                     double epsilon, double sigma, double cutoff, double switch_width,
+                                     int32_t half_list, float* atomic_energies, float* forces, float* virials,
+                                     float* system_energies, void* workspace, size_t workspace_bytes, void* stream) {
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
     if (!(switch_width >= 0.0) || switch_width > cutoff)
@@ -660,12 +649,12 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const
     a.order = half_list ? nullptr : row_order;  // (the half-list kernel walks rows in index order)
     a.sys_first = nullptr;
     a.sys_last = nullptr;
-    a.lds_atoms = getenv("NVAMD_LJ_NO_LDS") ? 0 : kLdsAtoms;
+    a.lds_atoms = kLdsAtoms;
     a.r_on = switch_width > 0.0 ? cutoff - switch_width : 0.0;
     a.inv_sw = switch_width > 0.0 ? 1.0 / switch_width : 0.0;
     // (a list built with a smaller cutoff than the potential's would be the caller's mistake:
     // the larger of the two is the safe bound)
-    a.list_rc = (neighbor_list_cutoff > 0.0 && !half_list && !getenv("NVAMD_LJ_READ_SHIFTS"))
+    a.list_rc = (neighbor_list_cutoff > 0.0 && !half_list)
                     ? (neighbor_list_cutoff > cutoff ? neighbor_list_cutoff : cutoff)
                     : 0.0;
     const bool shifts = neighbor_matrix_shifts != nullptr;
@@ -719,4 +708,21 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const
     }
     NVAMD_LAUNCH_CHECK("lj launch");
     return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells,
+                                                    const int32_t* neighbor_matrix,
+                                                    const int32_t* neighbor_matrix_shifts,
+                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
+                                                    const int32_t* row_order, double neighbor_list_cutoff,
+                                                    int32_t n_atoms,
+                                                    int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
+                                                    double epsilon, double sigma, double cutoff,
+                                                    double switch_width, int32_t half_list, float* atomic_energies,
+                                                    float* forces, float* virials, float* system_energies,
+                                                    void* workspace, size_t workspace_bytes, void* stream) {
+    return lj_energy_forces_impl(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors, batch_idx,
+                                 row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
+                                 sigma, cutoff, switch_width, half_list, atomic_energies, forces, virials,
+                                 system_energies, workspace, workspace_bytes, stream);
 }

@@ -1207,6 +1207,20 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
                                     int32_t tail_mode, int32_t* neighbor_matrix, int32_t* num_neighbors,
                                     int32_t* neighbor_matrix_shifts, void* workspace,
                                     size_t workspace_bytes, void* stream) {
+    return nvamd_nl_build_path(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, n_atoms, n_systems, cutoff,
+                               max_neighbors, half_fill, tail_mode, NVAMD_NL_SORT_AUTO, neighbor_matrix, num_neighbors,
+                               neighbor_matrix_shifts, workspace, workspace_bytes, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* cell, const uint8_t* pbc,
+                                         const int32_t* batch_ptr, const int32_t* batch_idx,
+                                         const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                                         double cutoff, int32_t max_neighbors, int32_t half_fill,
+                                         int32_t tail_mode, int32_t sort_path, int32_t* neighbor_matrix,
+                                         int32_t* num_neighbors, int32_t* neighbor_matrix_shifts, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+    if (sort_path != NVAMD_NL_SORT_AUTO && sort_path != NVAMD_NL_SORT_PER_SYSTEM && sort_path != NVAMD_NL_SORT_GLOBAL)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: unknown sort_path %d", (int)sort_path);
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: negative size");
     if (!(cutoff > 0.0)) return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: cutoff must be positive");
@@ -1249,9 +1263,9 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
     hipStream_t st = static_cast<hipStream_t>(stream);
     dim3 blk(kBlock);
     auto blocks = [](size_t n) { return dim3((unsigned)((n + kBlock - 1) / kBlock)); };
-    // (looked up on every call so that one process can exercise both paths)
-    const bool forbid_per_system = getenv("NVAMD_NL_NO_PER_SYSTEM") != nullptr;
-    if (!forbid_per_system && n_atoms / n_systems <= kPerSystemMeanAtoms) {
+    const bool per_system = sort_path == NVAMD_NL_SORT_AUTO ? (n_atoms / n_systems <= kPerSystemMeanAtoms)
+                                                            : (sort_path == NVAMD_NL_SORT_PER_SYSTEM);
+    if (per_system) {
         // many small systems: set-up to scatter in one workgroup per system
         hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws);
         hipLaunchKernelGGL(nl_system_sort_kernel, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);

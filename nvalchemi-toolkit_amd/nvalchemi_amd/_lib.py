@@ -30,6 +30,8 @@ _SIGNATURES = {
     "nvamd_nl_workspace_bytes": (_i32, [_i32, _i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_nl_build": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32,
                               _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_nl_build_path": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32, _i32,
+                                   _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_coo_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_nl_edge_ptr": (_i32, [_vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_matrix_to_coo": (_i32, [_vp, _vp, _vp, _i32, _i32, _c.c_int64, _vp, _vp, _vp]),
@@ -168,10 +170,18 @@ def nl_workspace_bytes(n_atoms: int, n_systems: int) -> int:
     return _size(library().nvamd_nl_workspace_bytes, int(n_atoms), int(n_systems))
 
 
+NL_SORT_AUTO, NL_SORT_PER_SYSTEM, NL_SORT_GLOBAL = 0, 1, 2
+# how nl_build brings the atoms into cell order when its caller does not say (sort_path=None): the
+# library's own choice.  The GPU tests set this to run every case on both paths.
+nl_sort_path = NL_SORT_AUTO
+
+
 def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, max_neighbors,
              half_fill, tail_mode, neighbor_matrix, num_neighbors, neighbor_matrix_shifts,
-             workspace: torch.Tensor | None = None) -> None:
+             workspace: torch.Tensor | None = None, sort_path: int | None = None) -> None:
     lib = library()
+    if sort_path is None:
+        sort_path = nl_sort_path
     N = positions.shape[0]
     B = batch_ptr.shape[0] - 1
     K = int(max_neighbors)
@@ -188,9 +198,9 @@ def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, 
     ws = workspace if workspace is not None else workspaces.get(positions.device, "nl", need)
     if ws.device != positions.device or ws.numel() * ws.element_size() < need:
         raise ValueError("neighbor-list workspace too small or on another device")
-    _check(lib.nvamd_nl_build(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,
-                              int(bool(half_fill)), int(tail_mode), p_nm, p_nn, p_sh, ws.data_ptr(),
-                              ws.numel() * ws.element_size(), _stream(positions.device)),
+    _check(lib.nvamd_nl_build_path(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,
+                                   int(bool(half_fill)), int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
+                                   ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)),
            "nvamd_nl_build")
 
 

@@ -2,15 +2,20 @@
 
 Same schema and mutation set as ``nvalchemi::_fire_step_op`` and the same public
 ``fire_step`` signature (nvalchemi/dynamics/_ops/fire.py:79-140,245-362).  Per system, with
-the reductions ``vf = sum F.v``, ``vv = sum v.v``, ``ff = sum F.F`` taken at entry:
+the reductions ``vf = sum F.v``, ``vv = sum v.v``, ``ff = sum F.F`` taken over the arrays as
+passed in, "an MD integration step followed by FIRE velocity mixing and adaptive parameter
+updates" (nvalchemi/dynamics/_ops/fire.py:270-272):
 
-    vf > 0 : v <- (1-alpha) v + alpha sqrt(vv/ff) F        (alpha as stored)
-             n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max) ; alpha *= f_alpha
-    else   : v <- 0 ; n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
-    then   : v += dt F/m ; dr = dt v ; |dr| > maxstep -> dr *= maxstep/|dr| ; r += dr
+    MD      : v1 = v + dt F/m ; dr = dt v1 ; |dr| > maxstep -> dr *= maxstep/|dr| ; r += dr
+              (dt as stored)
+    vf >= 0 : v <- (1-alpha) v1 + alpha sqrt(vv/ff) F        (alpha as stored)
+              n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max) ; alpha *= f_alpha
+    vf < 0  : v <- 0 ; n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
 
-All atoms of a system see the same pre-update scalars.  Only the vanilla branch exists:
-``uphill_flag`` entries are ignored by the kernel (the ``FIRE`` class refuses ``uphill``).
+All atoms of a system see the same pre-update scalars.  The reference's own step is in a kernel
+library outside its tree, so what its sentences leave open (the side of ``vf == 0``, ``>`` against
+``>=`` for ``n_min``, the Euler form) is this library's choice.  Only the vanilla branch exists:
+``fire_step`` raises ``NotImplementedError`` for a non-zero ``uphill_flag``.
 """
 
 from __future__ import annotations
@@ -50,10 +55,18 @@ def fire_step(positions: torch.Tensor, velocities: torch.Tensor, forces: torch.T
               maxstep: torch.Tensor, n_min: torch.Tensor, f_dec: torch.Tensor, f_inc: torch.Tensor,
               uphill_flag: torch.Tensor, *, vf: torch.Tensor | None = None, vv: torch.Tensor | None = None,
               ff: torch.Tensor | None = None, batch_idx: torch.Tensor | None = None,
-              compute_reductions: bool = True, active: torch.Tensor | None = None) -> None:
+              compute_reductions: bool = True, active: torch.Tensor | None = None,
+              uphill_checked: bool = False) -> None:
     """Full FIRE step; mutates positions, velocities, alpha, dt, n_steps_positive (and the
     scratch ``vf``/``vv``/``ff``, allocated when ``None``).  ``active [M] bool`` (extension):
-    systems with ``False`` are left untouched."""
+    systems with ``False`` are left untouched.
+
+    Only vanilla FIRE is built: a non-zero ``uphill_flag`` raises ``NotImplementedError`` (its
+    semantics are not stated anywhere in the reference's tree).  Looking at the flag costs a
+    read-back from the device; a caller that has made the flag itself and knows it to be zero
+    (the ``FIRE`` class) says so with ``uphill_checked=True`` (extension) and pays nothing."""
+    if not uphill_checked and uphill_flag is not None and bool((uphill_flag != 0).any()):
+        raise NotImplementedError("fire_step: uphill_flag = 1 (FIRE with uphill step checks) is not implemented")
     M = alpha.shape[0]
     dtype, device = positions.dtype, positions.device
     if vf is None:

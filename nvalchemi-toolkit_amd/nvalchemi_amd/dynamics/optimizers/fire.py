@@ -72,7 +72,7 @@ class FIRE(BaseDynamics):
         fire_step(batch.positions, batch.velocities, batch.forces, batch.atomic_masses, s.alpha, s.dt,
                   s.n_steps_positive, s.alpha_start, s.f_alpha, s.dt_min, s.dt_max, s.maxstep, s.n_min,
                   s.f_dec, s.f_inc, s.uphill_flag, vf=s.vf, vv=s.vv, ff=s.ff, batch_idx=batch.batch_idx,
-                  active=self._active_mask)
+                  active=self._active_mask, uphill_checked=True)  # the flag is this class's own zeros
 
     def post_update(self, batch) -> None:
         """No-op; the new forces are consumed by the next ``pre_update``."""

@@ -52,11 +52,14 @@
  *                  taken and checked for what C2 continuity demands: S = 1 / 0 and zero slope
  *                  and curvature at the ends, S(1/2) = 1/2, F = -dE/dr by finite differences).
  *   orc_vv_*       pinned: harmonic-oscillator closed form, time reversibility.
- *   orc_fire_step  PARITY UNPINNED against the reference: the exact ordering of FIRE's
- *                  sub-steps is only visible inside the absent wheel.  The restatement
- *                  follows Bitzek 2006 / ASE ordering, constrained by the reference's
- *                  notes (reductions at entry; mixing with the stored alpha; per-atom
- *                  maxstep clamp; vanilla branch only).  Checked by invariants only.
+ *   orc_fire_step  PARITY UNPINNED against the reference: the step is inside the absent wheel.
+ *                  The order of its sub-steps follows the reference's own sentences (reductions
+ *                  over what is passed in; MD integration with the stored dt, then mixing with
+ *                  the stored alpha, then the parameter update; per-atom maxstep clamp; vanilla
+ *                  branch only), each cited at the function.  Checked against those sentences
+ *                  (tests that a mix-first order, post-kick reductions or an updated dt in the
+ *                  integration would fail) and by invariants; what no sentence decides is
+ *                  listed at the function.
  *   orc_langevin_half_step  PARITY UNPINNED against the reference: its random stream and the rounding
  *                  of its kernel are inside the absent library.  Pinned as mathematics: the generator
  *                  by the published Philox4x32-10 known answers, the deviates by their moments, the
@@ -816,14 +819,31 @@ ORC_API void orc_vv_post(float* vel, const float* forces, const float* masses, c
 }
 
 /* ------------------------------------------------------------------------------------------
- * FIRE step (vanilla branch).  Reductions vf, vv, ff per system in double at entry, then
- *   P > 0 : v <- (1-alpha) v + alpha sqrt(vv/ff) F   with the STORED alpha;
- *           n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max), alpha *= f_alpha
- *   else  : v <- 0 ; n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
- *   MD    : v += dt F/m (clamped to +-3e38) ; dr = dt v ; |dr| > maxstep -> dr *= maxstep/|dr| ;
- *           r += dr   (|dr| is evaluated scaled by its largest component, so it cannot overflow)
+ * FIRE step (vanilla branch).  PARITY UNPINNED against the reference: the step itself is in a
+ * kernel library that is not in the reference's tree.  The order below is the one the reference's
+ * own sentences give, each choice with the sentence that decides it:
+ *   1 reductions vf = sum F.v, vv = sum v.v, ff = sum F.F per system over the velocities and
+ *     forces AS PASSED IN (double accumulation): nvalchemi/distributed/_dynamics_coordinator.py:
+ *     296-322,325-396 computes them before the call from the same arrays and hands them over with
+ *     compute_reductions=False as "the ones the op would compute"; _ops/fire.py:317-322.
+ *   2 MD integration with the STORED dt: v1 = v + dt F/m (clamped to +-3e38) ; dr = dt v1 ;
+ *     |dr| > maxstep -> dr *= maxstep/|dr| per atom ; r += dr.  "Performs an MD integration step
+ *     followed by FIRE velocity mixing and adaptive parameter updates" (_ops/fire.py:270-272),
+ *     "full FIRE step (MD integration + mixing)" (optimizers/fire.py:31-32); the per-atom clamp:
+ *     _dynamics_coordinator.py:329-331.  Semi-implicit Euler (kick, then drift) and the norm of
+ *     the clamp are this file's choice: no sentence decides them.
+ *   3 mixing with the STORED alpha (test/distributed/test_fire_dd.py:39-50: every atom is meant to
+ *     mix with the alpha of before the update):
+ *       P >= 0 : v <- (1-alpha) v1 + alpha sqrt(vv/ff) F      P < 0 : v <- 0
+ *   4 parameter update:  P >= 0 : n+ += 1 ; if n+ > n_min : dt = min(dt f_inc, dt_max),
+ *     alpha *= f_alpha        P < 0 : n+ = 0 ; dt = max(dt f_dec, dt_min) ; alpha = alpha_start
+ * Where the zero of P belongs is not said anywhere.  It goes with the downhill branch here
+ * because, with the reductions taken at entry and the velocities zeroed after the integration, a
+ * system that starts at rest (P = 0 on every entry) would otherwise never gain a velocity.
+ * n+ > n_min (rather than >=) is likewise undecided.
  * Every atom of a system uses the same pre-update scalars.  vf/vv/ff outputs are the
- * float32-rounded reductions.
+ * float32-rounded reductions.  |dr| is evaluated scaled by its largest component, so it cannot
+ * overflow.
  * ---------------------------------------------------------------------------------------- */
 ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const float* masses,
                            float* alpha, float* dt, const float* alpha_start,
@@ -835,7 +855,7 @@ ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const fl
     double* acc = (double*)calloc((size_t)n_systems * 3, sizeof(double));
     float* mixa = (float*)malloc(sizeof(float) * n_systems);
     float* mixb = (float*)malloc(sizeof(float) * n_systems);
-    float* dtn = (float*)malloc(sizeof(float) * n_systems);
+    float* dtu = (float*)malloc(sizeof(float) * n_systems);
     for (int i = 0; i < n_atoms; ++i) {
         int s = batch_idx[i];
         for (int a = 0; a < 3; ++a) {
@@ -848,9 +868,9 @@ ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const fl
     for (int s = 0; s < n_systems; ++s) {
         double P = acc[3 * s], VV = acc[3 * s + 1], FF = acc[3 * s + 2];
         vf[s] = (float)P; vv[s] = (float)VV; ff[s] = (float)FF;
-        dtn[s] = dt[s]; mixa[s] = 1.0f; mixb[s] = 0.0f;
+        dtu[s] = dt[s]; mixa[s] = 1.0f; mixb[s] = 0.0f;
         if (active && !active[s]) continue;
-        if (P > 0.0) {
+        if (P >= 0.0) {
             float al = alpha[s];
             mixa[s] = 1.0f - al;
             mixb[s] = (FF > 0.0) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
@@ -867,18 +887,16 @@ ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const fl
             dt[s] = nd > dt_min[s] ? nd : dt_min[s];
             alpha[s] = alpha_start[s];
         }
-        dtn[s] = dt[s];
     }
     for (int i = 0; i < n_atoms; ++i) {
         int s = batch_idx[i];
         if (active && !active[s]) continue;
-        float h = dtn[s], m = masses[i], ms = maxstep[s];
+        float h = dtu[s], m = masses[i], ms = maxstep[s];
         float dr[3], v[3];
         for (int a = 0; a < 3; ++a) {
             float f = forces[3 * i + a];
-            float vm = (mixa[s] * vel[3 * i + a]) + (mixb[s] * f);
             float acc1 = f / m;
-            v[a] = vm + (h * acc1);
+            v[a] = vel[3 * i + a] + (h * acc1);
             v[a] = fminf(fmaxf(v[a], -ORC_VMAX), ORC_VMAX); /* keep dr finite */
             dr[a] = h * v[a];
         }
@@ -894,11 +912,12 @@ ORC_API void orc_fire_step(float* pos, float* vel, const float* forces, const fl
             for (int a = 0; a < 3; ++a) dr[a] = dr[a] * sc;
         }
         for (int a = 0; a < 3; ++a) {
-            vel[3 * i + a] = v[a];
+            float f = forces[3 * i + a];
+            vel[3 * i + a] = (mixa[s] * v[a]) + (mixb[s] * f);
             pos[3 * i + a] = pos[3 * i + a] + dr[a];
         }
     }
-    free(acc); free(mixa); free(mixb); free(dtn);
+    free(acc); free(mixa); free(mixb); free(dtu);
 }
 
 /* per-system max over atoms of the float32 force norm (reference: vector_norm then

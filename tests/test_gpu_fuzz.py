@@ -56,8 +56,7 @@ def T(a, dtype=None):
 def test_random_case(seed, monkeypatch):
     from nvalchemi_amd import _lib
 
-    if seed % 2:
-        monkeypatch.setenv("NVAMD_NL_NO_PER_SYSTEM", "1")
+    monkeypatch.setattr(_lib, "nl_sort_path", _lib.NL_SORT_GLOBAL if seed % 2 else _lib.NL_SORT_PER_SYSTEM)
     P, C, pb, ptr, rc, half = random_case(seed)
     N, B = len(P), len(ptr) - 1
     ref = oracle.nl_brute(P, C, pb, ptr, rc, half=half)

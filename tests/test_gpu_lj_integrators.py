@@ -241,6 +241,40 @@ def test_fire_matches_oracle_over_many_steps(masked):
         tv.copy_(T(v))
 
 
+def test_fire_order_of_the_reference_sentences_through_the_abi():
+    """The literal numbers of tests/test_oracle_integrators.py (integration with the stored dt first,
+    then the mixing with the reductions of entry; nvalchemi/dynamics/_ops/fire.py:270-272), from the
+    kernels: one atom, v = 1, F = 2 -> r = 0.12, v = 1.18; v = 1, F = -2 -> r = 0.08, v = 0, dt halved."""
+    from nvalchemi_amd.dynamics._ops.fire import fire_step
+
+    for F0, r1, v1, dt1, np1 in ((2.0, 0.12, 1.18, 0.1, 1), (-2.0, 0.08, 0.0, 0.05, 0)):
+        f32 = lambda x: torch.full((1,), x, dtype=torch.float32, device=DEV)  # noqa: E731
+        i32 = lambda x: torch.full((1,), x, dtype=torch.int32, device=DEV)  # noqa: E731
+        r = torch.zeros(1, 3, device=DEV)
+        v = torch.tensor([[1.0, 0, 0]], device=DEV)
+        f = torch.tensor([[F0, 0, 0]], device=DEV)
+        alpha, dt, npos = f32(0.1), f32(0.1), i32(0)
+        fire_step(r, v, f, torch.ones(1, device=DEV), alpha, dt, npos, f32(0.1), f32(0.99), f32(0.002), f32(1.0),
+                  f32(0.2), i32(5), f32(0.5), f32(1.1), i32(0))
+        assert float(r[0, 0]) == pytest.approx(r1, rel=1e-6)
+        assert float(v[0, 0]) == pytest.approx(v1, rel=1e-6, abs=0)
+        assert float(dt[0]) == pytest.approx(dt1, rel=1e-6) and int(npos[0]) == np1
+
+
+def test_fire_step_refuses_the_uphill_branch():
+    from nvalchemi_amd.dynamics._ops.fire import fire_step
+
+    f32 = lambda x: torch.full((2,), x, dtype=torch.float32, device=DEV)  # noqa: E731
+    i32 = lambda x: torch.full((2,), x, dtype=torch.int32, device=DEV)  # noqa: E731
+    r = torch.zeros(4, 3, device=DEV)
+    uph = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+    with pytest.raises(NotImplementedError):
+        fire_step(r, torch.zeros_like(r), torch.ones_like(r), torch.ones(4, device=DEV), f32(0.1), f32(0.1), i32(0),
+                  f32(0.1), f32(0.99), f32(0.002), f32(1.0), f32(0.2), i32(5), f32(0.5), f32(1.1), uph,
+                  batch_idx=torch.tensor([0, 0, 1, 1], dtype=torch.int32, device=DEV))
+    assert float(r.abs().max()) == 0.0
+
+
 def test_fire_survives_huge_forces():
     from nvalchemi_amd import _lib
 

@@ -21,11 +21,11 @@ DEV = "cuda:0"
 def sort_path(request, monkeypatch):
     """Every test runs twice: with the workgroup-per-system sort that batches of small systems
     take by default, and with the global histogram/scan/scatter pipeline that large systems take
-    (forced here through the library's environment switch, which is read on every call)."""
-    if request.param == "global_sort":
-        monkeypatch.setenv("NVAMD_NL_NO_PER_SYSTEM", "1")
-    else:
-        monkeypatch.delenv("NVAMD_NL_NO_PER_SYSTEM", raising=False)
+    (nvamd_nl_build_path's sort_path argument, through the binding's default for it)."""
+    from nvalchemi_amd import _lib
+
+    monkeypatch.setattr(_lib, "nl_sort_path",
+                        _lib.NL_SORT_GLOBAL if request.param == "global_sort" else _lib.NL_SORT_PER_SYSTEM)
     return request.param
 
 

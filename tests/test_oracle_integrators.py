@@ -73,22 +73,73 @@ def _fire_state(M, dt=0.1, **kw):
     return st
 
 
-def test_fire_hand_worked_first_two_steps():
+def _one_atom(v0, F0):
     r = np.zeros((1, 3), dtype=np.float32)
-    v = np.zeros((1, 3), dtype=np.float32)
-    F = np.array([[2.0, 0, 0]], dtype=np.float32)
-    m = np.ones(1, dtype=np.float32)
+    v = np.array([[v0, 0, 0]], dtype=np.float32)
+    F = np.array([[F0, 0, 0]], dtype=np.float32)
+    return r, v, F, np.ones(1, dtype=np.float32)
+
+
+def test_fire_integrates_first_then_mixes_with_the_reductions_of_entry():
+    """nvalchemi/dynamics/_ops/fire.py:270-272: "an MD integration step followed by FIRE velocity mixing
+    and adaptive parameter updates".  One atom, v = 1, F = 2, m = 1, dt = 0.1, alpha = 0.1; the expected
+    numbers come from that sentence and from the reductions being those of the arrays passed in
+    (nvalchemi/distributed/_dynamics_coordinator.py:296-322), not from the oracle's code:
+      kick   v1 = 1 + 0.1*2 = 1.2 ; drift r = 0.1*1.2 = 0.12
+      mix    |v|/|F| from entry = 1/2 :  v = 0.9*1.2 + 0.1*0.5*2 = 1.18
+    The orders this rules out give other numbers:
+      mix first, then integrate (Bitzek/ASE):   v = (0.9*1 + 0.1) + 0.2 = 1.2,  r = 0.12
+      reductions after the kick (|v1|/|F| = .6): v = 0.9*1.2 + 0.1*0.6*2 = 1.2
+      drift with the mixed velocity:             r = 0.118
+    """
+    r, v, F, m = _one_atom(1.0, 2.0)
     st = _fire_state(1)
     oracle.fire_step(r, v, F, m, st, [0])
-    # P = 0 is not > 0: dt halves, alpha resets, v zeroed; then v = dt F/m, r += dt v
-    assert st["dt"][0] == np.float32(0.05) and st["n_steps_positive"][0] == 0
-    assert v[0, 0] == pytest.approx(0.1, rel=1e-6) and r[0, 0] == pytest.approx(0.005, rel=1e-6)
-    assert st["vf"][0] == 0 and st["ff"][0] == 4
+    assert st["vf"][0] == 2 and st["vv"][0] == 1 and st["ff"][0] == 4  # of the entry arrays
+    assert r[0, 0] == pytest.approx(0.12, rel=1e-6)
+    assert v[0, 0] == pytest.approx(1.18, rel=1e-6)
+    assert abs(float(v[0, 0]) - 1.2) > 1e-3
+    assert st["n_steps_positive"][0] == 1 and st["dt"][0] == np.float32(0.1) and st["alpha"][0] == np.float32(0.1)
+
+
+def test_fire_uphill_step_is_integrated_with_the_stored_dt_before_the_reset():
+    """F.v < 0 at entry: the integration still happens first, with the time step of before the
+    update, and only then are the velocities zeroed and dt halved.  A mix-first order would move the
+    atom by dt'^2 F/m = -0.005 with the halved dt' and leave v = dt' F/m = -0.1."""
+    r, v, F, m = _one_atom(1.0, -2.0)
+    st = _fire_state(1)
+    st["n_steps_positive"][:] = 3
     oracle.fire_step(r, v, F, m, st, [0])
-    # P = 0.2 > 0: v <- 0.9*0.1 + 0.1*(0.1/2)*2 = 0.1 ; n+ = 1 <= n_min ; v += 0.05*2 ; r += 0.05*0.2
-    assert st["vf"][0] == pytest.approx(0.2, rel=1e-6) and st["n_steps_positive"][0] == 1
-    assert st["dt"][0] == np.float32(0.05) and st["alpha"][0] == np.float32(0.1)
-    assert v[0, 0] == pytest.approx(0.2, rel=1e-6) and r[0, 0] == pytest.approx(0.015, rel=1e-6)
+    assert r[0, 0] == pytest.approx(0.1 * (1.0 - 0.2), rel=1e-6)  # dt (v + dt F/m) with dt = 0.1
+    assert v[0, 0] == 0.0
+    assert st["dt"][0] == np.float32(0.05) and st["alpha"][0] == np.float32(0.1) and st["n_steps_positive"][0] == 0
+
+
+def test_fire_the_time_step_grown_by_a_step_is_first_used_by_the_next():
+    """Parameter updates come last: the step that grows dt (n+ passes n_min) still integrates with
+    the old one."""
+    r, v, F, m = _one_atom(1.0, 2.0)
+    st = _fire_state(1)
+    st["n_steps_positive"][:] = 5
+    oracle.fire_step(r, v, F, m, st, [0])
+    assert r[0, 0] == pytest.approx(0.12, rel=1e-6)  # 0.1 * 1.2, not 0.11 * 1.22
+    assert st["dt"][0] == pytest.approx(0.11, rel=1e-6) and st["alpha"][0] == pytest.approx(0.099, rel=1e-6)
+    v1 = float(v[0, 0])
+    oracle.fire_step(r, v, F, m, st, [0])
+    assert r[0, 0] == pytest.approx(0.12 + 0.11 * (v1 + 0.11 * 2.0), rel=1e-6)
+
+
+def test_fire_leaves_rest():
+    """A system at rest has F.v = 0 on entry.  With the velocities reset AFTER the integration, that
+    zero has to count as downhill, or the velocity gained by the kick would be thrown away on every
+    step and the system would creep at dt_min for ever."""
+    r, v, F, m = _one_atom(0.0, 2.0)
+    st = _fire_state(1)
+    oracle.fire_step(r, v, F, m, st, [0])
+    assert v[0, 0] == pytest.approx(0.9 * 0.2, rel=1e-6) and r[0, 0] == pytest.approx(0.02, rel=1e-6)
+    assert st["dt"][0] == np.float32(0.1) and st["n_steps_positive"][0] == 1
+    oracle.fire_step(r, v, F, m, st, [0])
+    assert st["vf"][0] > 0 and v[0, 0] > 0.18
 
 
 def test_fire_dt_growth_after_n_min_and_caps():
@@ -102,11 +153,11 @@ def test_fire_dt_growth_after_n_min_and_caps():
         oracle.fire_step(r, v, F, m, st, [0])
         dts.append(float(st["dt"][0]))
         alphas.append(float(st["alpha"][0]))
-    # step 1 shrinks; steps 2..6 are positive steps 1..5 (no growth); growth starts at the 6th
-    assert dts[0] == pytest.approx(0.05) and dts[5] == pytest.approx(0.05)
-    assert dts[6] == pytest.approx(0.05 * 1.1, rel=1e-6) and alphas[6] == pytest.approx(0.099, rel=1e-6)
+    # steps 1..5 are downhill steps 1..5 (no growth); growth starts at the 6th
+    assert dts[0] == pytest.approx(0.1) and dts[4] == pytest.approx(0.1)
+    assert dts[5] == pytest.approx(0.1 * 1.1, rel=1e-6) and alphas[5] == pytest.approx(0.099, rel=1e-6)
     assert max(dts) == pytest.approx(1.0, rel=1e-6)  # dt_max = 10 dt
-    assert all(b >= a for a, b in zip(dts[1:], dts[2:]))
+    assert all(b >= a for a, b in zip(dts, dts[1:]))
 
 
 def test_fire_maxstep_clamp_is_per_atom():
@@ -118,7 +169,7 @@ def test_fire_maxstep_clamp_is_per_atom():
     oracle.fire_step(r, v, F, m, st, [0, 0])
     assert np.linalg.norm(r[0]) == pytest.approx(0.2, rel=1e-5)
     assert r[0, 0] / r[0, 1] == pytest.approx(0.75, rel=1e-5)
-    assert r[1, 0] == pytest.approx(0.05 * 0.05 * 1e-3, rel=1e-5)
+    assert r[1, 0] == pytest.approx(0.1 * 0.1 * 1e-3, rel=1e-5)
 
 
 def test_fire_relaxes_a_quadratic_bowl_and_respects_masks():
