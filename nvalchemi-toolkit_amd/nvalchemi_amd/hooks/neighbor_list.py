@@ -13,7 +13,8 @@ batch tensors directly), and the padding of rows is maintained by the build kern
 instead of a masked fill over the whole ``(N,K)`` buffers after every build (:377-380).
 With ``skin > 0`` the list is searched out to ``cutoff + skin`` and, from the second call on, only
 the systems in which some atom moved more than ``skin / 2`` since their last build are rebuilt
-(:295-311): the displacement test writes the per-system ``_rebuild_flags`` and refreshes
+(:295-311; the displacement is the plain one, so that an atom wrapped back into the cell by another
+hook counts as moved and the shifts of its system are made afresh): the displacement test writes the per-system ``_rebuild_flags`` and refreshes
 ``_ref_positions`` for the flagged systems, and the build kernel leaves the rows of the others as
 they are.  The potential applies the bare cutoff to the wider list.
 """
@@ -106,11 +107,16 @@ class NeighborListHook:
             self._rebuild_flags = torch.ones(B, dtype=torch.bool, device=positions.device)
             self._ref_positions = None
         if self.skin > 0.0 and self._ref_positions is not None:
+            # The displacement is the plain one, not the one reduced to the nearest image (the
+            # reference passes its cell here, nvalchemi/hooks/neighbor_list.py:295-311): rows that are
+            # kept hold integer shifts that belong to the coordinates they were built from, so an
+            # atom that a wrap has moved by a lattice vector must count as moved, and its system is
+            # rebuilt.  (Only a lattice vector shorter than skin / 2 would escape this.)
             batch_neighbor_list_rebuild_inplace(
                 reference_positions=self._ref_positions, current_positions=positions,
                 batch_idx=batch.batch_idx, rebuild_flags=self._rebuild_flags,
                 skin_distance_threshold=self.skin / 2, update_reference_positions=True,
-                cell=cell if periodic else None, pbc=pbc)
+                cell=None, pbc=None)
 
         cutoff = self.config.cutoff + self.skin
         self._build(batch, cutoff, cell, pbc,

@@ -236,3 +236,47 @@ def test_wrap_hook_in_a_periodic_run_changes_nothing_physical():
     assert abs(float(res[True].energy.sum() - res[False].energy.sum())) < 1e-4 * abs(float(res[False].energy.sum()))
     d = (res[True].positions - res[False].positions).cpu().numpy().astype(np.float64) / 10.8
     assert np.abs(d - np.round(d)).max() < 1e-4
+
+
+def test_skin_and_wrap_together_on_cells_whose_shifts_are_read():
+    """Cells narrower than twice the search radius (the pair kernel reads the stored shifts there) with a
+    Verlet skin AND the wrap hook: an atom that the wrap moves by a lattice vector between two builds
+    must make its system's list be built afresh, or the kept rows would pair its new coordinates with the
+    shifts of the old ones.  The run with the wrap must be the run without it, up to lattice vectors."""
+    from nvalchemi_amd.dynamics import NVE
+    from nvalchemi_amd.dynamics.base import DynamicsStage
+    from nvalchemi_amd.hooks import WrapPeriodicHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=3, n_boxes=3, reps=2, a=3.6)  # 7.2 wide: less than 2 (4.5 + 0.5)
+    N = len(P)
+    M = np.full(N, 63.546, dtype=np.float32)
+    V = np.tile(np.array([[0.35, -0.25, 0.15]], np.float32), (N, 1))  # a drift that carries atoms across the faces
+    V += np.random.default_rng(5).normal(0, 0.01, (N, 3)).astype(np.float32)
+    Z = np.full(N, 29, dtype=np.int64)
+    sig = float((3.6 / np.sqrt(2)) / 2 ** (1 / 6))
+    res, kept = {}, 0
+    for wrap in (False, True):
+        batch = make_batch(P, Z, M, C, pb, ptr, V)
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=sig, cutoff=4.5)
+        hooks = model.make_neighbor_hooks()
+        for h in hooks:
+            h.skin = 0.5
+        if wrap:
+            hooks.append(WrapPeriodicHook(frequency=1, stage=DynamicsStage.AFTER_POST_UPDATE))
+        dyn = NVE(model, dt=2.0, hooks=hooks)
+        for _ in range(100):
+            dyn.run(batch, n_steps=1)
+            if wrap and not bool(hooks[0]._rebuild_flags.all()):
+                kept += 1
+        res[wrap] = batch
+    assert kept > 20  # the skin did keep lists in the wrapped run
+    assert np.abs(res[False].positions.cpu().numpy() / 7.2).max() > 1.3  # atoms did leave the box
+    frac = res[True].positions.cpu().numpy().astype(np.float64) / 7.2
+    assert frac.min() > -0.02 and frac.max() < 1.02
+    for key, tol in (("forces", 2e-4), ("velocities", 2e-5)):
+        a = getattr(res[True], key).cpu().numpy().astype(np.float64)
+        b = getattr(res[False], key).cpu().numpy().astype(np.float64)
+        assert np.abs(a - b).max() < tol, (key, np.abs(a - b).max())
+    d = (res[True].positions - res[False].positions).cpu().numpy().astype(np.float64) / 7.2
+    assert np.abs(d - np.round(d)).max() < 1e-4
