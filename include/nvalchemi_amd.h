@@ -264,6 +264,29 @@ int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells
                                       float* system_energies, void* workspace, size_t workspace_bytes,
                                       void* stream);
 
+/* nvamd_lj_energy_forces_hinted for callers that cannot allocate device memory or carry a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
+ * the reference.  The scratch of the pair kernel (per-system float64 accumulators, first and last atom of
+ * each system) lives in a device array built into the library, NVAMD_LJ_STATIC_SCRATCH_BYTES per GPU,
+ * held until the process ends; the call allocates and frees nothing.  Limits: full list only (there is
+ * no half_list argument), n_systems <= NVAMD_LJ_STATIC_MAX_SYSTEMS (more returns NVAMD_ERR_UNSUPPORTED);
+ * n_atoms is not limited.  The first call on a device looks up the array's address
+ * (hipGetSymbolAddress): make it outside a graph capture.  All calls on one GPU share the one array:
+ * calls that overlap on a GPU (two streams, two threads) race; what has to start at zero is cleared
+ * by every call.  Results are those of nvamd_lj_energy_forces_hinted. */
+#define NVAMD_LJ_STATIC_MAX_SYSTEMS 16384
+#define NVAMD_LJ_STATIC_SCRATCH_BYTES \
+    ((((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 80 + 255) / 256 + 2 * (((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 4 + 255) / 256)) * 256)
+int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells,
+                                      const int32_t* neighbor_matrix,
+                                      const int32_t* neighbor_matrix_shifts,
+                                      const int32_t* num_neighbors, const int32_t* batch_idx,
+                                      const int32_t* row_order, double neighbor_list_cutoff, int32_t n_atoms,
+                                      int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
+                                      double epsilon, double sigma, double cutoff, double switch_width,
+                                      float* atomic_energies, float* forces, float* virials,
+                                      float* system_energies, void* stream);
+
 /* Atom indices in the cell order of the neighbor build that last used this workspace with the same
  * n_atoms / n_systems: atom_order[k] for k in a system's range [batch_ptr[s], batch_ptr[s+1]) are that
  * system's atoms, cell by cell.  With rebuild_flags, only the ranges of flagged systems are written

@@ -14,6 +14,8 @@
 // wavefront.  Per-system energy and virial go through one fp64 atomic per run of rows
 // of the same system per workgroup.  Pair math is double on the float32 inputs
 // ("internal math is performed in float64", nvalchemi/models/_ops/lj.py:49-50).
+#include <mutex>
+
 #include "common.h"
 #include "geom.h"
 
@@ -725,4 +727,59 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const
                                  row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
                                  sigma, cutoff, switch_width, half_list, atomic_energies, forces, virials,
                                  system_energies, workspace, workspace_bytes, stream);
+}
+
+// ---- the variant that allocates nothing ------------------------------------------------------
+// For callers that cannot allocate or bring a workspace (code under HIP graph capture, tight serving
+// loops): the pair kernel's scratch (per-system fp64 accumulators, first and last atom of each
+// system) lives in a file-scope device array of fixed size.  Every GPU holds its own copy of the
+// array at its own address, found once per device with hipGetSymbolAddress; from then on only that
+// pointer is used (the array's name is a host-side stand-in, not a device address).
+namespace {
+constexpr int kStaticMaxSystems = NVAMD_LJ_STATIC_MAX_SYSTEMS;
+constexpr size_t kStaticScratchBytes = NVAMD_LJ_STATIC_SCRATCH_BYTES;
+constexpr int kStaticMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kStaticMaxDevices];  // per device; null until the first call on it
+static std::mutex g_scratch_mutex;
+
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells,
+                                                    const int32_t* neighbor_matrix,
+                                                    const int32_t* neighbor_matrix_shifts,
+                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
+                                                    const int32_t* row_order, double neighbor_list_cutoff,
+                                                    int32_t n_atoms, int32_t max_neighbors, int32_t n_systems,
+                                                    int32_t fill_value, double epsilon, double sigma, double cutoff,
+                                                    double switch_width, float* atomic_energies, float* forces,
+                                                    float* virials, float* system_energies, void* stream) {
+    if (n_systems > kStaticMaxSystems)
+        return fail(NVAMD_ERR_UNSUPPORTED, "lj (static scratch): %d systems, the built-in scratch holds at most %d",
+                    (int)n_systems, kStaticMaxSystems);
+    size_t need = 0;
+    if (nvamd_lj_workspace_bytes(n_atoms, n_systems, 0, &need) != NVAMD_OK) return NVAMD_ERR_INVALID_ARGUMENT;
+    if (need > kStaticScratchBytes)
+        return fail(NVAMD_ERR_UNSUPPORTED, "lj (static scratch): needs %zu bytes, has %zu", need, kStaticScratchBytes);
+    int dev = -1;
+    int32_t rc = check_hip(hipGetDevice(&dev), "lj (static scratch): hipGetDevice");
+    if (rc != NVAMD_OK) return rc;
+    if (dev < 0 || dev >= kStaticMaxDevices)
+        return fail(NVAMD_ERR_UNSUPPORTED, "lj (static scratch): device %d out of range", dev);
+    void* ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[dev]) {
+            void* p = nullptr;
+            rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "lj (static scratch): hipGetSymbolAddress");
+            if (rc != NVAMD_OK) return rc;
+            if (!p) return fail(NVAMD_ERR_HIP, "lj (static scratch): null symbol address on device %d", dev);
+            g_scratch_ptr[dev] = p;
+        }
+        ptr = g_scratch_ptr[dev];
+    }
+    // full list only: the half-list kernel needs 32 bytes of scratch per atom
+    return lj_energy_forces_impl(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors, batch_idx,
+                                 row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
+                                 sigma, cutoff, switch_width, /*half_list=*/0, atomic_energies, forces, virials,
+                                 system_energies, ptr, kStaticScratchBytes, stream);
 }

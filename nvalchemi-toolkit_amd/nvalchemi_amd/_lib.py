@@ -44,6 +44,7 @@ _SIGNATURES = {
     "nvamd_fire_step": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_lj_energy_forces_hinted": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
+    "nvamd_lj_energy_forces_static": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_vp] * 5),
     "nvamd_nl_atom_order": (_i32, [_vp, _c.c_size_t, _vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_segment_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_segment_reduce": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
@@ -257,6 +258,36 @@ def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, 
         _opt(virials, "virials", torch.float32, (B, 9)),
         _opt(system_energies, "system_energies", torch.float32, (B,)),
         ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_hinted")
+
+
+LJ_STATIC_MAX_SYSTEMS = 16384
+
+
+def lj_energy_forces_static(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
+                            batch_idx, fill_value, epsilon, sigma, cutoff, switch_width,
+                            atomic_energies, forces, virials=None, system_energies=None, row_order=None,
+                            neighbor_list_cutoff: float = 0.0) -> None:
+    """``lj_energy_forces`` (full list) through the entry point that allocates nothing: the kernel's
+    scratch is a device array built into the library (at most ``LJ_STATIC_MAX_SYSTEMS`` systems;
+    calls that overlap on one GPU race)."""
+    lib = library()
+    N = positions.shape[0]
+    K = neighbor_matrix.shape[1]
+    B = cells.shape[0]
+    _check(lib.nvamd_lj_energy_forces_static(
+        _dev(positions, "positions", torch.float32, (N, 3)),
+        _dev(cells, "cells", torch.float32, (B, 3, 3)),
+        _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+        _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+        _dev(num_neighbors, "num_neighbors", torch.int32, (N,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _opt(row_order, "row_order", torch.int32, (N,)), float(neighbor_list_cutoff),
+        N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), float(switch_width),
+        _dev(atomic_energies, "atomic_energies", torch.float32, (N,)),
+        _dev(forces, "forces", torch.float32, (N, 3)),
+        _opt(virials, "virials", torch.float32, (B, 9)),
+        _opt(system_energies, "system_energies", torch.float32, (B,)),
+        _stream(positions.device)), "nvamd_lj_energy_forces_static")
 
 
 def nl_atom_order(batch_idx, n_systems: int, atom_order, rebuild_flags=None) -> None:
