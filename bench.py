@@ -4,7 +4,7 @@
 
 Workload (the configuration the metric is quoted on): 256 periodic cubic Lennard-Jones
 liquid boxes of 3900 atoms (998 400 atoms), reduced units, density 0.8 sigma^-3, uniform
-random positions (seed 0) relaxed by 50 FIRE steps, then NVE velocity Verlet with dt = 0.005,
+random positions (seed 0) relaxed by 50 FIRE steps (dt 0.005, maxstep 0.07 sigma), then NVE velocity Verlet with dt = 0.005,
 cutoff 2.5 sigma, the neighbor list rebuilt on every step.  One step is one pass of the hot
 path through the package's own API: ``NVE.step`` = velocity-Verlet position update ->
 ``NeighborListHook`` (cell-list build) -> ``LennardJonesModelWrapper`` (pair kernel + per-system
@@ -34,6 +34,9 @@ for p in (ROOT, ROOT / "nvalchemi-toolkit_amd"):
         sys.path.insert(0, str(p))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# largest displacement of an atom per FIRE step of the relaxation, in sigma (the optimizer's default of 0.2 is
+# meant for Angstrom-sized atoms; from a random gas it lets overlapping atoms jump through each other)
+RELAX_MAXSTEP = 0.07
 
 # HBM bytes per launch on the default workload (256 boxes, seed 0), from rocprofv3 --pmc runs of
 # this script (FETCH_SIZE, then WRITE_SIZE; averages over the timed steps).  FETCH_SIZE reads
@@ -167,7 +170,7 @@ def main() -> int:
     model = LennardJonesModelWrapper(epsilon=1.0, sigma=1.0, cutoff=rc)
 
     t0 = time.perf_counter()
-    relax = FIRE(model, dt=dt, hooks=model.make_neighbor_hooks())
+    relax = FIRE(model, dt=dt, maxstep=RELAX_MAXSTEP, hooks=model.make_neighbor_hooks())
     relax.run(batch, n_steps=args.relax_steps)
     torch.cuda.synchronize()
     log(f"[bench] N={N} B={B} L={L:.3f}; {args.relax_steps} FIRE steps in {time.perf_counter() - t0:.2f}s; "

@@ -139,7 +139,7 @@ def test_fcc_batch_of_64_boxes_against_the_oracle():
 
 def relaxed_liquid(B, n, rho, rc, steps=50):
     """The quoted workload's own preparation: uniform random positions (seed 0) relaxed by 50 FIRE steps
-    (dt 0.005, the optimizer's defaults) of the package's own FIRE over its own neighbor hook and model."""
+    (dt 0.005, maxstep 0.07 sigma, as bench.py does) of the package's own FIRE over its own neighbor hook and model."""
     from nvalchemi_amd.data import AtomicData, Batch
     from nvalchemi_amd.dynamics import FIRE
     from nvalchemi_amd.models import LennardJonesModelWrapper
@@ -151,7 +151,7 @@ def relaxed_liquid(B, n, rho, rc, steps=50):
                        forces=torch.zeros(n, 3), energy=torch.zeros(1, 1)) for _ in range(B)]
     batch = Batch.from_data_list(data, device=DEV)
     model = LennardJonesModelWrapper(epsilon=1.0, sigma=1.0, cutoff=rc)
-    FIRE(model, dt=0.005, hooks=model.make_neighbor_hooks()).run(batch, n_steps=steps)
+    FIRE(model, dt=0.005, maxstep=0.07, hooks=model.make_neighbor_hooks()).run(batch, n_steps=steps)
     torch.cuda.synchronize()
     return batch.positions.detach().clone().contiguous(), batch.cell.detach().clone().contiguous(), L
 
