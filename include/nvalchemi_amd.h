@@ -276,7 +276,8 @@ int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells
  * by every call.  Results are those of nvamd_lj_energy_forces_hinted. */
 #define NVAMD_LJ_STATIC_MAX_SYSTEMS 16384
 #define NVAMD_LJ_STATIC_SCRATCH_BYTES \
-    ((((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 80 + 255) / 256 + 2 * (((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 4 + 255) / 256)) * 256)
+    ((((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 80 + 255) / 256 + 2 * (((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 4 + 255) / 256) + \
+      ((size_t)NVAMD_LJ_STATIC_MAX_SYSTEMS * 96 + 255) / 256) * 256)
 int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells,
                                       const int32_t* neighbor_matrix,
                                       const int32_t* neighbor_matrix_shifts,

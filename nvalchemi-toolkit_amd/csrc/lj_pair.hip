@@ -4,16 +4,18 @@
 // nvalchemi::lj_energy_forces_virial_batch (nvalchemi/models/_ops/lj.py:116-216,246-321),
 // plus the per-system fp64 energy scatter of nvalchemi/models/lj.py:467-477, fused here.
 //
-// Bound: HBM.  Per directed edge the kernel must read the neighbor index (4 B) and the
-// shift (12 B); per atom it reads its position once through the row owner and writes
-// energy and force.  Work decomposition: LPR lanes of a wavefront own one row of the
-// matrix (LPR = 8..64 chosen from the row width), so the row and its shifts are read as
-// contiguous segments, the neighbor positions are gathered through L2 (a system's atoms
-// are contiguous in index space, and workgroups are laid out so that one XCD's L2 serves
-// one contiguous slice of atoms), and the row sum is a shuffle reduction inside the
-// wavefront.  Per-system energy and virial go through one fp64 atomic per run of rows
-// of the same system per workgroup.  Pair math is double on the float32 inputs
-// ("internal math is performed in float64", nvalchemi/models/_ops/lj.py:49-50).
+// Work decomposition: a workgroup of 512 lanes owns a run of consecutive rows of the matrix and takes
+// them one system at a time, with that system's positions staged in LDS when they fit (atom order
+// carries no spatial locality); LPR lanes of a wavefront own one row (LPR = 8..64 chosen from the row
+// width) and read its indices, and its shifts where they are needed, as 16-byte vectors; the row sum
+// is a reduction inside the wavefront.  Where the neighbor list's search radius is below half of
+// every perpendicular width of a system's cell, the shifts are not read at all but follow from the
+// positions (the listed image of a pair is then the nearest one): 4 instead of 16 bytes per pair.
+// Per-system energy and virial go through LDS accumulators and one fp64 atomic per workgroup and
+// system.  Pair math is double on the float32 inputs ("internal math is performed in float64",
+// nvalchemi/models/_ops/lj.py:49-50).
+// Bound: with the shifts read, HBM; with the shifts derived, the double-precision pair arithmetic
+// (about 70 vector instructions per pair) and the latency of its operands.
 #include <mutex>
 
 #include "common.h"
@@ -47,6 +49,7 @@ struct LjArgs {
     const int32_t* order;      // (N) row k of the kernel's walk is atom order[k]; null: the identity
     const int32_t* sys_first;  // (B) first atom of each non-empty system
     const int32_t* sys_last;   // (B) one past its last atom
+    const struct LjSysImage* sys_image;  // (B) how the images of its pairs are found
     int lds_atoms;             // stage positions in LDS when the systems of a run have at most this many atoms
     double list_rc;            // cutoff the neighbor list was built with (0: unknown, shifts are always read)
     double r_on, inv_sw;       // switching region [r_on, cutoff] and 1 / its width (0, 0: no switching)
@@ -67,10 +70,24 @@ __device__ __forceinline__ void apply_switch(const LjArgs& a, double r2, double&
     u = u * S;
 }
 
+// Sum over the LPR lanes of a row, valid in the row's first lane only.  Steps below 16 lanes are
+// data-parallel moves inside a row of 16 lanes (lane i takes lane i + o): no lane numbers to keep in
+// registers and no trip through the LDS crossbar.
+template <int O>
+__device__ __forceinline__ double lane_above(double v) {
+    static_assert(O >= 1 && O < 16, "a shift inside a row of 16 lanes");
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), 0x100 + O, 0xf, 0xf, true);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), 0x100 + O, 0xf, 0xf, true);
+    return __hiloint2double(hi, lo);
+}
 template <int LPR>
 __device__ __forceinline__ double group_sum(double v) {
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    if (LPR > 32) v += __shfl_xor(v, 32, kWave);
+    if (LPR > 16) v += __shfl_xor(v, 16, kWave);
+    if (LPR > 8) v += lane_above<8>(v);
+    if (LPR > 4) v += lane_above<4>(v);
+    if (LPR > 2) v += lane_above<2>(v);
+    if (LPR > 1) v += lane_above<1>(v);
     return v;
 }
 
@@ -78,15 +95,57 @@ constexpr int kSysSlots = 8;      // consecutive systems a workgroup accumulates
 constexpr int kLdsAtoms = 4096;   // positions of this many consecutive atoms fit the LDS stage
 constexpr int kBlockFull = 512;   // workgroup size of the full-list kernel
 
-// first/last atom of every non-empty system, from the non-decreasing batch_idx
+// How the images of a system's listed pairs are found.
+struct LjSysImage {
+    int img;         // 0: read the shifts; 1: shift = -rint((r_j - r_i) . H^-1); 2: the same per component (diagonal cell)
+    float hinv[9];   // inverse cell
+    double diag[6];  // diagonal of the cell and of its inverse (img == 2)
+    int pad[2];
+};
+static_assert(sizeof(LjSysImage) == 96, "carved from the workspace 96 bytes a system");
+
+// first/last atom of every non-empty system, from the non-decreasing batch_idx; the thread that
+// finds a system's first atom also decides how the images of its pairs will be found
 __global__ __launch_bounds__(kBlock) void lj_sys_range_kernel(const int32_t* __restrict__ bidx, int n_atoms,
+                                                              const float* __restrict__ cells, double list_rc,
                                                               int32_t* __restrict__ first,
-                                                              int32_t* __restrict__ last) {
+                                                              int32_t* __restrict__ last,
+                                                              LjSysImage* __restrict__ image) {
     int i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n_atoms) return;
     int s = bidx[i];
-    if (i == 0 || bidx[i - 1] != s) first[s] = i;
     if (i == n_atoms - 1 || bidx[i + 1] != s) last[s] = i + 1;
+    if (!(i == 0 || bidx[i - 1] != s)) return;
+    first[s] = i;
+    // shifts need not be read when the list's cutoff is below half of every perpendicular
+    // width of the cell (1 / |column of the inverse|): then no pair has two listed images
+    LjSysImage im;
+    im.img = 0;
+    for (int k = 0; k < 9; ++k) im.hinv[k] = 0.f;
+    for (int k = 0; k < 6; ++k) im.diag[k] = 0.0;
+    im.pad[0] = im.pad[1] = 0;
+    if (cells && list_rc > 0.0) {
+        const float* c = cells + 9 * (size_t)s;
+        double h[9], hv[9];
+        for (int k = 0; k < 9; ++k) h[k] = (double)c[k];
+        inv3(h, hv);  // (a singular cell gives infinities or NaNs: they fail the test below)
+        int ok = 1;
+        const double lim = 1.0 / (2.0002 * list_rc);  // |column| must stay below this
+        for (int k = 0; k < 3; ++k) {
+            const double n2 = hv[k] * hv[k] + hv[3 + k] * hv[3 + k] + hv[6 + k] * hv[6 + k];
+            if (!(n2 < lim * lim)) ok = 0;
+        }
+        for (int k = 0; k < 9; ++k) im.hinv[k] = (float)hv[k];
+        if (ok && h[1] == 0.0 && h[2] == 0.0 && h[3] == 0.0 && h[5] == 0.0 && h[6] == 0.0 && h[7] == 0.0) {
+            ok = 2;
+            for (int k = 0; k < 3; ++k) {
+                im.diag[k] = h[4 * k];
+                im.diag[3 + k] = hv[4 * k];
+            }
+        }
+        im.img = ok;
+    }
+    image[s] = im;
 }
 
 // One pass over the rows [row0, row_end).  LDS_POS: neighbor positions come from the LDS stage
@@ -327,14 +386,12 @@ template <int LPR, bool VIRIAL, bool SHIFTS, bool SYS, bool VEC, bool SWITCH>
 // to write them, so this chain of dependent loads goes through the scalar cache.
 __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_matrix_kernel(
     LjArgs a, const int32_t* __restrict__ bidx_ro, const int32_t* __restrict__ order_ro,
-    const int32_t* __restrict__ first_ro, const int32_t* __restrict__ last_ro, const float* __restrict__ cells_ro) {
+    const int32_t* __restrict__ first_ro, const int32_t* __restrict__ last_ro, const float* __restrict__ cells_ro,
+    const LjSysImage* __restrict__ image_ro) {
     constexpr int NV = VIRIAL ? 7 : 1;
     __shared__ double s_acc[kSysSlots][NV];
     __shared__ float s_pos[3 * kLdsAtoms];
     __shared__ double s_shift[27][3];  // shift . cell of the system in hand, shifts -1..1 per axis
-    __shared__ float s_hinv[9];        // its inverse cell
-    __shared__ double s_diag[6];       // diagonal of the cell and of its inverse
-    __shared__ int s_img;              // its pairs' shifts follow from the positions alone (2: diagonal cell)
 
     // a workgroup owns rows_per_block consecutive rows; workgroups are numbered so that each
     // XCD walks one contiguous eighth of the atoms
@@ -359,45 +416,25 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
         const bool range_ok = span0 <= r && r < span_end;
         const int seg_end = (range_ok && span_end < row_end) ? span_end : row_end;
         const bool staged = range_ok && span_n <= a.lds_atoms;
+        // (what the set-up of a system derives from the thread's number is worked out again for every
+        // system: kept in registers across the rows instead, it is spilled to scratch memory)
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
         if (staged) {
             const float* src = a.pos + 3 * (size_t)span0;
-            for (int t = threadIdx.x; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
+            for (int t = tid; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
         }
-        if (SHIFTS && threadIdx.x < 27) {
-            const int t = threadIdx.x;
+        if (SHIFTS && tid < 27) {
+            const int t = tid;
             shift_vector(cells_ro + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
                          s_shift[t][2]);
         }
-        if (SHIFTS && threadIdx.x == 32) {
-            // shifts need not be read when the list's cutoff is below half of every perpendicular
-            // width of the cell (1 / |column of the inverse|): then no pair has two listed images
-            int ok = 0;
-            if (a.list_rc > 0.0) {
-                const float* c = cells_ro + 9 * (size_t)sys;
-                double h[9], hv[9];
-                for (int k = 0; k < 9; ++k) h[k] = (double)c[k];
-                inv3(h, hv);  // (a singular cell gives infinities or NaNs: they fail the test below)
-                {
-                    ok = 1;
-                    const double lim = 1.0 / (2.0002 * a.list_rc);  // |column| must stay below this
-                    for (int k = 0; k < 3; ++k) {
-                        const double n2 = hv[k] * hv[k] + hv[3 + k] * hv[3 + k] + hv[6 + k] * hv[6 + k];
-                        if (!(n2 < lim * lim)) ok = 0;
-                    }
-                    for (int k = 0; k < 9; ++k) s_hinv[k] = (float)hv[k];
-                    if (ok && h[1] == 0.0 && h[2] == 0.0 && h[3] == 0.0 && h[5] == 0.0 && h[6] == 0.0 && h[7] == 0.0) {
-                        ok = 2;
-                        for (int k = 0; k < 3; ++k) {
-                            s_diag[k] = h[4 * k];
-                            s_diag[3 + k] = hv[4 * k];
-                        }
-                    }
-                }
-            }
-            s_img = ok;
-        }
         __syncthreads();
-        const int img = SHIFTS ? s_img : 0;
+        // (whether this system's shifts follow from the positions alone was decided with its range)
+        const LjSysImage& image = image_ro[sys];
+        const int img = SHIFTS ? image.img : 0;
+        const float* s_hinv = image.hinv;
+        const double* s_diag = image.diag;
 #define NVAMD_LJ_ROWS(STAGED, IMG)                                                                              \
     lj_rows<LPR, VIRIAL, SHIFTS, SYS, STAGED, VEC, (SHIFTS ? IMG : 0), SWITCH>(                                  \
         a, r, seg_end, sys_lo, s_pos, STAGED ? span0 : 0, STAGED ? span_n : 0, s_shift, sys, s_hinv, s_diag, s_acc)
@@ -546,8 +583,8 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
     const bool sw = a.inv_sw > 0.0;
 #define NVAMD_LJ_LAUNCH(V, S, Y, W)                                                                  \
     {                                                                                                \
-        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true, W>), grid, blk, 0, st, b, b.bidx, b.order, b.sys_first, b.sys_last, b.cells); \
-        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false, W>), grid, blk, 0, st, b, b.bidx, b.order, b.sys_first, b.sys_last, b.cells);    \
+        if (vec) hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, true, W>), grid, blk, 0, st, b, b.bidx, b.order, b.sys_first, b.sys_last, b.cells, b.sys_image); \
+        else hipLaunchKernelGGL((lj_matrix_kernel<LPR, V, S, Y, false, W>), grid, blk, 0, st, b, b.bidx, b.order, b.sys_first, b.sys_last, b.cells, b.sys_image);    \
         return;                                                                                      \
     }
 #define NVAMD_LJ_CASE(V, S, Y)                                                                 \
@@ -581,6 +618,7 @@ NVAMD_EXPORT int32_t nvamd_lj_workspace_bytes(int32_t n_atoms, int32_t n_systems
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj workspace: bad argument");
     size_t b = align_up((size_t)(n_systems > 0 ? n_systems : 1) * 10 * sizeof(double));
     b += 2 * align_up((size_t)(n_systems > 0 ? n_systems : 1) * sizeof(int32_t));
+    b += align_up((size_t)(n_systems > 0 ? n_systems : 1) * sizeof(LjSysImage));
     if (half_list) b += align_up((size_t)(n_atoms > 0 ? n_atoms : 1) * 4 * sizeof(double));
     *bytes = b;
     return NVAMD_OK;
@@ -651,6 +689,7 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
     a.order = half_list ? nullptr : row_order;  // (the half-list kernel walks rows in index order)
     a.sys_first = nullptr;
     a.sys_last = nullptr;
+    a.sys_image = nullptr;
     a.lds_atoms = kLdsAtoms;
     a.r_on = switch_width > 0.0 ? cutoff - switch_width : 0.0;
     a.inv_sw = switch_width > 0.0 ? 1.0 / switch_width : 0.0;
@@ -665,7 +704,10 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
     int32_t* sys_first = reinterpret_cast<int32_t*>(w + align_up(nsys * 10 * sizeof(double)));
     int32_t* sys_last = reinterpret_cast<int32_t*>(w + align_up(nsys * 10 * sizeof(double)) +
                                                    align_up(nsys * sizeof(int32_t)));
-    char* w_half = w + align_up(nsys * 10 * sizeof(double)) + 2 * align_up(nsys * sizeof(int32_t));
+    LjSysImage* sys_image = reinterpret_cast<LjSysImage*>(w + align_up(nsys * 10 * sizeof(double)) +
+                                                          2 * align_up(nsys * sizeof(int32_t)));
+    char* w_half = w + align_up(nsys * 10 * sizeof(double)) + 2 * align_up(nsys * sizeof(int32_t)) +
+                   align_up(nsys * sizeof(LjSysImage));
     if (want_sys && n_systems > 0) {
         a.sys_acc = reinterpret_cast<double*>(w);
         size_t n = (size_t)n_systems * 10;
@@ -692,9 +734,10 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
             const bool vir = virials != nullptr;
             const bool sys = a.sys_acc != nullptr;
             hipLaunchKernelGGL(lj_sys_range_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
-                               batch_idx, n_atoms, sys_first, sys_last);
+                               batch_idx, n_atoms, shifts ? cells : nullptr, a.list_rc, sys_first, sys_last, sys_image);
             a.sys_first = sys_first;
             a.sys_last = sys_last;
+            a.sys_image = sys_image;
             switch (lanes_per_row(max_neighbors)) {
                 case 8: launch_full<8>(a, vir, shifts, sys, st); break;
                 case 16: launch_full<16>(a, vir, shifts, sys, st); break;
