@@ -1,8 +1,12 @@
 """Throughput of the batched MD inner loop on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--boxes B] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {2,3,4,5}] [--boxes B] [--no-cpu-baseline]
 
-Workload (the configuration the metric is quoted on): 256 periodic cubic Lennard-Jones
+Other configurations of the baseline (``--config``): 2 = 64 FCC boxes of 500 atoms, NVE; 4 = 2048
+triclinic cells of 8-2000 atoms, FIRE with per-system convergence masks; 5 = one box of 4 M atoms,
+NVE.  They print the same line (without the CPU baseline, which is timed on the quoted workload only).
+
+Workload (the configuration the metric is quoted on, ``--config 3``, the default): 256 periodic cubic Lennard-Jones
 liquid boxes of 3900 atoms (998 400 atoms), reduced units, density 0.8 sigma^-3, uniform
 random positions (seed 0) relaxed by 50 FIRE steps (dt 0.005, maxstep 0.07 sigma), then NVE velocity Verlet with dt = 0.005,
 cutoff 2.5 sigma, the neighbor list rebuilt on every step.  One step is one pass of the hot
@@ -52,21 +56,83 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_liquid_batch(n_boxes: int, n_per_box: int, density: float, seed: int, device):
+def _batch_of(systems, device):
+    """systems: list of (positions (n,3) float32 tensor, cell (3,3) tensor); argon-like atoms of unit mass."""
     import torch
 
     from nvalchemi_amd.data import AtomicData, Batch
 
+    data = []
+    for pos, cell in systems:
+        n = pos.shape[0]
+        data.append(AtomicData(pos, torch.full((n,), 18, dtype=torch.long), atomic_masses=torch.ones(n), cell=cell,
+                               pbc=torch.tensor([True, True, True]), forces=torch.zeros(n, 3),
+                               energy=torch.zeros(1, 1)))
+    return Batch.from_data_list(data, device=device)
+
+
+def make_liquid_batch(n_boxes: int, n_per_box: int, density: float, seed: int, device):
+    import torch
+
     L = (n_per_box / density) ** (1.0 / 3.0)
     g = torch.Generator().manual_seed(seed)
-    data = []
-    for _ in range(n_boxes):
-        pos = torch.rand(n_per_box, 3, generator=g) * L
-        data.append(AtomicData(pos, torch.full((n_per_box,), 18, dtype=torch.long),
-                               atomic_masses=torch.ones(n_per_box), cell=torch.eye(3) * L,
-                               pbc=torch.tensor([True, True, True]), forces=torch.zeros(n_per_box, 3),
-                               energy=torch.zeros(1, 1)))
-    return Batch.from_data_list(data, device=device), L
+    systems = [(torch.rand(n_per_box, 3, generator=g) * L, torch.eye(3) * L) for _ in range(n_boxes)]
+    return _batch_of(systems, device), L
+
+
+def make_fcc_batch(device, n_boxes=64, reps=5, a=3.6, jitter=0.05, seed=0):
+    """BASELINE configuration 2: cubic FCC boxes of 4 reps^3 atoms with Gaussian jitter."""
+    import numpy as np
+    import torch
+
+    rng = np.random.default_rng(seed)
+    base = np.array([[0, 0, 0], [0.5, 0.5, 0], [0.5, 0, 0.5], [0, 0.5, 0.5]])
+    g = np.stack(np.meshgrid(*[np.arange(reps)] * 3, indexing="ij"), -1).reshape(-1, 1, 3)
+    lat = ((g + base[None]) * a).reshape(-1, 3)
+    cell = torch.eye(3) * (reps * a)
+    systems = [(torch.from_numpy((lat + rng.normal(0, jitter, lat.shape)).astype(np.float32)), cell)
+               for _ in range(n_boxes)]
+    return _batch_of(systems, device)
+
+
+def _triclinic_cell(rng, length):
+    """Lattice vectors of length 0.8-1.2 x ``length`` with angles uniform in 60-120 degrees."""
+    import numpy as np
+
+    while True:
+        al, be, ga = np.deg2rad(rng.uniform(60.0, 120.0, 3))
+        la, lb, lc = length * rng.uniform(0.8, 1.2, 3)
+        cx = lc * np.cos(be)
+        cy = lc * (np.cos(al) - np.cos(be) * np.cos(ga)) / np.sin(ga)
+        cz2 = lc * lc - cx * cx - cy * cy
+        if cz2 <= (0.3 * lc) ** 2:
+            continue
+        return np.array([[la, 0, 0], [lb * np.cos(ga), lb * np.sin(ga), 0], [cx, cy, np.sqrt(cz2)]])
+
+
+def make_inflight_mix(device, n_systems=2048, n_lo=8, n_hi=2000, density=0.0764, seed=0):
+    """BASELINE configuration 4: triclinic cells of 8-2000 atoms (log-uniform), about 40 neighbors per
+    atom inside 5 Angstrom, uniform random positions."""
+    import numpy as np
+    import torch
+
+    rng = np.random.default_rng(seed)
+    counts = np.exp(rng.uniform(np.log(n_lo), np.log(n_hi), n_systems)).astype(np.int64)
+    systems = []
+    for n in counts:
+        H = _triclinic_cell(rng, (n / density) ** (1.0 / 3.0))
+        pos = rng.uniform(0, 1, (n, 3)) @ H
+        systems.append((torch.from_numpy(pos.astype(np.float32)), torch.from_numpy(H.astype(np.float32))))
+    return _batch_of(systems, device)
+
+
+def make_single_box(device, n_atoms=4_000_000, density=0.1, seed=0):
+    """BASELINE configuration 5: one periodic cubic box, uniform random positions."""
+    import torch
+
+    L = (n_atoms / density) ** (1.0 / 3.0)
+    g = torch.Generator().manual_seed(seed)
+    return _batch_of([(torch.rand(n_atoms, 3, generator=g) * L, torch.eye(3) * L)], device)
 
 
 class StageTimer:
@@ -74,7 +140,7 @@ class StageTimer:
     velocity-Verlet halves), recorded on the stream the kernels are enqueued on."""
 
     ENTRY = {"nl": "nl_build", "lj": "lj_energy_forces", "vv_pre": "vv_position_update",
-             "vv_post": "vv_velocity_finalize"}
+             "vv_post": "vv_velocity_finalize", "fire": "fire_step", "fmax": "segment_fmax"}
 
     def __init__(self):
         import torch
@@ -136,51 +202,109 @@ def cpu_baseline(pos, cell, pbc, n_per_box, n_boxes_sample, K, steps):
     return out, n
 
 
+# fp64 operations of one pair on the shifts-derived path of the pair kernel, multiply-adds counted twice:
+# r_j - r_i (3), nearest image per component (mul, rint, fma: 12), r^2 (5), reciprocal (estimate + two
+# Newton steps: 9), (s/r)^2, ^6, ^12 (4), u (2), u'/r (4), energy sum (2), force sums (6)
+LJ_FP64_FLOPS_PER_PAIR = 47
+FP64_PEAK_TFLOPS = 78.6  # MI355X vector fp64, published
+
+
+def setup_config(cfg: int, args, device):
+    """Batch, model and dynamics of a BASELINE configuration; returns (batch, dyn, description, warm)."""
+    import torch
+
+    from nvalchemi_amd.dynamics import FIRE, NVE, ConvergenceHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    fs = 10.180505710759414  # NVE takes femtoseconds; one internal time unit of the eV / Angstrom / amu system
+    if cfg == 3:
+        n_per_box, density, rc, dt = 3900, 0.8, 2.5, 0.005
+        batch, L = make_liquid_batch(args.boxes, n_per_box, density, 0, device)
+        model = LennardJonesModelWrapper(epsilon=1.0, sigma=1.0, cutoff=rc)
+        t0 = time.perf_counter()
+        relax = FIRE(model, dt=dt, maxstep=RELAX_MAXSTEP, hooks=model.make_neighbor_hooks())
+        relax.run(batch, n_steps=args.relax_steps)
+        torch.cuda.synchronize()
+        log(f"[bench] L={L:.3f}; {args.relax_steps} FIRE steps in {time.perf_counter() - t0:.2f}s; "
+            f"E/atom={float(batch.energy.sum()) / batch.num_nodes:.3f} fmax={float(batch.forces.norm(dim=1).max()):.3e}")
+        batch.velocities.zero_()
+        if args.skin > 0.0:
+            model.model_config.neighbor_config.skin = args.skin
+        dyn = NVE(model, dt=dt * fs, hooks=model.make_neighbor_hooks())
+        what = (f"{batch.num_graphs} periodic LJ-liquid boxes x {n_per_box} atoms, rho=0.8, rc=2.5 sigma, "
+                f"{args.relax_steps} FIRE steps then NVE dt=0.005, "
+                + ("neighbor rebuild every step" if args.skin <= 0.0 else
+                   f"Verlet skin {args.skin} sigma (rebuild when an atom has moved skin/2)"))
+        return batch, dyn, what
+    if cfg == 2:
+        batch = make_fcc_batch(device)
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=2.268, cutoff=6.0)  # pair minimum at the FCC spacing
+        dyn = NVE(model, dt=0.5, hooks=model.make_neighbor_hooks())
+        return batch, dyn, ("64 periodic cubic boxes x 500 atoms (FCC a=3.6 A + N(0, 0.05 A) jitter), cutoff 6 A, LJ, "
+                            "NVE velocity Verlet dt=0.5 fs, neighbor rebuild every step")
+    if cfg == 4:
+        batch = make_inflight_mix(device)
+        batch.status = torch.zeros(batch.num_graphs, 1, dtype=torch.long, device=device)
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=2.5, cutoff=5.0)
+        hook = ConvergenceHook.from_fmax(0.05, source_status=0, target_status=1)
+        dyn = FIRE(model, dt=0.02, maxstep=0.1, hooks=model.make_neighbor_hooks() + [hook])
+        return batch, dyn, ("2048 periodic triclinic cells of 8-2000 atoms (log-uniform, angles 60-120 deg, uniform random "
+                            "positions, ~40 neighbors/atom), cutoff 5 A, LJ, FIRE with a per-system fmax criterion that "
+                            "freezes converged systems, neighbor rebuild every step")
+    if cfg == 5:
+        batch = make_single_box(device)
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=1.5, cutoff=6.0)
+        # (a random gas has pairs far up the repulsive wall: a few FIRE steps with a short leash take them
+        # off it, so that the timed dynamics stays finite)
+        t0 = time.perf_counter()
+        FIRE(model, dt=0.02, maxstep=0.05, hooks=model.make_neighbor_hooks()).run(batch, n_steps=args.relax_steps)
+        torch.cuda.synchronize()
+        log(f"[bench] {args.relax_steps} FIRE steps in {time.perf_counter() - t0:.2f}s; "
+            f"E/atom={float(batch.energy.sum()) / batch.num_nodes:.3e} fmax={float(batch.forces.norm(dim=1).max()):.3e}")
+        batch.velocities.zero_()
+        dyn = NVE(model, dt=0.05, hooks=model.make_neighbor_hooks())
+        return batch, dyn, ("one periodic cubic box of 4,000,000 atoms, density 0.1 /A^3 (uniform random positions, "
+                            f"{args.relax_steps} FIRE steps), cutoff 6 A (~90 neighbors/atom), LJ with fp64 per-system "
+                            "energy, NVE velocity Verlet dt=0.05 fs, neighbor rebuild every step")
+    raise ValueError(f"unknown configuration {cfg}")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--boxes", type=int, default=256, help="number of 3900-atom boxes (256 = the quoted workload)")
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--config", type=int, default=3, choices=(2, 3, 4, 5),
+                    help="BASELINE configuration (3 = the 1M-atom liquid the metric is quoted on)")
+    ap.add_argument("--boxes", type=int, default=256, help="configuration 3: number of 3900-atom boxes (256 = the quoted workload)")
     ap.add_argument("--relax-steps", type=int, default=50)
     ap.add_argument("--skin", type=float, default=0.0,
-                    help="Verlet skin of the neighbor hook (0 = rebuild every step, the quoted workload)")
+                    help="configuration 3: Verlet skin of the neighbor hook (0 = rebuild every step, the quoted workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-stage-events", action="store_true", help="do not record per-stage HIP events")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         return 2
+    if args.steps is None:
+        args.steps = 30 if args.config == 5 else 200
+    if args.warmup is None:
+        args.warmup = 5 if args.config == 5 else 20
 
     import numpy as np
     import torch
 
     from nvalchemi_amd import _lib
-    from nvalchemi_amd.dynamics import FIRE, NVE
-    from nvalchemi_amd.models import LennardJonesModelWrapper
 
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm device", file=sys.stderr)
         return 2
     _lib.library()  # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
-    n_per_box, density, rc, dt = 3900, 0.8, 2.5, 0.005
-    batch, L = make_liquid_batch(args.boxes, n_per_box, density, 0, dev)
+    batch, dyn, what = setup_config(args.config, args, dev)
     N, B = batch.num_nodes, batch.num_graphs
-    model = LennardJonesModelWrapper(epsilon=1.0, sigma=1.0, cutoff=rc)
+    log(f"[bench] configuration {args.config}: N={N} B={B}")
 
-    t0 = time.perf_counter()
-    relax = FIRE(model, dt=dt, maxstep=RELAX_MAXSTEP, hooks=model.make_neighbor_hooks())
-    relax.run(batch, n_steps=args.relax_steps)
-    torch.cuda.synchronize()
-    log(f"[bench] N={N} B={B} L={L:.3f}; {args.relax_steps} FIRE steps in {time.perf_counter() - t0:.2f}s; "
-        f"E/atom={float(batch.energy.sum()) / N:.3f} fmax={float(batch.forces.norm(dim=1).max()):.3e}")
-    batch.velocities.zero_()
-
-    if args.skin > 0.0:
-        model.model_config.neighbor_config.skin = args.skin
-    hooks = model.make_neighbor_hooks()
-    dyn = NVE(model, dt=dt * 10.180505710759414, hooks=hooks)  # NVE takes fs; 0.005 internal units
     timer = None if args.no_stage_events else StageTimer()
     for _ in range(args.warmup):
         dyn.step(batch)
@@ -205,26 +329,40 @@ def main() -> int:
 
     ms_per_step = wall / args.steps * 1e3
     value = N * args.steps / wall
+    quoted = args.config == 3 and B == 256 and args.relax_steps == 50 and args.skin <= 0.0
     stages = {}
     if timer:
         ms = timer.mean_ms()
         # Algorithmic bytes are the compulsory traffic at the API's own I/O layout: a pair is its
         # 4-byte index and its 12-byte shift.  The pair kernel derives shifts from positions in
-        # cells wider than twice the search radius (this workload's are) and then does not read
-        # them: the bytes it still has to touch are reported beside the API-level figure.
+        # cells wider than twice the search radius and then does not read them; it is then bound
+        # by its double-precision arithmetic, and both figures are given.
         stamp = getattr(batch, "_neighbor_search_cutoff", None)
         widths = 1.0 / torch.linalg.inv(batch.cell.double()).norm(dim=1)
         shifts_derived = bool(stamp) and bool((widths > 2.0002 * stamp[0]).all())
-        alg = {"nl": 20 * N + 16 * E, "lj": 36 * N + 16 * E + 4 * B, "vv_pre": 68 * N, "vv_post": 44 * N}
+        alg = {"nl": 20 * N + 16 * E, "lj": 36 * N + 16 * E + 4 * B, "vv_pre": 68 * N, "vv_post": 44 * N,
+               "fire": 96 * N, "fmax": 12 * N + 4 * B}
         for k, b in alg.items():
+            if not (ms[k] == ms[k]):  # an entry point this configuration never calls
+                continue
             gbps = b / (ms[k] * 1e-3) / 1e9
             stages[k] = {"ms": round(ms[k], 4), "alg_bytes": b, "GBps": round(gbps, 1),
                          "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+        lj = stages["lj"]
+        tflops = LJ_FP64_FLOPS_PER_PAIR * E / (ms["lj"] * 1e-3) / 1e12
+        lj["fp64_flops_per_pair"] = LJ_FP64_FLOPS_PER_PAIR
+        lj["fp64_TFLOPs"] = round(tflops, 2)
+        lj["fp64_frac"] = round(tflops / FP64_PEAK_TFLOPS, 4)
         if shifts_derived:
+            # the API-level figure counts 12 bytes of shifts per pair that this path never reads: the
+            # fraction of the HBM peak that stands for this stage is that of the bytes it must touch
             touched = 36 * N + 4 * E + 4 * B
-            stages["lj"]["shifts_derived_not_read"] = True
-            stages["lj"]["bytes_it_must_touch"] = touched
-            stages["lj"]["GBps_touched"] = round(touched / (ms["lj"] * 1e-3) / 1e9, 1)
+            lj["shifts_derived_not_read"] = True
+            lj["api_alg_bytes"], lj["api_GBps"], lj["api_frac"] = lj["alg_bytes"], lj["GBps"], lj["frac"]
+            lj["alg_bytes"] = touched
+            lj["GBps"] = round(touched / (ms["lj"] * 1e-3) / 1e9, 1)
+            lj["frac"] = round(lj["GBps"] / HBM_PEAK_GBPS, 4)
+            lj["bound"] = "fp64 vector arithmetic"
         log("[bench] stage ms: " + ", ".join(f"{k}={v['ms']}" for k, v in stages.items())
             + f"; sum={sum(v['ms'] for v in stages.values()):.3f} vs wall/step={ms_per_step:.3f}")
     result = {
@@ -240,10 +378,7 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"{B} periodic LJ-liquid boxes x {n_per_box} atoms, rho=0.8, rc=2.5 sigma, "
-                               f"{args.relax_steps} FIRE steps then NVE dt=0.005, "
-                               + ("neighbor rebuild every step" if args.skin <= 0.0 else
-                                  f"Verlet skin {args.skin} sigma (rebuild when an atom has moved skin/2)"),
+        "config": {"workload": what, "baseline_config": args.config,
                    "n_atoms": N, "n_systems": B, "edges": E, "max_neighbors": K, "seed": 0},
         "edges_per_s": (E / (stages["nl"]["ms"] * 1e-3)) if stages else None,
     }
@@ -251,12 +386,15 @@ def main() -> int:
         nl = stages["nl"]
         result["roofline"] = {"bound": "hbm", "achieved": nl["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                               "frac": nl["frac"],
-                              "traffic": MEASURED_TRAFFIC_BYTES["nl"] if (B == 256 and args.relax_steps == 50 and args.skin <= 0.0) else None,
+                              "traffic": MEASURED_TRAFFIC_BYTES["nl"] if quoted else None,
+                              "traffic_source": ("profiles/hbm_traffic_lj_liquid_1M.txt: rocprofv3 --pmc FETCH_SIZE and "
+                                                 "WRITE_SIZE runs of this command, not measured in this run") if quoted else None,
                               "kernel": "neighbor build (nvamd_nl_build)",
                               "alg_bytes_per_launch": nl["alg_bytes"], "ms_per_launch": nl["ms"]}
         result["stages"] = stages
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.config == 3:
         # about ten seconds of host work: 32 boxes, 20 steps on one thread, then on the box's share of cores
+        n_per_box = 3900
         sample_boxes, cpu_steps = min(B, 32), 20
         cb, n_s = cpu_baseline(batch.positions.cpu().numpy(), batch.cell.cpu().numpy(), batch.pbc.cpu().numpy(),
                                n_per_box, sample_boxes, K, steps=cpu_steps)
