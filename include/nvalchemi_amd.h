@@ -288,6 +288,21 @@ int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells
                                       float* atomic_energies, float* forces, float* virials,
                                       float* system_energies, void* stream);
 
+/* What the neighbor builds through this workspace had to report.  No counterpart in the reference, whose
+ * kernels report nothing (a caller there compares num_neighbors with max_neighbors on the host:
+ * nvalchemi/neighbors.py:269-273, nvalchemi/hooks/neighbor_list.py:446-469).
+ * status (2) i32 on the device: status[0] = bits of the last build, status[1] = bits of every build since the
+ *   bits were last cleared (the header of a workspace that has never held a build must be zero for status[1]
+ *   to mean anything).  clear != 0 clears both words after they are read.  No host synchronisation.
+ * NVAMD_NL_STATUS_CELL_TOO_THIN: some periodic cell is singular or thinner than cutoff / 32 along an axis; the
+ *   search looks at 32 images per axis and direction at most, so that system's list is truncated.
+ * NVAMD_NL_STATUS_ROW_OVERFLOW: some atom has more than max_neighbors neighbors (its count says how many; the
+ *   row holds the first max_neighbors found). */
+#define NVAMD_NL_STATUS_CELL_TOO_THIN 1
+#define NVAMD_NL_STATUS_ROW_OVERFLOW 2
+int32_t nvamd_nl_status(void* workspace, size_t workspace_bytes, int32_t n_atoms, int32_t n_systems,
+                        int32_t* status, int32_t clear, void* stream);
+
 /* Atom indices in the cell order of the neighbor build that last used this workspace with the same
  * n_atoms / n_systems: atom_order[k] for k in a system's range [batch_ptr[s], batch_ptr[s+1]) are that
  * system's atoms, cell by cell.  With rebuild_flags, only the ranges of flagged systems are written

@@ -93,9 +93,10 @@ static_assert(kMaxStencilRadius < 64, "stencil radii are packed 6 bits each");
 
 struct NlHeader {
     int total_cells;
-    int error;  // bit 0: a system's cell is degenerate or narrower than cutoff/kMaxStencilRadius
+    int error;   // of the build in hand: NVAMD_NL_STATUS_* bits
     int total_units;
-    int pad[13];
+    int sticky;  // the bits of all earlier builds through this workspace since they were last cleared
+    int pad[12];
 };
 
 struct NlWorkspace {
@@ -206,7 +207,10 @@ __device__ __forceinline__ void system_setup(NlSys& s, const NlArgs& a, int t) {
 __global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspace ws) {
     int t = blockIdx.x * kBlock + threadIdx.x;
     if (t < ws.max_cells) ws.cell_count[t] = 0;
-    if (t == 0) ws.hdr->error = 0;
+    if (t == 0) {
+        ws.hdr->sticky |= ws.hdr->error;
+        ws.hdr->error = 0;
+    }
     if (t >= a.n_systems) return;
     NlSys s;
     system_setup(s, a, t);
@@ -274,7 +278,7 @@ __device__ __forceinline__ void choose_grid(NlSys& s, const NlArgs& a, const uin
             if (r >= 1.0 && r <= (double)kMaxStencilRadius) R = (int)r;
             else {
                 R = (r > (double)kMaxStencilRadius) ? kMaxStencilRadius : 1;
-                if (n_at > 0) atomicOr(error_flag, 1);
+                if (n_at > 0) atomicOr(error_flag, NVAMD_NL_STATUS_CELL_TOO_THIN);
             }
             if (!s.per[d] && R > s.nc[d] - 1) R = s.nc[d] - 1;
         }
@@ -704,6 +708,7 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
 __global__ void nl_reset_kernel(NlWorkspace ws) {
     ws.hdr->total_units = 0;
     ws.hdr->total_cells = 0;  // not used on the per-system path: cell ids are not dense
+    ws.hdr->sticky |= ws.hdr->error;
     ws.hdr->error = 0;
 }
 
@@ -1126,7 +1131,10 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                     srow[3 * k + 2] = 0;
                                 }
                             }
-                            if (lane == 0) a.nn[i_atom] = base;
+                            if (lane == 0) {
+                                a.nn[i_atom] = base;
+                                if (base > a.K) atomicOr(&ws.hdr->error, NVAMD_NL_STATUS_ROW_OVERFLOW);
+                            }
                         } else if (lane == 0) {
                             ca_meta[ca].w = base;
                         }
@@ -1152,11 +1160,24 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             srow[3 * k + 2] = 0;
                         }
                     }
-                    if (lane == 0) a.nn[i_atom] = cnt;
+                    if (lane == 0) {
+                        a.nn[i_atom] = cnt;
+                        if (cnt > a.K) atomicOr(&ws.hdr->error, NVAMD_NL_STATUS_ROW_OVERFLOW);
+                    }
                 }
             }
             __syncthreads();
         }
+    }
+}
+
+__global__ void nl_status_kernel(NlHeader* hdr, int32_t* out, int clear) {
+    const int now = hdr->error, all = hdr->sticky | now;
+    out[0] = now;
+    out[1] = all;
+    if (clear) {
+        hdr->sticky = 0;
+        hdr->error = 0;
     }
 }
 
@@ -1190,6 +1211,20 @@ NVAMD_EXPORT int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace
     hipLaunchKernelGGL(nl_atom_order_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0,
                        static_cast<hipStream_t>(stream), ws.sorted_pos, batch_idx, rebuild_flags, n_atoms, atom_order);
     NVAMD_LAUNCH_CHECK("atom order launch");
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_status(void* workspace, size_t workspace_bytes, int32_t n_atoms, int32_t n_systems,
+                                     int32_t* status, int32_t clear, void* stream) {
+    if (n_atoms < 0 || n_systems < 0 || !status) return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl status: bad argument");
+    size_t need = carve(nullptr, nullptr, n_atoms, n_systems);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "nl status: workspace %zu < %zu bytes", workspace_bytes, need);
+    NlWorkspace ws;
+    carve(&ws, static_cast<char*>(workspace), n_atoms, n_systems);
+    hipLaunchKernelGGL(nl_status_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), ws.hdr, status,
+                       clear ? 1 : 0);
+    NVAMD_LAUNCH_CHECK("nl status launch");
     return NVAMD_OK;
 }
 

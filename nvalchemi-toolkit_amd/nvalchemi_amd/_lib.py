@@ -28,6 +28,7 @@ _SIGNATURES = {
     "nvamd_abi_version": (_i32, []),
     "nvamd_last_error": (_c.c_char_p, []),
     "nvamd_nl_workspace_bytes": (_i32, [_i32, _i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_nl_status": (_i32, [_vp, _c.c_size_t, _i32, _i32, _vp, _i32, _vp]),
     "nvamd_nl_build": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32,
                               _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_build_path": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32, _i32,
@@ -151,6 +152,7 @@ class _Workspaces:
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+            buf[:256].zero_()  # (the neighbor build keeps status bits in its workspace's header from build to build)
             self._bufs[key] = buf
         return buf
 
@@ -203,6 +205,24 @@ def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, 
                                    int(bool(half_fill)), int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
                                    ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)),
            "nvamd_nl_build")
+
+
+NL_STATUS_CELL_TOO_THIN = 1
+NL_STATUS_ROW_OVERFLOW = 2
+
+
+def nl_status(n_atoms: int, n_systems: int, device, clear: bool = False,
+              workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """``(2,)`` int32 on the device: status bits of the last neighbor build through the workspace of
+    this device and stream, and the bits of all builds since they were last cleared.  No host
+    synchronisation here; reading the tensor on the host is one."""
+    lib = library()
+    need = nl_workspace_bytes(n_atoms, n_systems)
+    ws = workspace if workspace is not None else workspaces.get(torch.device(device), "nl", need)
+    out = torch.empty(2, dtype=torch.int32, device=device)
+    _check(lib.nvamd_nl_status(ws.data_ptr(), ws.numel() * ws.element_size(), int(n_atoms), int(n_systems),
+                               out.data_ptr(), int(bool(clear)), _stream(torch.device(device))), "nvamd_nl_status")
+    return out
 
 
 def nl_edge_ptr(num_neighbors, max_neighbors, edge_ptr) -> None:

@@ -29,7 +29,7 @@ from .. import _lib
 from .._neighbor_ops import ceil16, estimate_max_neighbors, neighbor_list
 from ..dynamics._ops.neighbor_list_rebuild import batch_neighbor_list_rebuild_inplace
 from ..models.base import NeighborConfig, NeighborListFormat
-from ..neighbors import _write_neighbor_data_to_batch
+from ..neighbors import _raise_on_truncated_search, _write_neighbor_data_to_batch
 from ._context import HookContext
 
 
@@ -125,6 +125,7 @@ class NeighborListHook:
         if self._first_build:
             # the one host synchronisation: validate K against the actual maximum
             self._first_build = False
+            _raise_on_truncated_search(N, B, positions.device, cutoff)
             self._actual_max_k = self._num_neighbors.max() if N > 0 else None
             if self._check_and_resize_k(N, positions.device, pbc):
                 self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
@@ -140,6 +141,15 @@ class NeighborListHook:
             neighbor_matrix_shifts=self._neighbor_matrix_shifts,
             format=NeighborListFormat.COO if self._neighbor_list_flag else NeighborListFormat.MATRIX,
             cutoff=self.config.cutoff, search_cutoff=None if self.config.half_list else cutoff)
+
+    def overflowed(self, clear: bool = True) -> bool:
+        """Whether any build since the last call left an atom with more neighbors than the rows hold
+        (the reference never notices this after its first build, nvalchemi/hooks/neighbor_list.py:351-355;
+        the kernels here count past K on the device and keep a flag).  One host synchronisation."""
+        if self._neighbor_matrix is None or self._alloc_N in (None, 0):
+            return False
+        st = _lib.nl_status(self._alloc_N, self._alloc_B, self._neighbor_matrix.device, clear=clear)
+        return bool(int(st[1]) & _lib.NL_STATUS_ROW_OVERFLOW)
 
     #: systems larger than this do not fit the pair kernel's LDS stage (csrc/lj_pair.hip kLdsAtoms)
     _ROW_ORDER_MIN_ATOMS = 4096

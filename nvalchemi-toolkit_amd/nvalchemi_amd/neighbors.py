@@ -18,6 +18,20 @@ from .models.base import NeighborConfig, NeighborListFormat
 __all__ = ["compute_neighbors"]
 
 
+def _raise_on_truncated_search(n_atoms: int, n_systems: int, device, cutoff: float) -> None:
+    """The search looks at 32 periodic images per axis and direction at most: a cell that is singular
+    or thinner than cutoff / 32 gives a truncated list, which the build reports in its status bits.
+    Called where the host waits for the device anyway."""
+    if n_atoms == 0:
+        return
+    from . import _lib
+
+    now = int(_lib.nl_status(n_atoms, n_systems, device)[0])
+    if now & _lib.NL_STATUS_CELL_TOO_THIN:
+        raise ValueError(f"a periodic cell is singular or thinner than cutoff / 32 (cutoff {cutoff}): "
+                         "its neighbor list would be truncated")
+
+
 def _write_neighbor_data_to_batch(batch: Batch, neighbor_matrix: torch.Tensor, num_neighbors: torch.Tensor,
                                   neighbor_matrix_shifts: torch.Tensor | None,
                                   format: NeighborListFormat, cutoff: float,
@@ -111,6 +125,7 @@ def compute_neighbors(batch: Batch, cutoff: float | None = None, *, config: Neig
         if actual_max < max_neighbors:
             break
         max_neighbors = int(actual_max * 1.5) + 1
+    _raise_on_truncated_search(N, batch.num_graphs, device, cutoff)
 
     _write_neighbor_data_to_batch(batch, nb_matrix, nb_counts, nb_shifts, format, cutoff,
                                   search_cutoff=None if half_list else cutoff)

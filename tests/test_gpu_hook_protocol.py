@@ -139,3 +139,49 @@ def test_shrinking_neighbors_leave_no_stale_coo_edges():
     assert (0, 1) not in after and (1, 0) not in after and (1, 2) in after and (2, 1) in after
     counts = torch.bincount(b.neighbor_list[:, 0].cpu().long(), minlength=b.num_nodes)
     assert torch.equal(counts, h._num_neighbors.cpu().long())
+
+
+def test_a_cell_too_thin_for_the_search_is_refused_not_truncated():
+    """The search looks at 32 periodic images per axis and direction at most.  A cell thinner than
+    cutoff / 32 used to give a truncated list with an OK status; the build now reports it in its
+    status bits, and the callers that wait for the device anyway raise."""
+    from nvalchemi_amd import _lib
+    from nvalchemi_amd.data import AtomicData, Batch
+    from nvalchemi_amd.neighbors import compute_neighbors
+
+    thin = Batch.from_data_list([AtomicData(torch.tensor([[0.0, 0, 0], [0.01, 0.5, 0.5]]), torch.tensor([1, 1]),
+                                            cell=torch.diag(torch.tensor([0.05, 4.0, 4.0])),
+                                            pbc=torch.tensor([True, True, True]))], device=DEV)
+    with pytest.raises(ValueError, match="thinner than cutoff / 32"):
+        compute_neighbors(thin, cutoff=2.0)
+    with pytest.raises(ValueError, match="thinner than cutoff / 32"):
+        hook(config=cfg(cutoff=2.0))(ctx(thin), stage())
+    # a cell of ordinary proportions clears the bit of the last build; the accumulated bits keep it until read
+    ok = line_batch(pbc=True)
+    compute_neighbors(ok, cutoff=2.5)
+    st = _lib.nl_status(ok.num_nodes, ok.num_graphs, ok.positions.device).tolist()
+    assert st[0] == 0
+
+
+def test_rows_that_overflow_after_the_first_build_leave_a_flag():
+    """After its first build the reference's hook never compares counts with K again
+    (nvalchemi/hooks/neighbor_list.py:351-355).  The kernels count past K on the device and leave a
+    bit in the workspace; ``overflowed()`` reads it."""
+    from nvalchemi_amd.data import AtomicData, Batch
+
+    g = torch.Generator().manual_seed(3)
+    pos = torch.rand(64, 3, generator=g) * 6.0
+    b = Batch.from_data_list([AtomicData(pos, torch.ones(64, dtype=torch.long), cell=torch.eye(3) * 6.0,
+                                         pbc=torch.tensor([True, True, True]))], device=DEV)
+    h = hook(config=cfg(cutoff=2.5))
+    h(ctx(b), stage())
+    assert not h.overflowed()
+    K = h._max_neighbors
+    # squeeze every atom into a corner of the cell: every row now wants 63 neighbors or more
+    b.positions.mul_(0.05)
+    h(ctx(b), stage())
+    if int(h._num_neighbors.max()) > K:
+        assert h.overflowed()
+        assert not h.overflowed()  # (read and cleared)
+    h(ctx(b), stage())
+    assert h.overflowed() == (int(h._num_neighbors.max()) > K)
