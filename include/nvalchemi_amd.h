@@ -288,6 +288,47 @@ int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells
                                       float* atomic_energies, float* forces, float* virials,
                                       float* system_energies, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * float64 forms.  The reference's ops take float32 or float64 arrays (nvalchemi/dynamics/_ops/_bridge.py
+ * _vec_type / _scalar_type; nvalchemi/dynamics/_ops/fire.py:281-287; nvalchemi/models/_ops/lj.py:116-216).
+ * Same arguments, meaning and order of operations as the float32 entry points above, with every float
+ * array a double array (cells included; per-system parameters too).  The neighbor decision is made in
+ * double on the float64 positions.  The pair kernel's per-system energy is the sum of the float64 atomic
+ * energies.  nvamd_f64_workspace_bytes(n_systems) serves nvamd_fire_step_f64, nvamd_segment_fmax_f64 and
+ * nvamd_lj_energy_forces_f64 (which needs it only with virials or system_energies); the neighbor build uses
+ * nvamd_nl_workspace_bytes.  Not built for float64: the Verlet-skin test, the wrap, the thermostats, FIRE 2.0.
+ * ---------------------------------------------------------------------------------------- */
+int32_t nvamd_nl_build_f64(const double* positions, const double* cell, const uint8_t* pbc,
+                           const int32_t* batch_ptr, const int32_t* batch_idx, const uint8_t* rebuild_flags,
+                           int32_t n_atoms, int32_t n_systems, double cutoff, int32_t max_neighbors,
+                           int32_t half_fill, int32_t tail_mode, int32_t sort_path, int32_t* neighbor_matrix,
+                           int32_t* num_neighbors, int32_t* neighbor_matrix_shifts, void* workspace,
+                           size_t workspace_bytes, void* stream);
+int32_t nvamd_f64_workspace_bytes(int32_t n_systems, size_t* bytes);
+int32_t nvamd_lj_energy_forces_f64(const double* positions, const double* cells, const int32_t* neighbor_matrix,
+                                   const int32_t* neighbor_matrix_shifts, const int32_t* num_neighbors,
+                                   const int32_t* batch_idx, int32_t n_atoms, int32_t max_neighbors,
+                                   int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
+                                   double cutoff, double switch_width, int32_t half_list, double* atomic_energies,
+                                   double* forces, double* virials, double* system_energies, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+int32_t nvamd_vv_position_update_f64(double* positions, double* velocities, const double* forces,
+                                     const double* masses, const double* dt, const int32_t* batch_idx,
+                                     const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* stream);
+int32_t nvamd_vv_velocity_finalize_f64(double* velocities, const double* forces_new, const double* masses,
+                                       const double* dt, const int32_t* batch_idx, const uint8_t* active,
+                                       int32_t n_atoms, int32_t n_systems, void* stream);
+int32_t nvamd_fire_step_f64(double* positions, double* velocities, const double* forces, const double* masses,
+                            double* alpha, double* dt, const double* alpha_start, const double* f_alpha,
+                            const double* dt_min, const double* dt_max, const double* maxstep,
+                            int32_t* n_steps_positive, const int32_t* n_min, const double* f_dec,
+                            const double* f_inc, const int32_t* uphill_flag, double* vf, double* vv, double* ff,
+                            const int32_t* batch_idx, int32_t compute_reductions, const uint8_t* active,
+                            int32_t n_atoms, int32_t n_systems, void* workspace, size_t workspace_bytes,
+                            void* stream);
+int32_t nvamd_segment_fmax_f64(const double* forces, const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
+                               double* fmax, void* workspace, size_t workspace_bytes, void* stream);
+
 /* What the neighbor builds through this workspace had to report.  No counterpart in the reference, whose
  * kernels report nothing (a caller there compares num_neighbors with max_neighbors on the host:
  * nvalchemi/neighbors.py:269-273, nvalchemi/hooks/neighbor_list.py:446-469).

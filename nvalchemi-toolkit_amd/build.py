@@ -19,7 +19,7 @@ CSRC = HERE / "csrc"
 INCLUDE = HERE.parent / "include"
 OUT_DIR = HERE / "nvalchemi_amd" / "lib"
 LIB = OUT_DIR / "libnvalchemi_amd.so"
-SOURCES = ["common.hip", "integrators.hip", "lj_pair.hip", "neighbor_list.hip", "coo.hip", "skin_wrap.hip", "observables.hip", "buffers.hip", "filter.hip", "langevin.hip", "nhc.hip"]
+SOURCES = ["common.hip", "integrators.hip", "lj_pair.hip", "neighbor_list.hip", "coo.hip", "skin_wrap.hip", "observables.hip", "buffers.hip", "filter.hip", "langevin.hip", "nhc.hip", "f64.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950",

@@ -52,8 +52,9 @@ __device__ __forceinline__ double pair_d2_nearest_diagonal(float xi, float yi, f
     return (d0 * d0 + d1 * d1) + d2 * d2;
 }
 
-__device__ __forceinline__ double pair_d2_exact(float xi, float yi, float zi, float xj, float yj,
-                                                float zj, int s0, int s1, int s2,
+// (the coordinates come as doubles: float32 inputs convert exactly, float64 inputs are used as they are)
+__device__ __forceinline__ double pair_d2_exact(double xi, double yi, double zi, double xj, double yj,
+                                                double zj, int s0, int s1, int s2,
                                                 const double* __restrict__ h, double& d0,
                                                 double& d1, double& d2) {
 #pragma clang fp contract(off)
@@ -61,9 +62,9 @@ __device__ __forceinline__ double pair_d2_exact(float xi, float yi, float zi, fl
     double tx = (a * h[0] + b * h[3]) + c * h[6];
     double ty = (a * h[1] + b * h[4]) + c * h[7];
     double tz = (a * h[2] + b * h[5]) + c * h[8];
-    d0 = ((double)xj - (double)xi) + tx;
-    d1 = ((double)yj - (double)yi) + ty;
-    d2 = ((double)zj - (double)zi) + tz;
+    d0 = (xj - xi) + tx;
+    d1 = (yj - yi) + ty;
+    d2 = (zj - zi) + tz;
     return (d0 * d0 + d1 * d1) + d2 * d2;
 }
 

@@ -154,8 +154,10 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
 }
 
 struct NlArgs {
-    const float* pos;
+    const float* pos;      // float32 positions and cells ...
     const float* cell;
+    const double* pos64;   // ... or float64 ones (then pos and cell are null)
+    const double* cell64;
     const uint8_t* pbc;
     const int32_t* ptr;
     const int32_t* bidx;
@@ -168,8 +170,26 @@ struct NlArgs {
     int32_t* shifts;
 };
 
-__device__ __forceinline__ void frac_of(const NlSys& s, const float* __restrict__ r, double* f) {
-    double x = (double)r[0], y = (double)r[1], z = (double)r[2];
+// position of atom i in double, whichever type it is stored in
+struct Pos3 {
+    double x, y, z;
+};
+__device__ __forceinline__ Pos3 load_pos(const NlArgs& a, size_t i) {
+    Pos3 p;
+    if (a.pos64) {
+        p.x = a.pos64[3 * i + 0];
+        p.y = a.pos64[3 * i + 1];
+        p.z = a.pos64[3 * i + 2];
+    } else {
+        p.x = (double)a.pos[3 * i + 0];
+        p.y = (double)a.pos[3 * i + 1];
+        p.z = (double)a.pos[3 * i + 2];
+    }
+    return p;
+}
+
+__device__ __forceinline__ void frac_of(const NlSys& s, const Pos3& r, double* f) {
+    double x = r.x, y = r.y, z = r.z;
     f[0] = x * s.hinv[0] + y * s.hinv[3] + z * s.hinv[6];
     f[1] = x * s.hinv[1] + y * s.hinv[4] + z * s.hinv[7];
     f[2] = x * s.hinv[2] + y * s.hinv[5] + z * s.hinv[8];
@@ -178,9 +198,11 @@ __device__ __forceinline__ void frac_of(const NlSys& s, const float* __restrict_
 // ---- 1 prepare ------------------------------------------------------------------------------
 // Per-system constants that do not depend on the atoms: cell, inverse, widths, periodic flags.
 __device__ __forceinline__ void system_setup(NlSys& s, const NlArgs& a, int t) {
-    const bool has_cell = a.cell != nullptr;
+    const bool has_cell = a.cell != nullptr || a.cell64 != nullptr;
 #pragma unroll
-    for (int k = 0; k < 9; ++k) s.h[k] = has_cell ? (double)a.cell[9 * (size_t)t + k] : ((k % 4 == 0) ? 1.0 : 0.0);
+    for (int k = 0; k < 9; ++k)
+        s.h[k] = a.cell64 ? a.cell64[9 * (size_t)t + k]
+                          : (a.cell ? (double)a.cell[9 * (size_t)t + k] : ((k % 4 == 0) ? 1.0 : 0.0));
     inv3(s.h, s.hinv);
 #pragma unroll
     for (int d = 0; d < 3; ++d) {
@@ -230,7 +252,7 @@ __global__ __launch_bounds__(kBlock) void nl_bounds_kernel(NlArgs a, NlWorkspace
     const NlSys& s = ws.sys[sidx];
     if (s.per[0] && s.per[1] && s.per[2]) return;
     double f[3];
-    frac_of(s, a.pos + 3 * (size_t)i, f);
+    frac_of(s, load_pos(a, (size_t)i), f);
 #pragma unroll
     for (int d = 0; d < 3; ++d) {
         if (s.per[d]) continue;
@@ -410,7 +432,7 @@ struct Binned {
     float u[3];    // cartesian offset from the cell's corner
 };
 
-__device__ __forceinline__ Binned bin_atom(const NlSys& s, const float* __restrict__ r) {
+__device__ __forceinline__ Binned bin_atom(const NlSys& s, const Pos3& r) {
     Binned b;
     double f[3], g[3];
     frac_of(s, r, f);
@@ -473,7 +495,7 @@ __global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws
     }
     if (i >= a.n_atoms) return;
     const NlSys& s = ws.sys[a.bidx[i]];
-    Binned b = bin_atom(s, a.pos + 3 * (size_t)i);
+    Binned b = bin_atom(s, load_pos(a, (size_t)i));
     ws.atom_rank[i] = atomicAdd(ws.cell_count + b.cell, 1);
 }
 
@@ -481,7 +503,7 @@ __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspac
     int i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= a.n_atoms) return;
     const NlSys& s = ws.sys[a.bidx[i]];
-    Binned b = bin_atom(s, a.pos + 3 * (size_t)i);
+    Binned b = bin_atom(s, load_pos(a, (size_t)i));
     int slot = ws.cell_start[b.cell] + ws.atom_rank[i];
     ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
     ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
@@ -534,7 +556,7 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
     // up to kKeep atoms per thread stay in registers from here to the scatter; their positions
     // are requested now, so that they arrive while thread 0 works out the system's grid
     constexpr int kKeep = 4;
-    const bool kept = (end - begin) <= kKeep * kSortBlock;
+    const bool kept = !a.pos64 && (end - begin) <= kKeep * kSortBlock;
     float my_pos[kKeep][3];
     if (kept) {
 #pragma unroll
@@ -558,7 +580,7 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
     if (!idle && !(s_sys.per[0] && s_sys.per[1] && s_sys.per[2])) {
         for (int i = begin + tid; i < end; i += kSortBlock) {
             double f[3];
-            frac_of(s_sys, a.pos + 3 * (size_t)i, f);
+            frac_of(s_sys, load_pos(a, (size_t)i), f);
 #pragma unroll
             for (int d = 0; d < 3; ++d) {
                 if (s_sys.per[d]) continue;
@@ -612,14 +634,14 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         for (int k = 0; k < kKeep; ++k) {
             const int i = begin + tid + k * kSortBlock;
             if (i < end) {
-                mine[k] = bin_atom(s_sys, my_pos[k]);
+                mine[k] = bin_atom(s_sys, Pos3{(double)my_pos[k][0], (double)my_pos[k][1], (double)my_pos[k][2]});
                 const int lc = mine[k].cell - cell_base;
                 my_rank[k] = in_lds ? atomicAdd(&s_hist[lc], 1) : atomicAdd(&g_hist[lc], 1);
             }
         }
     } else {
         for (int i = begin + tid; i < end; i += kSortBlock) {
-            const Binned b = bin_atom(s_sys, a.pos + 3 * (size_t)i);
+            const Binned b = bin_atom(s_sys, load_pos(a, (size_t)i));
             const int lc = b.cell - cell_base;
             ws.atom_rank[i] = in_lds ? atomicAdd(&s_hist[lc], 1) : atomicAdd(&g_hist[lc], 1);
         }
@@ -666,7 +688,7 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
             if (i < end) place(mine[k], i, my_rank[k]);
         }
     } else {
-        for (int i = begin + tid; i < end; i += kSortBlock) place(bin_atom(s_sys, a.pos + 3 * (size_t)i), i, ws.atom_rank[i]);
+        for (int i = begin + tid; i < end; i += kSortBlock) place(bin_atom(s_sys, load_pos(a, (size_t)i)), i, ws.atom_rank[i]);
     }
     __syncthreads();
     // ---- the system's units of search work.  A run of cells with more centre atoms than one
@@ -1067,10 +1089,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                     j = __float_as_int(p.w);
                                     candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
                                     if (!(dist2(p) < rc2_lo)) {  // inside the band: decide exactly
-                                        const float* pi = a.pos + 3 * (size_t)i_atom;
-                                        const float* pj = a.pos + 3 * (size_t)j;
+                                        const Pos3 pi = load_pos(a, (size_t)i_atom), pj = load_pos(a, (size_t)j);
                                         double e0, e1d, e2d;
-                                        in = pair_d2_exact(pi[0], pi[1], pi[2], pj[0], pj[1], pj[2], s0, s1, s2,
+                                        in = pair_d2_exact(pi.x, pi.y, pi.z, pj.x, pj.y, pj.z, s0, s1, s2,
                                                            ws.sys[sidx].h, e0, e1d, e2d) < a.rc2;
                                     }
                                     if (HALF && in) in = half_keep(i_atom, j, s0, s1, s2);
@@ -1247,24 +1268,25 @@ NVAMD_EXPORT int32_t nvamd_nl_build(const float* positions, const float* cell, c
                                neighbor_matrix_shifts, workspace, workspace_bytes, stream);
 }
 
-NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* cell, const uint8_t* pbc,
-                                         const int32_t* batch_ptr, const int32_t* batch_idx,
-                                         const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
-                                         double cutoff, int32_t max_neighbors, int32_t half_fill,
-                                         int32_t tail_mode, int32_t sort_path, int32_t* neighbor_matrix,
-                                         int32_t* num_neighbors, int32_t* neighbor_matrix_shifts, void* workspace,
-                                         size_t workspace_bytes, void* stream) {
+static int32_t nl_build_impl(const float* positions, const float* cell, const double* positions64, const double* cell64,
+                             const uint8_t* pbc, const int32_t* batch_ptr, const int32_t* batch_idx,
+                             const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems, double cutoff,
+                             int32_t max_neighbors, int32_t half_fill, int32_t tail_mode, int32_t sort_path,
+                             int32_t* neighbor_matrix, int32_t* num_neighbors, int32_t* neighbor_matrix_shifts,
+                             void* workspace, size_t workspace_bytes, void* stream) {
     if (sort_path != NVAMD_NL_SORT_AUTO && sort_path != NVAMD_NL_SORT_PER_SYSTEM && sort_path != NVAMD_NL_SORT_GLOBAL)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: unknown sort_path %d", (int)sort_path);
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: negative size");
     if (!(cutoff > 0.0)) return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: cutoff must be positive");
     if (n_atoms == 0 || n_systems == 0) return NVAMD_OK;
-    if (!positions || !batch_ptr || !batch_idx || !num_neighbors || (max_neighbors > 0 && !neighbor_matrix))
+    if ((!positions && !positions64) || !batch_ptr || !batch_idx || !num_neighbors ||
+        (max_neighbors > 0 && !neighbor_matrix))
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: null buffer");
-    if ((cell == nullptr) != (pbc == nullptr))
+    const bool has_cell = cell != nullptr || cell64 != nullptr;
+    if (has_cell != (pbc != nullptr))
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: cell and pbc must be given together");
-    if (cell && !neighbor_matrix_shifts && max_neighbors > 0)
+    if (has_cell && !neighbor_matrix_shifts && max_neighbors > 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: periodic build needs neighbor_matrix_shifts");
     size_t need = carve(nullptr, nullptr, n_atoms, n_systems);
     if (!workspace || workspace_bytes < need)
@@ -1277,6 +1299,8 @@ NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* ce
     NlArgs a;
     a.pos = positions;
     a.cell = cell;
+    a.pos64 = positions64;
+    a.cell64 = cell64;
     a.pbc = pbc;
     a.ptr = batch_ptr;
     a.bidx = batch_idx;
@@ -1323,4 +1347,28 @@ NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* ce
     else hipLaunchKernelGGL(nl_search_kernel<false>, dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start);
     NVAMD_LAUNCH_CHECK("neighbor list launch");
     return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* cell, const uint8_t* pbc,
+                                         const int32_t* batch_ptr, const int32_t* batch_idx,
+                                         const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                                         double cutoff, int32_t max_neighbors, int32_t half_fill,
+                                         int32_t tail_mode, int32_t sort_path, int32_t* neighbor_matrix,
+                                         int32_t* num_neighbors, int32_t* neighbor_matrix_shifts, void* workspace,
+                                         size_t workspace_bytes, void* stream) {
+    return nl_build_impl(positions, cell, nullptr, nullptr, pbc, batch_ptr, batch_idx, rebuild_flags, n_atoms, n_systems,
+                         cutoff, max_neighbors, half_fill, tail_mode, sort_path, neighbor_matrix, num_neighbors,
+                         neighbor_matrix_shifts, workspace, workspace_bytes, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_build_f64(const double* positions, const double* cell, const uint8_t* pbc,
+                                        const int32_t* batch_ptr, const int32_t* batch_idx,
+                                        const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                                        double cutoff, int32_t max_neighbors, int32_t half_fill,
+                                        int32_t tail_mode, int32_t sort_path, int32_t* neighbor_matrix,
+                                        int32_t* num_neighbors, int32_t* neighbor_matrix_shifts, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+    return nl_build_impl(nullptr, nullptr, positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, n_atoms, n_systems,
+                         cutoff, max_neighbors, half_fill, tail_mode, sort_path, neighbor_matrix, num_neighbors,
+                         neighbor_matrix_shifts, workspace, workspace_bytes, stream);
 }

@@ -29,6 +29,15 @@ _SIGNATURES = {
     "nvamd_last_error": (_c.c_char_p, []),
     "nvamd_nl_workspace_bytes": (_i32, [_i32, _i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_nl_status": (_i32, [_vp, _c.c_size_t, _i32, _i32, _vp, _i32, _vp]),
+    "nvamd_nl_build_f64": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32, _i32,
+                                  _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_f64_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_lj_energy_forces_f64": (_i32, [_vp] * 6 + [_i32, _i32, _i32, _i32, _f64, _f64, _f64, _f64, _i32,
+                                          _vp, _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
+    "nvamd_vv_position_update_f64": (_i32, [_vp] * 7 + [_i32, _i32, _vp]),
+    "nvamd_vv_velocity_finalize_f64": (_i32, [_vp] * 6 + [_i32, _i32, _vp]),
+    "nvamd_fire_step_f64": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
+    "nvamd_segment_fmax_f64": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_build": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32,
                               _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_build_path": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32, _i32,
@@ -125,6 +134,13 @@ def _dev(t: torch.Tensor, name: str, dtype: torch.dtype, shape: tuple | None = N
     return t.data_ptr()
 
 
+def _real_dtype(t: torch.Tensor, name: str) -> torch.dtype:
+    """float32 (the tuned kernels) or float64 (the plain ones); anything else is refused."""
+    if t.dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"{name}: expected float32 or float64, got {t.dtype}")
+    return t.dtype
+
+
 def _opt(t, name, dtype, shape=None) -> int | None:
     return None if t is None else _dev(t, name, dtype, shape)
 
@@ -188,8 +204,10 @@ def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, 
     N = positions.shape[0]
     B = batch_ptr.shape[0] - 1
     K = int(max_neighbors)
-    p_pos = _dev(positions, "positions", torch.float32, (N, 3))
-    p_cell = _opt(cell, "cell", torch.float32, (B, 3, 3))
+    # float32 or float64 positions, the cell in the same type (the reference's ops take both)
+    real = _real_dtype(positions, "positions")
+    p_pos = _dev(positions, "positions", real, (N, 3))
+    p_cell = _opt(cell, "cell", real, (B, 3, 3))
     p_pbc = _opt(_as_u8(pbc), "pbc", torch.uint8, (B, 3))
     p_ptr = _dev(batch_ptr, "batch_ptr", torch.int32, (B + 1,))
     p_idx = _dev(batch_idx, "batch_idx", torch.int32, (N,))
@@ -201,9 +219,10 @@ def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, 
     ws = workspace if workspace is not None else workspaces.get(positions.device, "nl", need)
     if ws.device != positions.device or ws.numel() * ws.element_size() < need:
         raise ValueError("neighbor-list workspace too small or on another device")
-    _check(lib.nvamd_nl_build_path(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,
-                                   int(bool(half_fill)), int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
-                                   ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)),
+    entry = lib.nvamd_nl_build_f64 if real == torch.float64 else lib.nvamd_nl_build_path
+    _check(entry(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,
+                 int(bool(half_fill)), int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
+                 ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)),
            "nvamd_nl_build")
 
 
@@ -261,6 +280,21 @@ def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, 
     N = positions.shape[0]
     K = neighbor_matrix.shape[1]
     B = cells.shape[0]
+    if _real_dtype(positions, "positions") == torch.float64:
+        f64 = torch.float64
+        ws = workspaces.get(positions.device, "f64", _size(lib.nvamd_f64_workspace_bytes, B))
+        _check(lib.nvamd_lj_energy_forces_f64(
+            _dev(positions, "positions", f64, (N, 3)), _dev(cells, "cells", f64, (B, 3, 3)),
+            _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+            _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+            _dev(num_neighbors, "num_neighbors", torch.int32, (N,)),
+            _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+            N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), float(switch_width),
+            int(bool(half_list)), _dev(atomic_energies, "atomic_energies", f64, (N,)),
+            _dev(forces, "forces", f64, (N, 3)), _opt(virials, "virials", f64, (B, 9)),
+            _opt(system_energies, "system_energies", f64, (B,)),
+            ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_f64")
+        return
     need = _size(lib.nvamd_lj_workspace_bytes, N, B, int(bool(half_list)))
     ws = workspaces.get(positions.device, "lj", need)
     _check(lib.nvamd_lj_energy_forces_hinted(
@@ -328,12 +362,14 @@ def nl_atom_order(batch_idx, n_systems: int, atom_order, rebuild_flags=None) -> 
 def vv_position_update(positions, velocities, forces, masses, dt, batch_idx, active=None) -> None:
     N = positions.shape[0]
     M = dt.shape[0]
-    _check(library().nvamd_vv_position_update(
-        _dev(positions, "positions", torch.float32, (N, 3)),
-        _dev(velocities, "velocities", torch.float32, (N, 3)),
-        _dev(forces, "forces", torch.float32, (N, 3)),
-        _dev(masses, "masses", torch.float32, (N,)),
-        _dev(dt, "dt", torch.float32, (M,)),
+    real = _real_dtype(positions, "positions")
+    entry = library().nvamd_vv_position_update_f64 if real == torch.float64 else library().nvamd_vv_position_update
+    _check(entry(
+        _dev(positions, "positions", real, (N, 3)),
+        _dev(velocities, "velocities", real, (N, 3)),
+        _dev(forces, "forces", real, (N, 3)),
+        _dev(masses, "masses", real, (N,)),
+        _dev(dt, "dt", real, (M,)),
         _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         _opt(_as_u8(active), "active", torch.uint8, (M,)),
         N, M, _stream(positions.device)), "nvamd_vv_position_update")
@@ -342,11 +378,13 @@ def vv_position_update(positions, velocities, forces, masses, dt, batch_idx, act
 def vv_velocity_finalize(velocities, forces_new, masses, dt, batch_idx, active=None) -> None:
     N = velocities.shape[0]
     M = dt.shape[0]
-    _check(library().nvamd_vv_velocity_finalize(
-        _dev(velocities, "velocities", torch.float32, (N, 3)),
-        _dev(forces_new, "forces_new", torch.float32, (N, 3)),
-        _dev(masses, "masses", torch.float32, (N,)),
-        _dev(dt, "dt", torch.float32, (M,)),
+    real = _real_dtype(velocities, "velocities")
+    entry = library().nvamd_vv_velocity_finalize_f64 if real == torch.float64 else library().nvamd_vv_velocity_finalize
+    _check(entry(
+        _dev(velocities, "velocities", real, (N, 3)),
+        _dev(forces_new, "forces_new", real, (N, 3)),
+        _dev(masses, "masses", real, (N,)),
+        _dev(dt, "dt", real, (M,)),
         _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         _opt(_as_u8(active), "active", torch.uint8, (M,)),
         N, M, _stream(velocities.device)), "nvamd_vv_velocity_finalize")
@@ -358,10 +396,14 @@ def fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_a
     lib = library()
     N = positions.shape[0]
     M = alpha.shape[0]
-    f32, i32 = torch.float32, torch.int32
-    need = _size(lib.nvamd_fire_workspace_bytes, M)
-    ws = workspaces.get(positions.device, "fire", need)
-    _check(lib.nvamd_fire_step(
+    f32, i32 = _real_dtype(positions, "positions"), torch.int32
+    if f32 == torch.float64:
+        entry = lib.nvamd_fire_step_f64
+        ws = workspaces.get(positions.device, "f64", _size(lib.nvamd_f64_workspace_bytes, M))
+    else:
+        entry = lib.nvamd_fire_step
+        ws = workspaces.get(positions.device, "fire", _size(lib.nvamd_fire_workspace_bytes, M))
+    _check(entry(
         _dev(positions, "positions", f32, (N, 3)), _dev(velocities, "velocities", f32, (N, 3)),
         _dev(forces, "forces", f32, (N, 3)), _dev(masses, "masses", f32, (N,)),
         _dev(alpha, "alpha", f32, (M,)), _dev(dt, "dt", f32, (M,)),
@@ -378,6 +420,14 @@ def fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_a
 def segment_fmax(forces, batch_idx, fmax) -> None:
     N = forces.shape[0]
     M = fmax.shape[0]
+    if _real_dtype(forces, "forces") == torch.float64:
+        lib = library()
+        ws = workspaces.get(forces.device, "f64", _size(lib.nvamd_f64_workspace_bytes, M))
+        _check(lib.nvamd_segment_fmax_f64(
+            _dev(forces, "forces", torch.float64, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+            N, M, _dev(fmax, "fmax", torch.float64, (M,)), ws.data_ptr(), ws.numel(), _stream(forces.device)),
+            "nvamd_segment_fmax_f64")
+        return
     _check(library().nvamd_segment_fmax(
         _dev(forces, "forces", torch.float32, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         N, M, _dev(fmax, "fmax", torch.float32, (M,)), _stream(forces.device)), "nvamd_segment_fmax")

@@ -36,8 +36,8 @@ def suggest_neighbor_list_method(batch_ptr: torch.Tensor, cell: torch.Tensor, pb
     One cell-list kernel serves every input here, so the answer only says "batched cell list"; the
     reference's cost model lives in its kernel library and picks among strategies this build does
     not have.  Host-only, no synchronisation."""
-    if positions_dtype != torch.float32:
-        raise NotImplementedError("the HIP neighbor list takes float32 positions")
+    if positions_dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"neighbor list positions must be float32 or float64, got {positions_dtype}")
     return "batch_cell_list"
 
 
@@ -77,8 +77,8 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
     """
     if method not in _METHODS:
         raise ValueError(f"unknown neighbor list method {method!r}")
-    if positions.dtype != torch.float32:
-        raise NotImplementedError("the HIP neighbor list takes float32 positions")
+    if positions.dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"neighbor list positions must be float32 or float64, got {positions.dtype}")
     N = positions.shape[0]
     dev = positions.device
     if batch_ptr is None:
@@ -94,7 +94,7 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
         else:
             pbc = torch.zeros(B, 3, dtype=torch.bool, device=dev)
     if cell is not None:
-        cell = cell.to(torch.float32).reshape(B, 3, 3).contiguous()
+        cell = cell.to(positions.dtype).reshape(B, 3, 3).contiguous()
         pbc = pbc.reshape(B, 3).contiguous()
     K = int(max_neighbors if max_neighbors is not None else
             (neighbor_matrix.shape[1] if neighbor_matrix is not None else estimate_max_neighbors(cutoff)))

@@ -78,7 +78,7 @@ class _ConvergenceCriterion(BaseModel):
 
     def _is_force_norm(self, target: torch.Tensor, batch) -> bool:
         return (self.reduce_op == "norm" and self.reduce_dims in (-1, 1) and target.dim() == 2
-                and target.shape[1] == 3 and target.dtype == torch.float32 and target.is_cuda
+                and target.shape[1] == 3 and target.dtype in (torch.float32, torch.float64) and target.is_cuda
                 and target.shape[0] == batch.num_nodes and batch.num_nodes != batch.num_graphs)
 
     def __call__(self, batch) -> torch.Tensor:
@@ -90,7 +90,7 @@ class _ConvergenceCriterion(BaseModel):
             return self.custom_op(target)
         if self._is_force_norm(target, batch):
             # per-system max of the atomic force norms in one pass
-            fmax = torch.empty(batch.num_graphs, dtype=torch.float32, device=target.device)
+            fmax = torch.empty(batch.num_graphs, dtype=target.dtype, device=target.device)
             _lib.segment_fmax(target.contiguous(), batch.batch_idx, fmax)
             return fmax <= self.threshold
         target = self._reduce_within_entry(target)

@@ -122,6 +122,7 @@ class NeighborListHook:
         self._build(batch, cutoff, cell, pbc,
                     rebuild_flags=self._rebuild_flags if (self.skin > 0.0 and self._ref_positions is not None) else None)
 
+        first = self._first_build
         if self._first_build:
             # the one host synchronisation: validate K against the actual maximum
             self._first_build = False
@@ -135,6 +136,10 @@ class NeighborListHook:
                     self._realloc_k(N, positions.device, pbc)
                     self._build(batch, cutoff, cell, pbc, rebuild_flags=None)
 
+        if first and N > 0:
+            # whatever earlier builds left in the workspace's status bits (the first build's own overflow
+            # has been dealt with above) is not this hook's: overflowed() starts from here
+            _lib.nl_status(N, B, positions.device, clear=True)
         self._publish_row_order(batch, N, B)
         _write_neighbor_data_to_batch(
             batch=batch, neighbor_matrix=self._neighbor_matrix, num_neighbors=self._num_neighbors,
@@ -145,7 +150,9 @@ class NeighborListHook:
     def overflowed(self, clear: bool = True) -> bool:
         """Whether any build since the last call left an atom with more neighbors than the rows hold
         (the reference never notices this after its first build, nvalchemi/hooks/neighbor_list.py:351-355;
-        the kernels here count past K on the device and keep a flag).  One host synchronisation."""
+        the kernels here count past K on the device and keep a flag).  One host synchronisation.  The flag
+        lives in the build's workspace, which all builds of a device and stream share: another hook's
+        overflow on the same stream shows up here too."""
         if self._neighbor_matrix is None or self._alloc_N in (None, 0):
             return False
         st = _lib.nl_status(self._alloc_N, self._alloc_B, self._neighbor_matrix.device, clear=clear)

@@ -24,9 +24,10 @@ from ... import _lib
 
 
 def _check_dtype(positions: Tensor) -> None:
-    if positions.dtype != torch.float32:
-        raise NotImplementedError("the HIP Lennard-Jones kernel takes float32 positions "
-                                  "(pair math is double internally)")
+    """float32 (the tuned kernel; pair math is double internally) or float64 (a plain kernel: shifts
+    always read, no staging, no walk order), as the reference's ops take both."""
+    if positions.dtype not in (torch.float32, torch.float64):
+        raise TypeError(f"Lennard-Jones positions must be float32 or float64, got {positions.dtype}")
 
 
 def _shifts_or_none(neighbor_matrix_shifts: Tensor | None) -> Tensor | None:
@@ -45,7 +46,7 @@ def lj_energy_forces_batch(positions: Tensor, cells: Tensor, neighbor_matrix: Te
     N = positions.shape[0]
     e = torch.empty(N, dtype=positions.dtype, device=positions.device)
     f = torch.empty(N, 3, dtype=positions.dtype, device=positions.device)
-    _lib.lj_energy_forces(positions.contiguous(), cells.contiguous(), neighbor_matrix.contiguous(),
+    _lib.lj_energy_forces(positions.contiguous(), cells.to(positions.dtype).contiguous(), neighbor_matrix.contiguous(),
                           neighbor_matrix_shifts.contiguous(), num_neighbors.contiguous(),
                           batch_idx.contiguous(), fill_value, epsilon, sigma, cutoff, switch_width,
                           half_list, e, f)
@@ -73,7 +74,7 @@ def lj_energy_forces_virial_batch(positions: Tensor, cells: Tensor, neighbor_mat
     e = torch.empty(N, dtype=positions.dtype, device=positions.device)
     f = torch.empty(N, 3, dtype=positions.dtype, device=positions.device)
     w = torch.empty(B, 9, dtype=positions.dtype, device=positions.device)
-    _lib.lj_energy_forces(positions.contiguous(), cells.contiguous(), neighbor_matrix.contiguous(),
+    _lib.lj_energy_forces(positions.contiguous(), cells.to(positions.dtype).contiguous(), neighbor_matrix.contiguous(),
                           neighbor_matrix_shifts.contiguous(), num_neighbors.contiguous(),
                           batch_idx.contiguous(), fill_value, epsilon, sigma, cutoff, switch_width,
                           half_list, e, f, virials=w)
@@ -123,7 +124,7 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
         w = out.get("virials")
         if w is None:
             w = torch.empty(B, 9, dtype=dt, device=dev)
-    _lib.lj_energy_forces(positions, cells, neighbor_matrix, _shifts_or_none(neighbor_matrix_shifts),
+    _lib.lj_energy_forces(positions, cells.to(dt), neighbor_matrix, _shifts_or_none(neighbor_matrix_shifts),
                           num_neighbors, batch_idx, fill_value, epsilon, sigma, cutoff, switch_width,
                           half_list, e, f, virials=w, system_energies=es, row_order=row_order,
                           neighbor_list_cutoff=neighbor_list_cutoff)

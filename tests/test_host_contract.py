@@ -253,9 +253,12 @@ def test_strategy_helpers_of_the_neighbor_hook():
     assert neighbor_list_strategy_run_args("batch_cell_list_pair_centric")[0] == "batch_cell_list"
     with pytest.raises(ValueError):
         neighbor_list_strategy_run_args("no_such_strategy")
-    with pytest.raises(NotImplementedError):
+    # float32 and float64 positions are both served (as in the reference); anything else is refused
+    assert suggest_neighbor_list_method(ptr, torch.eye(3).repeat(2, 1, 1), torch.ones(2, 3, dtype=torch.bool), 3.0,
+                                        positions_dtype=torch.float64) == name
+    with pytest.raises(TypeError):
         suggest_neighbor_list_method(ptr, torch.eye(3).repeat(2, 1, 1), torch.ones(2, 3, dtype=torch.bool), 3.0,
-                                     positions_dtype=torch.float64)
+                                     positions_dtype=torch.float16)
 
 
 def test_batch_index_select_append_and_trim():
