@@ -110,8 +110,11 @@ __global__ __launch_bounds__(kBlock) void lj_sys_range_kernel(const int32_t* __r
                                                               const float* __restrict__ cells, double list_rc,
                                                               int32_t* __restrict__ first,
                                                               int32_t* __restrict__ last,
-                                                              LjSysImage* __restrict__ image) {
+                                                              LjSysImage* __restrict__ image,
+                                                              double* __restrict__ sys_acc, int n_acc) {
     int i = blockIdx.x * kBlock + threadIdx.x;
+    // (the per-system accumulators start at zero: cleared here rather than by a launch of their own)
+    if (sys_acc && i < n_acc) sys_acc[i] = 0.0;
     if (i >= n_atoms) return;
     int s = bidx[i];
     if (i == n_atoms - 1 || bidx[i + 1] != s) last[s] = i + 1;
@@ -708,11 +711,15 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
                                                           2 * align_up(nsys * sizeof(int32_t)));
     char* w_half = w + align_up(nsys * 10 * sizeof(double)) + 2 * align_up(nsys * sizeof(int32_t)) +
                    align_up(nsys * sizeof(LjSysImage));
+    // the full-list path clears the accumulators in its range kernel when there are at least as many atoms
+    // as accumulator words
+    const bool clear_with_ranges = !half_list && (size_t)n_atoms >= (size_t)n_systems * 10;
     if (want_sys && n_systems > 0) {
         a.sys_acc = reinterpret_cast<double*>(w);
         size_t n = (size_t)n_systems * 10;
-        hipLaunchKernelGGL(clear_f64_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                           st, a.sys_acc, n);
+        if (!clear_with_ranges)
+            hipLaunchKernelGGL(clear_f64_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                               st, a.sys_acc, n);
     }
     if (n_atoms > 0) {
         if (half_list) {
@@ -734,7 +741,8 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
             const bool vir = virials != nullptr;
             const bool sys = a.sys_acc != nullptr;
             hipLaunchKernelGGL(lj_sys_range_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
-                               batch_idx, n_atoms, shifts ? cells : nullptr, a.list_rc, sys_first, sys_last, sys_image);
+                               batch_idx, n_atoms, shifts ? cells : nullptr, a.list_rc, sys_first, sys_last, sys_image,
+                               clear_with_ranges ? a.sys_acc : nullptr, n_systems * 10);
             a.sys_first = sys_first;
             a.sys_last = sys_last;
             a.sys_image = sys_image;
