@@ -795,7 +795,7 @@ __device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, i
 // candidates a centre cell of the run has to look at are one contiguous range of the LDS tile;
 // what a range picks up beyond its own layers (ranges are widened to multiples of 64) lies
 // further than the stencil radius away and can never pass the distance test.
-template <bool HALF>
+template <bool HALF, bool F64>
 // The tables that every lane of a workgroup reads at the same address (unit records, the per-system
 // constants, the run's cell ranges) come in as read-only arguments of their own besides the workspace:
 // nothing in the kernel can be seen to write them, so they are fetched through the scalar cache, which
@@ -1089,7 +1089,18 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                     j = __float_as_int(p.w);
                                     candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
                                     if (!(dist2(p) < rc2_lo)) {  // inside the band: decide exactly
-                                        const Pos3 pi = load_pos(a, (size_t)i_atom), pj = load_pos(a, (size_t)j);
+                                        // (the type of the positions is a compile-time matter here: looking at it
+                                        // at run time costs the float32 kernel registers it does not have)
+                                        Pos3 pi, pj;
+                                        if (F64) {
+                                            pi = Pos3{a.pos64[3 * (size_t)i_atom], a.pos64[3 * (size_t)i_atom + 1], a.pos64[3 * (size_t)i_atom + 2]};
+                                            pj = Pos3{a.pos64[3 * (size_t)j], a.pos64[3 * (size_t)j + 1], a.pos64[3 * (size_t)j + 2]};
+                                        } else {
+                                            const float* fi = a.pos + 3 * (size_t)i_atom;
+                                            const float* fj = a.pos + 3 * (size_t)j;
+                                            pi = Pos3{(double)fi[0], (double)fi[1], (double)fi[2]};
+                                            pj = Pos3{(double)fj[0], (double)fj[1], (double)fj[2]};
+                                        }
                                         double e0, e1d, e2d;
                                         in = pair_d2_exact(pi.x, pi.y, pi.z, pj.x, pj.y, pj.z, s0, s1, s2,
                                                            ws.sys[sidx].h, e0, e1d, e2d) < a.rc2;
@@ -1343,8 +1354,16 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     unsigned n_search = 8u * 2048u;
     size_t cells_bound = max_cells_for(n_atoms, n_systems);
     if (cells_bound < n_search) n_search = (unsigned)((cells_bound + 7) / 8 * 8);
-    if (a.half) hipLaunchKernelGGL(nl_search_kernel<true>, dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start);
-    else hipLaunchKernelGGL(nl_search_kernel<false>, dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start);
+#define NVAMD_NL_SEARCH(H, D) \
+    hipLaunchKernelGGL((nl_search_kernel<H, D>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start)
+    if (a.pos64) {
+        if (a.half) NVAMD_NL_SEARCH(true, true);
+        else NVAMD_NL_SEARCH(false, true);
+    } else {
+        if (a.half) NVAMD_NL_SEARCH(true, false);
+        else NVAMD_NL_SEARCH(false, false);
+    }
+#undef NVAMD_NL_SEARCH
     NVAMD_LAUNCH_CHECK("neighbor list launch");
     return NVAMD_OK;
 }
