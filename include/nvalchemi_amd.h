@@ -110,6 +110,17 @@ int32_t nvamd_nl_matrix_to_coo(const int32_t* neighbor_matrix,
                                int32_t n_atoms, int32_t max_neighbors, int64_t edge_capacity,
                                int32_t* neighbor_list, int32_t* neighbor_list_shifts,
                                void* stream);
+/* Both steps in one call, for callers that bring buffers of a capacity of their choice and do not want to
+ * wait for the edge count in between (the same call site, nvalchemi/neighbors.py:92-103): the edge pointer
+ * is scanned on the device, edges below edge_capacity are written, and counts (2) i32 on the device receives
+ * the number of edges E and 1 if E exceeds edge_capacity (then the caller grows its buffers and calls again;
+ * the overflow protocol of the matrix build, for edges).  No host synchronisation.
+ * workspace: nvamd_coo_workspace_bytes(n_atoms). */
+int32_t nvamd_nl_coo_from_matrix(const int32_t* neighbor_matrix, const int32_t* neighbor_matrix_shifts,
+                                 const int32_t* num_neighbors, int32_t n_atoms, int32_t max_neighbors,
+                                 int64_t edge_capacity, int32_t* edge_ptr, int32_t* neighbor_list,
+                                 int32_t* neighbor_list_shifts, int32_t* counts, void* workspace,
+                                 size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Lennard-Jones pair kernel over the neighbor matrix.  Replaces the Warp launches inside

@@ -39,6 +39,14 @@ __global__ __launch_bounds__(kBlock) void coo_fill_kernel(const int32_t* __restr
     }
 }
 
+// total number of edges and whether it exceeds what the caller's buffers hold
+__global__ void coo_count_kernel(const int32_t* __restrict__ edge_ptr, int n_atoms, long long cap,
+                                 int32_t* __restrict__ counts) {
+    const int e = edge_ptr[n_atoms];
+    counts[0] = e;
+    counts[1] = (long long)e > cap ? 1 : 0;
+}
+
 }  // namespace
 }  // namespace nvamd
 
@@ -86,5 +94,22 @@ NVAMD_EXPORT int32_t nvamd_nl_matrix_to_coo(const int32_t* neighbor_matrix,
                        st, neighbor_matrix, neighbor_matrix_shifts, edge_ptr, n_atoms, max_neighbors,
                        (long long)edge_capacity, neighbor_list, neighbor_list_shifts);
     NVAMD_LAUNCH_CHECK("coo launch");
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_coo_from_matrix(const int32_t* neighbor_matrix, const int32_t* neighbor_matrix_shifts,
+                                              const int32_t* num_neighbors, int32_t n_atoms, int32_t max_neighbors,
+                                              int64_t edge_capacity, int32_t* edge_ptr, int32_t* neighbor_list,
+                                              int32_t* neighbor_list_shifts, int32_t* counts, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+    if (!counts) return fail(NVAMD_ERR_INVALID_ARGUMENT, "coo: null counts");
+    int32_t rc = nvamd_nl_edge_ptr(num_neighbors, n_atoms, max_neighbors, edge_ptr, workspace, workspace_bytes, stream);
+    if (rc != NVAMD_OK) return rc;
+    rc = nvamd_nl_matrix_to_coo(neighbor_matrix, neighbor_matrix_shifts, edge_ptr, n_atoms, max_neighbors,
+                                edge_capacity, neighbor_list, neighbor_list_shifts, stream);
+    if (rc != NVAMD_OK) return rc;
+    hipLaunchKernelGGL(coo_count_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream), edge_ptr, n_atoms,
+                       (long long)edge_capacity, counts);
+    NVAMD_LAUNCH_CHECK("coo count launch");
     return NVAMD_OK;
 }

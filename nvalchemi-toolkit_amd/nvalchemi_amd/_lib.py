@@ -43,6 +43,7 @@ _SIGNATURES = {
     "nvamd_nl_build_path": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _f64, _i32, _i32, _i32, _i32,
                                    _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_coo_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
+    "nvamd_nl_coo_from_matrix": (_i32, [_vp, _vp, _vp, _i32, _i32, _c.c_int64, _vp, _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_edge_ptr": (_i32, [_vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_matrix_to_coo": (_i32, [_vp, _vp, _vp, _i32, _i32, _c.c_int64, _vp, _vp, _vp]),
     "nvamd_lj_workspace_bytes": (_i32, [_i32, _i32, _i32, _c.POINTER(_c.c_size_t)]),
@@ -253,6 +254,25 @@ def nl_edge_ptr(num_neighbors, max_neighbors, edge_ptr) -> None:
                                  int(max_neighbors), _dev(edge_ptr, "edge_ptr", torch.int32, (N + 1,)),
                                  ws.data_ptr(), ws.numel(), _stream(num_neighbors.device)),
            "nvamd_nl_edge_ptr")
+
+
+def nl_coo_from_matrix(neighbor_matrix, neighbor_matrix_shifts, num_neighbors, edge_ptr, neighbor_list,
+                       neighbor_list_shifts, counts) -> None:
+    """Edge pointer and edges in one call; ``neighbor_list (E_cap, 2)`` sets the capacity, ``counts (2)``
+    receives the edge count and an overflow flag on the device.  No host synchronisation."""
+    lib = library()
+    N, K = neighbor_matrix.shape
+    cap = neighbor_list.shape[0]
+    ws = workspaces.get(neighbor_matrix.device, "coo", _size(lib.nvamd_coo_workspace_bytes, N))
+    _check(lib.nvamd_nl_coo_from_matrix(
+        _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+        _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+        _dev(num_neighbors, "num_neighbors", torch.int32, (N,)), N, K, cap,
+        _dev(edge_ptr, "edge_ptr", torch.int32, (N + 1,)),
+        _dev(neighbor_list, "neighbor_list", torch.int32, (cap, 2)),
+        _opt(neighbor_list_shifts, "neighbor_list_shifts", torch.int32, (cap, 3)),
+        _dev(counts, "counts", torch.int32, (2,)), ws.data_ptr(), ws.numel(),
+        _stream(neighbor_matrix.device)), "nvamd_nl_coo_from_matrix")
 
 
 def nl_matrix_to_coo(neighbor_matrix, neighbor_matrix_shifts, edge_ptr, neighbor_list,

@@ -110,20 +110,41 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
     return neighbor_matrix, num_neighbors, neighbor_matrix_shifts
 
 
+#: edge count of the last conversion of a matrix of the same shape: the capacity the next one starts with
+_last_edge_count: dict[tuple, int] = {}
+
+
 def get_neighbor_list_from_neighbor_matrix(neighbor_matrix: torch.Tensor, num_neighbors: torch.Tensor,
                                            neighbor_shift_matrix: torch.Tensor | None = None,
                                            fill_value: int | None = None):
     """Dense -> COO in row-major order.  Returns ``(edges (2,E) int32, edge_ptr (N+1) int32[,
     shifts (E,3) int32])`` like the reference's helper (the caller transposes ``[0]``).
-    Reads back one integer (the edge count) to size the output."""
+
+    The edge pointer is scanned and the edges are written on the device in one call, into buffers
+    sized by the edge count of the previous conversion of a matrix of this shape (plus headroom);
+    the host then reads the count once, to cut the views to size (tensor shapes live on the host:
+    the reference's helper waits for the same number), and repeats the call with larger buffers
+    only if they were too small."""
     N, K = neighbor_matrix.shape
     dev = neighbor_matrix.device
+    key = (dev.index, N, K)
+    guess = _last_edge_count.get(key)
+    cap = N * K if guess is None else min(N * K, int(guess * 1.05) + 1024)
+    if guess is None and N * K > (1 << 22):
+        cap = 0  # a first conversion of a large matrix: count first, rather than allocate N x K edges
     edge_ptr = torch.empty(N + 1, dtype=torch.int32, device=dev)
-    _lib.nl_edge_ptr(num_neighbors, K, edge_ptr)
-    E = int(edge_ptr[-1].item())
-    edges = torch.empty((E, 2), dtype=torch.int32, device=dev)
-    shifts = torch.empty((E, 3), dtype=torch.int32, device=dev) if neighbor_shift_matrix is not None else None
-    _lib.nl_matrix_to_coo(neighbor_matrix, neighbor_shift_matrix, edge_ptr, edges, shifts)
-    if shifts is None:
+    counts = torch.empty(2, dtype=torch.int32, device=dev)
+    want_shifts = neighbor_shift_matrix is not None
+    while True:
+        edges = torch.empty((cap, 2), dtype=torch.int32, device=dev)
+        shifts = torch.empty((cap, 3), dtype=torch.int32, device=dev) if want_shifts else None
+        _lib.nl_coo_from_matrix(neighbor_matrix, neighbor_shift_matrix, num_neighbors, edge_ptr, edges, shifts, counts)
+        E, over = (int(v) for v in counts.tolist())
+        if not over:
+            break
+        cap = E
+    _last_edge_count[key] = E
+    edges = edges[:E]
+    if not want_shifts:
         return edges.T, edge_ptr
-    return edges.T, edge_ptr, shifts
+    return edges.T, edge_ptr, shifts[:E]

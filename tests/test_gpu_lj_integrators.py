@@ -328,6 +328,42 @@ def test_matrix_to_coo_row_major():
     assert np.array_equal(nls.cpu().numpy(), sh[ii, kk])
 
 
+def test_coo_in_one_call_with_a_capacity_and_an_overflow_flag():
+    """Edge pointer, edges and the edge count in one call without a host synchronisation: buffers of the
+    caller's capacity, edges beyond it not written, the count and an overflow flag left on the device."""
+    from nvalchemi_amd import _lib
+    from nvalchemi_amd._neighbor_ops import get_neighbor_list_from_neighbor_matrix
+
+    P, C, pb, ptr = periodic_batch(92, 3, 30, 80, 0.3)
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, 3.0, 24)
+    N, K = nm.shape
+    clamped = np.minimum(nn, K)
+    E = int(clamped.sum())
+    ii, kk = np.nonzero(np.arange(K)[None, :] < clamped[:, None])
+    want_nl, want_sh = np.stack([ii, nm[ii, kk]], 1), sh[ii, kk]
+    tnm, tnn, tsh = T(nm), T(nn), T(sh)
+    for cap in (E + 100, E, E - 37, 0):
+        eptr = torch.empty(N + 1, dtype=torch.int32, device=DEV)
+        nl = torch.full((cap, 2), -1, dtype=torch.int32, device=DEV)
+        nls = torch.full((cap, 3), -9, dtype=torch.int32, device=DEV)
+        counts = torch.full((2,), -5, dtype=torch.int32, device=DEV)
+        _lib.nl_coo_from_matrix(tnm, tsh, tnn, eptr, nl, nls, counts)
+        assert counts.tolist() == [E, int(E > cap)]
+        assert np.array_equal(eptr.cpu().numpy(), np.concatenate([[0], np.cumsum(clamped)]))
+        n = min(cap, E)
+        assert np.array_equal(nl.cpu().numpy()[:n], want_nl[:n]) and np.array_equal(nls.cpu().numpy()[:n], want_sh[:n])
+        assert bool((nl[n:] == -1).all()) and bool((nls[n:] == -9).all())  # nothing written beyond
+    # the package's helper: exact shapes, whatever its first guess of the capacity was
+    for _ in range(2):
+        edges, eptr, shifts = get_neighbor_list_from_neighbor_matrix(tnm, tnn, tsh)
+        assert edges.shape == (2, E) and shifts.shape == (E, 3)
+        assert np.array_equal(edges.T.cpu().numpy(), want_nl) and np.array_equal(shifts.cpu().numpy(), want_sh)
+    # fewer edges than last time, and none at all
+    tnn2 = torch.zeros_like(tnn)
+    edges, eptr, shifts = get_neighbor_list_from_neighbor_matrix(tnm, tnn2, tsh)
+    assert edges.shape == (2, 0) and shifts.shape == (0, 3) and int(eptr[-1]) == 0
+
+
 def test_lj_row_order_changes_nothing_but_the_walk():
     """``row_order`` only permutes the order in which rows are worked on: per-atom outputs are
     bit-identical, per-system sums equal to rounding (their accumulation order differs)."""
