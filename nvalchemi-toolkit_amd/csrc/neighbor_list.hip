@@ -815,7 +815,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     __shared__ int st_prefix[kStencilBatch + 1];
     __shared__ int st_q[kStencilBatch][3];
     __shared__ float st_off[kStencilBatch][3];
-    __shared__ unsigned short hits[kWavesPerBlock][kHitCap];
+    __shared__ unsigned short hits[kWavesPerBlock][kHitCap + 2];
 
     const int total_units = ws.hdr->total_units;
     const int lane = lane_id();
@@ -1067,11 +1067,10 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         auto accept = [&](const int k, const float4& p, const float d2) {
                             const bool take = HALF ? (d2 < rc2_hi && i_atom <= __float_as_int(p.w)) : (d2 < rc2_hi);
                             const unsigned long long m = __builtin_amdgcn_ballot_w64(take);
-                            if (take) {
-                                const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
-                                                                             __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-                                my_hits[nh + before] = (unsigned short)k;
-                            }
+                            // (no branch around the store: lanes without a hit write to a slot past the list)
+                            const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                         __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                            my_hits[take ? nh + before : kHitCap] = (unsigned short)k;
                             nh += __popcll(m);
                         };
                         // Writing the list out, 64 entries a step: the self entry is dropped, an entry
@@ -1079,16 +1078,25 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         // shift and their slot.  This keeps everything but one comparison out of the
                         // per-candidate loop.
                         auto flush = [&]() {
+                            // (straight-line code: every lane reads some candidate, the lanes without an
+                            // entry read candidate 0 and drop out at the ballot; the two rare cases, a shift
+                            // too wide for its packed form and a candidate inside the band, share one branch)
                             for (int l0 = 0; l0 < nh; l0 += kWave) {
                                 const int l = l0 + lane;
-                                const int k = l < nh ? my_hits[l] : k_self;
-                                bool in = l < nh && k != k_self;
-                                int j = 0, s0 = 0, s1 = 0, s2 = 0;
-                                if (in) {
-                                    const float4 p = c_pos[k];
-                                    j = __float_as_int(p.w);
-                                    candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
-                                    if (!(dist2(p) < rc2_lo)) {  // inside the band: decide exactly
+                                const int k_read = my_hits[l < nh ? l : 0];
+                                bool in = l < nh && k_read != k_self;
+                                const int k = in ? k_read : 0;
+                                const float4 p = c_pos[k];
+                                const int pk = c_pk[k];
+                                const int j = __float_as_int(p.w);
+                                int s0 = (pk & 1023) - 512 + wi0;
+                                int s1 = ((pk >> 10) & 1023) - 512 + wi1;
+                                int s2 = ((pk >> 20) & 1023) - 512 + wi2;
+                                const bool wide = (pk & kPackOverflow) != 0;
+                                const bool band = !(dist2(p) < rc2_lo);
+                                if (__builtin_expect(__builtin_amdgcn_ballot_w64(in && (wide || band)) != 0, 0)) {
+                                    if (in && wide) candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
+                                    if (in && band) {  // inside the band: decide exactly
                                         // (the type of the positions is a compile-time matter here: looking at it
                                         // at run time costs the float32 kernel registers it does not have)
                                         Pos3 pi, pj;
@@ -1105,19 +1113,17 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                         in = pair_d2_exact(pi.x, pi.y, pi.z, pj.x, pj.y, pj.z, s0, s1, s2,
                                                            ws.sys[sidx].h, e0, e1d, e2d) < a.rc2;
                                     }
-                                    if (HALF && in) in = half_keep(i_atom, j, s0, s1, s2);
                                 }
+                                if (HALF) in = in && half_keep(i_atom, j, s0, s1, s2);
                                 const unsigned long long m = __builtin_amdgcn_ballot_w64(in);
-                                if (in) {
-                                    const int slot = base + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
-                                                                                      __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
-                                    if (slot < a.K) {
-                                        row[slot] = j;
-                                        if (srow) {
-                                            srow[3 * slot + 0] = s0;
-                                            srow[3 * slot + 1] = s1;
-                                            srow[3 * slot + 2] = s2;
-                                        }
+                                const int slot = base + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
+                                                                                  __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                if (in && slot < a.K) {
+                                    row[slot] = j;
+                                    if (srow) {
+                                        srow[3 * slot + 0] = s0;
+                                        srow[3 * slot + 1] = s1;
+                                        srow[3 * slot + 2] = s2;
                                     }
                                 }
                                 base += __popcll(m);
@@ -1134,10 +1140,10 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             const float da = dist2(pa), db = dist2(pb), dc = dist2(pc), dd = dist2(pd);
                             accept(k, pa, da);
                             accept(k + kWave, pb, db);
-                            if (nh > kHitCap - 3 * kWave) flush();
+                            if (__builtin_expect(nh > kHitCap - 3 * kWave, 0)) flush();
                             accept(k + 2 * kWave, pc, dc);
                             accept(k + 3 * kWave, pd, dd);
-                            if (nh > kHitCap - 3 * kWave) flush();
+                            if (__builtin_expect(nh > kHitCap - 3 * kWave, 0)) flush();
                         }
                         for (; k0 + kWave < k_hi; k0 += 2 * kWave) {
                             const int k = k0 + lane;
@@ -1145,7 +1151,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             const float da = dist2(pa), db = dist2(pb);
                             accept(k, pa, da);
                             accept(k + kWave, pb, db);
-                            if (nh > kHitCap - 3 * kWave) flush();
+                            if (__builtin_expect(nh > kHitCap - 3 * kWave, 0)) flush();
                         }
                         if (k0 < k_hi) {
                             const int k = k0 + lane;
