@@ -33,10 +33,10 @@ constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kTile = 1088;       // candidates staged in LDS at a time
 constexpr int kStencilBatch = 64; // stencil cells enumerated at a time (one per lane of a wave)
-constexpr int kCenterChunk = 96;  // centre atoms of a run of cells handled per pass
+constexpr int kCenterChunk = 72;  // centre atoms of a run of cells handled per pass
 constexpr int kMaxRun = 4;        // a workgroup's unit of work: up to this many cells in a row along z
-constexpr int kHitCap = 320;      // per-wave list of accepted candidates before it is written out
-constexpr int kPackOverflow = 1 << 30;
+constexpr int kHitCap = 256;      // per-wave list of accepted candidates before it is written out
+constexpr int kPackOverflow = 1 << 15;
 static_assert(kMaxRun <= 4, "a centre atom's place in its run is kept in two bits");
 constexpr int kMaxCellsPerAxis = 1024;
 static_assert(kMaxCellsPerAxis <= 1024, "a search unit's cell coordinates are packed 10 bits each");
@@ -51,6 +51,7 @@ struct NlSys {
     double ext[3];     // its length (1 on periodic axes)
     double step[9];    // row d = (ext[d]/nc[d]) * h[d,:] : one cell step along axis d
     float tol;         // relative half-width of the float32 uncertainty band on d^2
+    float tol_scan;    // the same for the expanded form |q|^2 - 2 p.q + |p|^2 that the candidate scan evaluates
     int nc[3];
     int R[3];
     int per[3];
@@ -66,6 +67,7 @@ struct NlSys {
 struct NlSearchSys {
     float step[9];  // cell step vectors, row d = one cell along axis d
     float tol;      // relative half-width of the float32 uncertainty band on d^2
+    float tol_scan; // the same for the expanded form of the candidate scan (wider: its terms are as large as reach^2)
     int nc[3];
     int R[3];
     int per[3];
@@ -335,12 +337,16 @@ __device__ __forceinline__ void choose_grid(NlSys& s, const NlArgs& a, const uin
     // largest cell-local coordinate the search can meet
     const double reach = (s.R[0] + 1) * len[0] + (s.R[1] + 1) * len[1] + (s.R[2] + zr) * len[2];
     s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
+    // |q|^2 - 2 p.q against rc^2 - |p|^2 in float32: ten roundings of terms no larger than 3 reach^2
+    // (three for |q|^2, three fused multiply-adds, four for the threshold), 2^-24 relative each
+    s.tol_scan = (float)((double)s.tol + 1.6e-6 * (reach / a.rc) * (reach / a.rc));
 }
 
 __device__ __forceinline__ NlSearchSys search_view(const NlSys& s) {
     NlSearchSys q;
     for (int k = 0; k < 9; ++k) q.step[k] = (float)s.step[k];
     q.tol = s.tol;
+    q.tol_scan = s.tol_scan;
     for (int d = 0; d < 3; ++d) {
         q.nc[d] = s.nc[d];
         q.R[d] = s.R[d];
@@ -748,10 +754,10 @@ __device__ __forceinline__ bool half_keep(int i, int j, int s0, int s1, int s2) 
 }
 
 __device__ __forceinline__ int pack_shift(int x, int y, int z) {
-    // three signed 10-bit fields; anything wider is flagged and recovered from global memory
-    if ((unsigned)(x + 512) > 1023u || (unsigned)(y + 512) > 1023u || (unsigned)(z + 512) > 1023u)
+    // three signed 5-bit fields; anything wider is flagged and recovered from global memory
+    if ((unsigned)(x + 16) > 31u || (unsigned)(y + 16) > 31u || (unsigned)(z + 16) > 31u)
         return kPackOverflow;
-    return (x + 512) | ((y + 512) << 10) | ((z + 512) << 20);
+    return (x + 16) | ((y + 16) << 5) | ((z + 16) << 10);
 }
 
 __device__ __forceinline__ float uniform_f(float v) {
@@ -761,7 +767,7 @@ __device__ __forceinline__ float uniform_f(float v) {
 // Shift of candidate k relative to the centre atom: packed fast path, or (wide shifts) recovered
 // from the sorted arrays through the stencil tables of the current batch.
 struct ShiftSource {
-    const int* c_pk;
+    const unsigned short* c_pk;
     const int* st_prefix;
     const int* st_start;
     const int (*st_q)[3];
@@ -783,9 +789,9 @@ __device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, i
         s1 = src.st_q[lo][1] - w.y + wi1;
         s2 = src.st_q[lo][2] - w.z + wi2;
     } else {
-        s0 = (pk & 1023) - 512 + wi0;
-        s1 = ((pk >> 10) & 1023) - 512 + wi1;
-        s2 = ((pk >> 20) & 1023) - 512 + wi2;
+        s0 = (pk & 31) - 16 + wi0;
+        s1 = ((pk >> 5) & 31) - 16 + wi1;
+        s2 = ((pk >> 10) & 31) - 16 + wi2;
     }
 }
 
@@ -804,8 +810,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                                               const NlUnit* __restrict__ units_ro,
                                                               const NlSearchSys* __restrict__ ssys_ro,
                                                               const int* __restrict__ cell_start_ro) {
-    __shared__ float4 c_pos[kTile];           // candidate: xyz relative to the run's first cell + atom index
-    __shared__ int c_pk[kTile];               // packed (image of its cell - its own wrap)
+    __shared__ float4 c_pos[kTile];           // candidate: xyz relative to the run's first cell, and |xyz|^2
+    __shared__ int c_j[kTile];                // its atom index
+    __shared__ unsigned short c_pk[kTile];    // packed (image of its cell - its own wrap)
     __shared__ float4 ca_pos[kCenterChunk];   // centre atoms of this pass: same frame + atom index
     __shared__ int4 ca_w[kCenterChunk];       // their wrap integers; .w = place of their cell in the run
     __shared__ int ca_pad[kCenterChunk];      // slot up to which their row has to be padded afterwards
@@ -863,7 +870,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         // one batch of stencil cells and (checked below) one tile: rows are finished in place and
         // every centre atom scans only the layers of its own cell's stencil
         const bool one_batch = n_stencil <= kStencilBatch;
-        const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol);
+        const float rc2_lo = rc2f * (1.0f - S.tol), rc2_hi = rc2f * (1.0f + S.tol), rc2_scan = rc2f * (1.0f + S.tol_scan);
         // (square cells never have a stencil cell out of reach: the test is skipped for them)
         const bool may_cull = S.cull_far > cull_reach + 2.0f * S.half_diag;
         // One batch of stencil cells: the last wave enumerates up to 64 of them, one per lane, and scans
@@ -1016,14 +1023,16 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                 p.x += st_off[e][0];
                                 p.y += st_off[e][1];
                                 p.z += st_off[e][2];
+                                c_j[f] = __float_as_int(p.w);
+                                p.w = p.x * p.x + p.y * p.y + p.z * p.z;
                                 c_pos[f] = p;
-                                c_pk[f] = pack_shift(st_q[e][0] - sw[i].x, st_q[e][1] - sw[i].y, st_q[e][2] - sw[i].z);
+                                c_pk[f] = (unsigned short)pack_shift(st_q[e][0] - sw[i].x, st_q[e][1] - sw[i].y, st_q[e][2] - sw[i].z);
                             }
                         }
                     }
                     // padding up to a multiple of 64: candidates that no centre atom can reach
                     if ((int)threadIdx.x < tile_pad - tile_n)
-                        c_pos[tile_n + threadIdx.x] = make_float4(3.0e38f, 0.f, 0.f, __int_as_float(-1));
+                        c_pos[tile_n + threadIdx.x] = make_float4(0.f, 0.f, 0.f, 3.0e38f);
                     // Every load above has landed before the centre loop starts (vmcnt(0)): otherwise
                     // the loop would begin each turn with a wait on "the loads that may still be in
                     // flight", which, the counter being in-order, waits for the previous centre
@@ -1038,7 +1047,10 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                     for (int ca = wave; ca < n_cc; ca += kWavesPerBlock) {
                         const float4 ci = ca_pos[ca];
                         const int4 wa = ca_w[ca];
-                        const float xi = uniform_f(ci.x), yi = uniform_f(ci.y), zi = uniform_f(ci.z);
+                        // The scan evaluates |q|^2 - 2 p.q against rc^2 - |p|^2: three fused multiply-adds and a
+                        // comparison per candidate, with |q|^2 staged beside q.  (-2 p is kept; p = -0.5 (-2 p) exactly.)
+                        const float mx = uniform_f(-2.0f * ci.x), my = uniform_f(-2.0f * ci.y), mz = uniform_f(-2.0f * ci.z);
+                        const float scan_lim = uniform_f(rc2_scan - (ci.x * ci.x + ci.y * ci.y + ci.z * ci.z));
                         const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ci.w));
                         const int wi0 = __builtin_amdgcn_readfirstlane(wa.x);
                         const int wi1 = __builtin_amdgcn_readfirstlane(wa.y);
@@ -1060,12 +1072,13 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         // is inside the outer edge of the float32 uncertainty band goes to the wave's hit
                         // list.  The list is a superset: it still holds the centre atom itself (distance 0)
                         // and the few candidates inside the band.
+                        auto scan_form = [&](const float4& p) { return fmaf(p.z, mz, fmaf(p.y, my, fmaf(p.x, mx, p.w))); };
                         auto dist2 = [&](const float4& p) {
-                            const float dx = p.x - xi, dy = p.y - yi, dz = p.z - zi;
+                            const float dx = fmaf(mx, 0.5f, p.x), dy = fmaf(my, 0.5f, p.y), dz = fmaf(mz, 0.5f, p.z);
                             return dx * dx + dy * dy + dz * dz;
                         };
-                        auto accept = [&](const int k, const float4& p, const float d2) {
-                            const bool take = HALF ? (d2 < rc2_hi && i_atom <= __float_as_int(p.w)) : (d2 < rc2_hi);
+                        auto accept = [&](const int k, const float4& p, const float t) {
+                            const bool take = t < scan_lim;
                             const unsigned long long m = __builtin_amdgcn_ballot_w64(take);
                             // (no branch around the store: lanes without a hit write to a slot past the list)
                             const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
@@ -1088,12 +1101,14 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                 const int k = in ? k_read : 0;
                                 const float4 p = c_pos[k];
                                 const int pk = c_pk[k];
-                                const int j = __float_as_int(p.w);
-                                int s0 = (pk & 1023) - 512 + wi0;
-                                int s1 = ((pk >> 10) & 1023) - 512 + wi1;
-                                int s2 = ((pk >> 20) & 1023) - 512 + wi2;
+                                const int j = c_j[k];
+                                int s0 = (pk & 31) - 16 + wi0;
+                                int s1 = ((pk >> 5) & 31) - 16 + wi1;
+                                int s2 = ((pk >> 10) & 31) - 16 + wi2;
                                 const bool wide = (pk & kPackOverflow) != 0;
-                                const bool band = !(dist2(p) < rc2_lo);
+                                const float d2 = dist2(p);
+                                in = in && d2 < rc2_hi;  // (the scan's form lets a few more through than this one)
+                                const bool band = !(d2 < rc2_lo);
                                 if (__builtin_expect(__builtin_amdgcn_ballot_w64(in && (wide || band)) != 0, 0)) {
                                     if (in && wide) candidate_shift(shifts, k, wi0, wi1, wi2, s0, s1, s2);
                                     if (in && band) {  // inside the band: decide exactly
@@ -1137,26 +1152,26 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             const int k = k0 + lane;
                             const float4 pa = c_pos[k], pb = c_pos[k + kWave], pc = c_pos[k + 2 * kWave],
                                          pd = c_pos[k + 3 * kWave];
-                            const float da = dist2(pa), db = dist2(pb), dc = dist2(pc), dd = dist2(pd);
+                            const float da = scan_form(pa), db = scan_form(pb), dc = scan_form(pc), dd = scan_form(pd);
                             accept(k, pa, da);
                             accept(k + kWave, pb, db);
-                            if (__builtin_expect(nh > kHitCap - 3 * kWave, 0)) flush();
+                            if (__builtin_expect(nh > kHitCap - 2 * kWave, 0)) flush();
                             accept(k + 2 * kWave, pc, dc);
                             accept(k + 3 * kWave, pd, dd);
-                            if (__builtin_expect(nh > kHitCap - 3 * kWave, 0)) flush();
+                            if (__builtin_expect(nh > kHitCap - 2 * kWave, 0)) flush();
                         }
                         for (; k0 + kWave < k_hi; k0 += 2 * kWave) {
                             const int k = k0 + lane;
                             const float4 pa = c_pos[k], pb = c_pos[k + kWave];
-                            const float da = dist2(pa), db = dist2(pb);
+                            const float da = scan_form(pa), db = scan_form(pb);
                             accept(k, pa, da);
                             accept(k + kWave, pb, db);
-                            if (__builtin_expect(nh > kHitCap - 3 * kWave, 0)) flush();
+                            if (__builtin_expect(nh > kHitCap - 2 * kWave, 0)) flush();
                         }
                         if (k0 < k_hi) {
                             const int k = k0 + lane;
                             const float4 pa = c_pos[k];
-                            accept(k, pa, dist2(pa));
+                            accept(k, pa, scan_form(pa));
                         }
                         flush();
                         if (fused) {

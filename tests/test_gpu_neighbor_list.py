@@ -129,6 +129,25 @@ def test_tiny_cell_many_images_and_self_images():
     check_against_oracle(P, C, np.ones((1, 3), bool), [0, 3], 4.5)
 
 
+def test_atoms_many_cells_away_take_the_unpacked_shift_path():
+    """Shifts travel through the search as three 5-bit fields; an atom that sits 20 to 40 cell lengths
+    outside its cell has a wider one, which is recovered from the sorted arrays instead.  (Multiples of
+    lattice vectors that float32 adds exactly: edge lengths are powers of two.)"""
+    rng = np.random.default_rng(5)
+    counts = [40, 70]
+    C = np.stack([np.diag([8.0, 8.0, 16.0]), np.array([[8.0, 0, 0], [2.0, 8.0, 0], [0, 4.0, 16.0]])]).astype(np.float32)
+    pos = []
+    for n, H in zip(counts, C):
+        f = rng.uniform(0, 1, (n, 3))
+        hop = rng.integers(-40, 41, (n, 3)) * (rng.random((n, 1)) < 0.5)
+        pos.append(((f + hop) @ H.astype(np.float64)).astype(np.float32))
+    P = np.concatenate(pos)
+    pb = np.ones((2, 3), bool)
+    nm, nn, sh = check_against_oracle(P, C, pb, ptr_from_counts(counts), 5.0)
+    assert int(sh.abs().max()) > 15
+    check_against_oracle(P, C, pb, ptr_from_counts(counts), 5.0, half=True)
+
+
 def test_empty_systems_and_single_atoms():
     pos = np.array([[0.0, 0, 0], [1.0, 0, 0], [9.0, 9, 9]], dtype=np.float32)
     check_against_oracle(pos, None, None, ptr_from_counts([0, 2, 0, 1]), 2.0, K=4)
