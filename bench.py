@@ -47,8 +47,8 @@ RELAX_MAXSTEP = 0.07
 # half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
 # bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
 MEASURED_TRAFFIC_BYTES = {
-    "nl": 1024 * (2 * (31564 + 8505) + (842239 + 77044)),   # search + per-system sort
-    "lj": 1024 * (2 * (166384 + 2473) + 15722 + 57),        # pair kernel + system ranges
+    "nl": 1024 * (2 * (47952 + 7603) + (874851 + 68510)),   # search + per-system sort
+    "lj": 1024 * (2 * (166404 + 2473) + 15722 + 57),        # pair kernel + system ranges
 }
 
 

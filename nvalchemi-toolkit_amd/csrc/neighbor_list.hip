@@ -1049,7 +1049,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         const int4 wa = ca_w[ca];
                         // The scan evaluates |q|^2 - 2 p.q against rc^2 - |p|^2: three fused multiply-adds and a
                         // comparison per candidate, with |q|^2 staged beside q.  (-2 p is kept; p = -0.5 (-2 p) exactly.)
-                        const float mx = uniform_f(-2.0f * ci.x), my = uniform_f(-2.0f * ci.y), mz = uniform_f(-2.0f * ci.z);
+                        float m2x = -2.0f * ci.x, m2y = -2.0f * ci.y, m2z = -2.0f * ci.z;
+                        asm volatile("" : "+v"(m2x), "+v"(m2y), "+v"(m2z));  // (so that the products, not ci, go to scalar registers)
+                        const float mx = uniform_f(m2x), my = uniform_f(m2y), mz = uniform_f(m2z);
                         const float scan_lim = uniform_f(rc2_scan - (ci.x * ci.x + ci.y * ci.y + ci.z * ci.z));
                         const int i_atom = __builtin_amdgcn_readfirstlane(__float_as_int(ci.w));
                         const int wi0 = __builtin_amdgcn_readfirstlane(wa.x);
