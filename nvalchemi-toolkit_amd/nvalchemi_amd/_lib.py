@@ -113,7 +113,15 @@ def _check(rc: int, what: str) -> None:
         raise KernelLibraryError(f"{what} failed with code {rc}: {msg}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device: torch.device) -> int:
+    """The current stream of ``device`` as a raw handle (without building a ``torch.cuda.Stream`` object
+    where Torch offers the direct call: six of these per MD step)."""
+    if _raw_stream is not None:
+        index = device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -130,7 +138,14 @@ def _dev(t: torch.Tensor, name: str, dtype: torch.dtype, shape: tuple | None = N
     if not t.is_contiguous():
         raise ValueError(f"{name}: tensor must be contiguous")
     if shape is not None:
-        if t.dim() != len(shape) or any(e is not None and int(s) != int(e) for s, e in zip(t.shape, shape)):
+        got = t.shape
+        ok = len(got) == len(shape)
+        if ok:
+            for s, e in zip(got, shape):
+                if e is not None and s != e:
+                    ok = False
+                    break
+        if not ok:
             raise ValueError(f"{name}: expected shape {shape}, got {tuple(t.shape)}")
     return t.data_ptr()
 
