@@ -148,6 +148,30 @@ def test_atoms_many_cells_away_take_the_unpacked_shift_path():
     check_against_oracle(P, C, pb, ptr_from_counts(counts), 5.0, half=True)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_pairs_within_a_hair_of_the_cutoff(seed):
+    """Pairs placed at rc (1 +- 10^-7.5 .. 10^-4) in cells from a fraction of the cutoff to six cutoffs wide,
+    skewed or not, atoms up to two cells outside: every one of them lies inside one of the float32 uncertainty
+    bands of the search (the scan's expanded form has the wider one) and has to come out as the double-precision
+    expression on the float32 inputs decides."""
+    rng = np.random.default_rng(7000 + seed)
+    rc = float(rng.choice([1.0, 2.5, 5.0]))
+    L = rc * rng.uniform(0.6, 6.0, 3)
+    H = np.diag(L)
+    if rng.random() < 0.7:
+        H[1, 0] = rng.uniform(-0.5, 0.5) * L[0]
+        H[2, 0] = rng.uniform(-0.5, 0.5) * L[0]
+        H[2, 1] = rng.uniform(-0.5, 0.5) * L[1]
+    n_pairs = int(rng.integers(20, 120))
+    base = rng.uniform(-1.0, 2.0, (n_pairs, 3)) @ H
+    dirs = rng.normal(size=(n_pairs, 3))
+    dirs /= np.linalg.norm(dirs, axis=1, keepdims=True)
+    eps = 10.0 ** rng.uniform(-7.5, -4.0, n_pairs) * rng.choice([-1.0, 1.0], n_pairs)
+    P = np.concatenate([base, base + dirs * (rc * (1.0 + eps))[:, None]]).astype(np.float32)
+    pb = (rng.random(3) < 0.8)[None]
+    check_against_oracle(P, H.astype(np.float32)[None], pb, ptr_from_counts([len(P)]), rc)
+
+
 def test_empty_systems_and_single_atoms():
     pos = np.array([[0.0, 0, 0], [1.0, 0, 0], [9.0, 9, 9]], dtype=np.float32)
     check_against_oracle(pos, None, None, ptr_from_counts([0, 2, 0, 1]), 2.0, K=4)
