@@ -289,17 +289,40 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 if (k >= cnt) jj[u] = -1;
             }
             }
+            if (LDS_POS) {
+                // every lane reads the stage (a neighbor outside the staged span reads the span's first atom for
+                // now); the lanes with such a neighbor, if there are any at all, fetch it from memory afterwards
+                unsigned outside = 0;
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const bool ok = jj[u] >= 0 && jj[u] < a.fill;
-                const int j = ok ? jj[u] : i;
-                if (!ok) jj[u] = -1;
-                const unsigned rel = (unsigned)(j - span0);
-                if (LDS_POS && rel < (unsigned)span_n) {
-                    xj[u] = s_pos[3 * rel + 0];
-                    yj[u] = s_pos[3 * rel + 1];
-                    zj[u] = s_pos[3 * rel + 2];
-                } else {
+                for (int u = 0; u < UNROLL; ++u) {
+                    const bool ok = jj[u] >= 0 && jj[u] < a.fill;
+                    const int j = ok ? jj[u] : i;
+                    if (!ok) jj[u] = -1;
+                    const unsigned rel = (unsigned)(j - span0);
+                    const bool in_span = rel < (unsigned)span_n;
+                    outside |= in_span ? 0u : (1u << u);
+                    const unsigned at = in_span ? rel : 0u;
+                    xj[u] = s_pos[3 * at + 0];
+                    yj[u] = s_pos[3 * at + 1];
+                    zj[u] = s_pos[3 * at + 2];
+                }
+                if (__builtin_expect(__builtin_amdgcn_ballot_w64(outside != 0) != 0, 0)) {
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) {
+                        if (outside & (1u << u)) {
+                            const float* pj = a.pos + 3 * (size_t)(jj[u] >= 0 ? jj[u] : i);
+                            xj[u] = pj[0];
+                            yj[u] = pj[1];
+                            zj[u] = pj[2];
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const bool ok = jj[u] >= 0 && jj[u] < a.fill;
+                    const int j = ok ? jj[u] : i;
+                    if (!ok) jj[u] = -1;
                     const float* pj = a.pos + 3 * (size_t)j;
                     xj[u] = pj[0];
                     yj[u] = pj[1];

@@ -79,6 +79,37 @@ def test_lj_full_list_matches_oracle(name, kw, rc, eps, sig, virial):
     assert_close(got, ref, name)
 
 
+def test_lj_neighbors_outside_the_rows_own_system_are_fetched_from_memory():
+    """The pair kernel stages the positions of the system whose rows it works on; an index that points into
+    another system (no list of this package holds one, a caller's own list may) is not in the stage and has
+    to be gathered from memory with the same result as the oracle, which knows nothing of stages."""
+    P, C, pb, ptr = periodic_batch(57, 3, 200, 400, 0.8)
+    bi = oracle.batch_idx_from_ptr(ptr)
+    rc = 2.5
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, rc, 8)
+    K = int(nn.max()) + 2
+    nm, nn, sh = oracle.nl_cell(P, C, pb, ptr, rc, K)
+    rng = np.random.default_rng(3)
+    N = len(P)
+    touched = 0
+    for i in rng.choice(N, 60, replace=False):
+        if nn[i] == 0:
+            continue
+        k = int(rng.integers(0, nn[i]))
+        others = np.flatnonzero(bi != bi[i])
+        # an atom of another system that happens to lie within the cutoff of atom i, taken without a shift
+        d = np.linalg.norm(P[others].astype(np.float64) - P[i].astype(np.float64), axis=1)
+        near = others[(d < rc) & (d > 0.7)]
+        if len(near) == 0:
+            continue
+        nm[i, k] = near[0]
+        sh[i, k] = 0
+        touched += 1
+    assert touched > 10
+    ref = oracle.lj_matrix(P, C, nm, sh, nn, bi, N, 1.0, 1.0, rc)
+    assert_close(gpu_lj(P, C, nm, sh, nn, bi, 1.0, 1.0, rc), ref, "neighbors in other systems")
+
+
 @pytest.mark.parametrize("lpr", ["8", "16", "32", "64"])
 def test_lj_all_row_widths(lpr, monkeypatch):
     # the row-ownership width is chosen once per process; exercise every variant through K
