@@ -48,8 +48,8 @@ RELAX_MAXSTEP = 0.07
 # half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
 # bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
 MEASURED_TRAFFIC_BYTES = {
-    "nl": 1024 * (2 * (47952 + 7603) + (874851 + 68510)),   # search + per-system sort
-    "lj": 1024 * (2 * (166404 + 2473) + 15722 + 57),        # pair kernel + system ranges
+    "nl": 1024 * (2 * (47679 + 7602) + (874855 + 68117)),   # search + per-system sort
+    "lj": 1024 * (2 * (167798 + 2473) + 15803 + 57),        # pair kernel + system ranges
 }
 
 
