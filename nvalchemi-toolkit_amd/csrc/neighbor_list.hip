@@ -13,15 +13,17 @@
 //   4 bin       per atom: wrapped fractional coordinate -> cell, rank inside the cell
 //   5 scan      exclusive scan of the histogram (three small kernels)
 //   6 scatter   counting-sort the atoms into cell order: cell-local coordinates + wrap
-//   7 search    one workgroup per cell: stage the stencil's atoms in LDS, one wavefront per
-//               centre atom, 64 candidates per step, ballot + prefix-popcount compaction
-//               into the atom's row
+//   7 search    one workgroup per run of cells along z: stage the stencil's atoms in LDS, one
+//               wavefront per centre atom, 64 candidates per step, ballot + prefix-popcount
+//               compaction into a hit list, the list written out into the atom's row
+// (batches of many small systems take 1-6 in one workgroup per system: nl_system_sort_kernel).
 //
-// Which pairs are neighbors is decided in double on the original float32 positions
-// (geom.h).  The search classifies candidates with a float32 distance on cell-local
-// coordinates whose rounding error is bounded by a per-system tolerance; only candidates
-// inside that band around the cutoff are re-evaluated exactly, so the list is independent
-// of the order of float32 operations in the fast path.
+// Which pairs are neighbors is decided in double on the original positions (geom.h).  The search
+// classifies candidates with float32 distances on cell-local coordinates whose rounding error is
+// bounded by per-system tolerances (a wider one for the three-instruction form of the scan, the
+// usual one for the direct form of the write-out); only candidates inside the band around the
+// cutoff are re-evaluated exactly, so the list is independent of the order of float32
+// operations in the fast path.
 #include "common.h"
 #include "geom.h"
 #include "scan.h"
