@@ -1,6 +1,7 @@
 """Throughput of the batched MD inner loop on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config {2,3,4,5}] [--boxes B] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--config {2,3,4,5}] [--boxes B]
+                    [--no-cpu-baseline] [--no-other-configs]
 
 Other configurations of the baseline (``--config``): 2 = 64 FCC boxes of 500 atoms, NVE; 4 = 2048
 triclinic cells of 8-2000 atoms, FIRE with per-system convergence masks; 5 = one box of 4 M atoms,
@@ -14,12 +15,16 @@ path through the package's own API: ``NVE.step`` = velocity-Verlet position upda
 ``NeighborListHook`` (cell-list build) -> ``LennardJonesModelWrapper`` (pair kernel + per-system
 energies) -> velocity finalize.  All inputs are resident in HBM when the timed region starts.
 
-Prints ONE JSON line.  ``value`` = atoms x steps / wall time of the timed region.  ``roofline``
-describes the neighbor build (the stage that dominates the step): algorithmic bytes
-20 N + 16 E per build divided by its average duration, measured with HIP events recorded on
-the stream the kernels run on, inside the timed region, on every 8th step (an event between two
-kernels costs the device about 4 us; recorded on every step they take 4.5 % off the throughput).  ``stages`` gives the same for the
-pair kernel (36 N + 16 E + 4 B) and the two velocity-Verlet halves (68 N and 44 N).
+Prints ONE JSON line.  The timed region of exactly ``--steps`` steps is run ``--repeats`` times (5) with a
+device synchronisation on both sides of each; ``value`` = atoms x steps / wall time of the region of
+median duration, and ``repeats`` lists them all.  ``roofline`` describes the neighbor build (the stage
+that dominates the step): algorithmic bytes 20 N + 16 E per build divided by its average duration,
+measured with HIP events recorded on the stream the kernels run on, inside the timed regions: at most
+every 4th step is sampled and a sampled step times one entry point, the entry points taking turns (an
+event between two kernels costs the device about 4 us; eight per step took 4.5 % off the throughput).
+``stages`` gives the same for the pair kernel (36 N + 16 E + 4 B) and the two velocity-Verlet halves
+(68 N and 44 N).  The default run appends ``other_configs``: configurations 2, 4 and 5 measured the
+same way over fewer steps.
 ``cpu_baseline`` times the CPU oracle (a port of the same algorithms, not the product) on a
 bounded sample of the same workload on this machine's host cores.
 """
@@ -137,8 +142,10 @@ def make_single_box(device, n_atoms=4_000_000, density=0.1, seed=0):
 
 
 class StageTimer:
-    """HIP events around each C-ABI entry point of a step (neighbor build, pair kernel, the two
-    velocity-Verlet halves), recorded on the stream the kernels are enqueued on."""
+    """HIP events around one C-ABI entry point of a sampled step (neighbor build, pair kernel, the two
+    velocity-Verlet halves, FIRE, fmax), recorded on the stream the kernels are enqueued on.  The entry points
+    that a configuration calls take turns from one sampled step to the next, so a sampled step carries two
+    events, not two per stage."""
 
     ENTRY = {"nl": "nl_build", "lj": "lj_energy_forces", "vv_pre": "vv_position_update",
              "vv_post": "vv_velocity_finalize", "fire": "fire_step", "fmax": "segment_fmax"}
@@ -149,14 +156,26 @@ class StageTimer:
         from nvalchemi_amd import _lib
 
         self.torch = torch
-        self.ev = {k: [] for k in self.ENTRY}
-        self.enabled = False
+        self.reset()
         for key, name in self.ENTRY.items():
             setattr(_lib, name, self._timed(getattr(_lib, name), key))
 
+    def reset(self):
+        self.ev = {k: [] for k in self.ENTRY}
+        self.seen = []      # entry points called so far, in the order of their first call
+        self.want = None    # the entry point the current step times (None: none)
+        self.turn = None
+
+    def select(self, turn):
+        """``turn``: running number of the sampled step, or None for a step that records nothing."""
+        self.turn = turn
+        self.want = None if (turn is None or not self.seen) else self.seen[turn % len(self.seen)]
+
     def _timed(self, fn, key):
         def call(*a, **k):
-            if not self.enabled:
+            if key not in self.seen:
+                self.seen.append(key)
+            if self.turn is None or self.want != key:
                 return fn(*a, **k)
             e0 = self.torch.cuda.Event(enable_timing=True)
             e1 = self.torch.cuda.Event(enable_timing=True)
@@ -233,7 +252,8 @@ def setup_config(cfg: int, args, device):
             model.model_config.neighbor_config.skin = args.skin
         dyn = NVE(model, dt=dt * fs, hooks=model.make_neighbor_hooks())
         what = (f"{batch.num_graphs} periodic LJ-liquid boxes x {n_per_box} atoms, rho=0.8, rc=2.5 sigma, "
-                f"{args.relax_steps} FIRE steps then NVE dt=0.005, "
+                f"{args.relax_steps} FIRE steps (relaxation maxstep {RELAX_MAXSTEP} sigma, not the FIRE default of 0.2) "
+                "then NVE dt=0.005, "
                 + ("neighbor rebuild every step" if args.skin <= 0.0 else
                    f"Verlet skin {args.skin} sigma (rebuild when an atom has moved skin/2)"))
         return batch, dyn, what
@@ -270,63 +290,45 @@ def setup_config(cfg: int, args, device):
     raise ValueError(f"unknown configuration {cfg}")
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None)
-    ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", type=int, default=3, choices=(2, 3, 4, 5),
-                    help="BASELINE configuration (3 = the 1M-atom liquid the metric is quoted on)")
-    ap.add_argument("--boxes", type=int, default=256, help="configuration 3: number of 3900-atom boxes (256 = the quoted workload)")
-    ap.add_argument("--relax-steps", type=int, default=50)
-    ap.add_argument("--skin", type=float, default=0.0,
-                    help="configuration 3: Verlet skin of the neighbor hook (0 = rebuild every step, the quoted workload)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-stage-events", action="store_true", help="do not record per-stage HIP events")
-    ap.add_argument("--stage-every", type=int, default=None,
-                    help="record the per-stage HIP events on every n-th timed step (an event between two kernels "
-                         "costs the device about 4 us: on every step, 4.5 %% of the quoted workload's step); "
-                         "default: about 25 sampled steps, every 8th at most")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        return 2
-    if args.steps is None:
-        args.steps = 30 if args.config == 5 else 200
-    if args.warmup is None:
-        args.warmup = 5 if args.config == 5 else 20
-
-    import numpy as np
+def measure(cfg: int, args, dev, steps: int, warmup: int, repeats: int, timer, with_cpu_baseline: bool):
+    """One configuration: set-up, ``warmup`` untimed steps, then ``repeats`` timed regions of exactly ``steps``
+    steps each (a device synchronisation on both sides of every region).  The region of median duration is the one
+    reported; the others are listed beside it."""
     import torch
 
-    from nvalchemi_amd import _lib
-
-    if not torch.cuda.is_available():
-        print("bench.py needs a ROCm device", file=sys.stderr)
-        return 2
-    _lib.library()  # fail loudly if the HIP library is missing
-    dev = torch.device("cuda:0")
-    batch, dyn, what = setup_config(args.config, args, dev)
+    batch, dyn, what = setup_config(cfg, args, dev)
     N, B = batch.num_nodes, batch.num_graphs
-    log(f"[bench] configuration {args.config}: N={N} B={B}")
-
-    timer = None if args.no_stage_events else StageTimer()
-    for _ in range(args.warmup):
-        dyn.step(batch)
-    torch.cuda.synchronize()
-    stage_every = max(1, args.stage_every) if args.stage_every else max(1, min(8, args.steps // 25))
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        if timer:
-            timer.enabled = i % stage_every == 0
-        dyn.step(batch)
-    host = time.perf_counter() - t0  # what the host needed to enqueue the steps (the device may lag behind it)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    log(f"[bench] host enqueued {args.steps} steps in {host / args.steps * 1e3:.3f} ms/step; with the device: "
-        f"{wall / args.steps * 1e3:.3f} ms/step")
+    log(f"[bench] configuration {cfg}: N={N} B={B}")
     if timer:
-        timer.enabled = False
+        timer.reset()
+    for _ in range(warmup):
+        dyn.step(batch)
+    torch.cuda.synchronize()
+    # Per-stage HIP events: a sampled step times ONE entry point (they take turns), and at most every 4th step is
+    # sampled, because an event between two kernels costs the device about 4 us.
+    stage_every = max(1, args.stage_every) if args.stage_every else (8 if steps >= 32 else 4 if steps >= 8 else 1)
+    walls, hosts = [], []
+    sampled = 0
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            if timer:
+                take = i % stage_every == 0
+                timer.select(sampled if take else None)
+                sampled += 1 if take else 0
+            dyn.step(batch)
+        hosts.append(time.perf_counter() - t0)  # what the host needed to enqueue the steps (the device may lag behind it)
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+    if timer:
+        timer.select(None)
+    order = sorted(range(repeats), key=lambda r: walls[r])
+    wall = walls[order[repeats // 2]]
+    host = hosts[order[repeats // 2]]
+    log(f"[bench] host enqueued {steps} steps in {host / steps * 1e3:.3f} ms/step; with the device: "
+        f"{wall / steps * 1e3:.3f} ms/step (median of {repeats}: "
+        + ", ".join(f"{w / steps * 1e3:.3f}" for w in walls) + ")")
 
     nn = batch.num_neighbors
     K = batch.neighbor_matrix.shape[1]
@@ -336,9 +338,9 @@ def main() -> int:
     log(f"[bench] E={E} ({E / N:.1f}/atom, max {int(nn.max())}, K={K}); PE/atom={float(batch.energy.sum()) / N:.3f} "
         f"KE/atom={ke / N:.3f} finite={finite}")
 
-    ms_per_step = wall / args.steps * 1e3
-    value = N * args.steps / wall
-    quoted = args.config == 3 and B == 256 and args.relax_steps == 50 and args.skin <= 0.0
+    ms_per_step = wall / steps * 1e3
+    value = N * steps / wall
+    quoted = cfg == 3 and B == 256 and args.relax_steps == 50 and args.skin <= 0.0
     stages = {}
     if timer:
         ms = timer.mean_ms()
@@ -356,7 +358,7 @@ def main() -> int:
                 continue
             gbps = b / (ms[k] * 1e-3) / 1e9
             stages[k] = {"ms": round(ms[k], 4), "alg_bytes": b, "GBps": round(gbps, 1),
-                         "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+                         "frac": round(gbps / HBM_PEAK_GBPS, 4), "samples": len(timer.ev[k])}
         lj = stages["lj"]
         tflops = LJ_FP64_FLOPS_PER_PAIR * E / (ms["lj"] * 1e-3) / 1e12
         lj["fp64_flops_per_pair"] = LJ_FP64_FLOPS_PER_PAIR
@@ -374,35 +376,10 @@ def main() -> int:
             lj["bound"] = "fp64 vector arithmetic"
         log("[bench] stage ms: " + ", ".join(f"{k}={v['ms']}" for k, v in stages.items())
             + f"; sum={sum(v['ms'] for v in stages.values()):.3f} vs wall/step={ms_per_step:.3f}")
-    result = {
-        "metric": "atom-steps/s",
-        "value": value,
-        "unit": "atom-steps/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": what, "baseline_config": args.config,
-                   "n_atoms": N, "n_systems": B, "edges": E, "max_neighbors": K, "seed": 0},
-        "edges_per_s": (E / (stages["nl"]["ms"] * 1e-3)) if stages else None,
-    }
-    if stages:
-        nl = stages["nl"]
-        result["roofline"] = {"bound": "hbm", "achieved": nl["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                              "frac": nl["frac"],
-                              "traffic": MEASURED_TRAFFIC_BYTES["nl"] if quoted else None,
-                              "traffic_source": ("profiles/hbm_traffic_lj_liquid_1M.txt: rocprofv3 --pmc FETCH_SIZE and "
-                                                 "WRITE_SIZE runs of this command, not measured in this run") if quoted else None,
-                              "kernel": "neighbor build (nvamd_nl_build)",
-                              "alg_bytes_per_launch": nl["alg_bytes"], "ms_per_launch": nl["ms"]}
-        result["stages"] = stages
-        result["stage_events"] = {"sampled_steps": len(timer.ev["nl"]), "every": stage_every}
-    if not args.no_cpu_baseline and args.config == 3:
+    out = {"value": value, "ms_per_step": ms_per_step, "what": what, "N": N, "B": B, "E": E, "K": K,
+           "stages": stages, "quoted": quoted, "stage_every": stage_every, "sampled_steps": sampled,
+           "repeat_ms_per_step": [round(w / steps * 1e3, 5) for w in walls], "finite": finite}
+    if with_cpu_baseline and cfg == 3:
         # about ten seconds of host work: 32 boxes, 20 steps on one thread, then on the box's share of cores
         n_per_box = 3900
         sample_boxes, cpu_steps = min(B, 32), 20
@@ -411,11 +388,106 @@ def main() -> int:
         v1, c1, t1 = cb["1"]
         va, ca, ta = cb["all"]
         log(f"[bench] cpu oracle: {v1:.3e} atom-steps/s on 1 thread ({t1:.1f}s), {va:.3e} on {ca} threads ({ta:.1f}s)")
-        result["cpu_baseline"] = {"value": v1, "unit": "atom-steps/s", "cores": c1, "kind": "port",
-                                  "sample": f"first {sample_boxes} boxes ({n_s} atoms) of the same workload, {cpu_steps} steps "
-                                            "(VV + cell-list build + LJ + VV), C oracle -O3",
-                                  "all_cores": {"value": va, "cores": ca,
-                                                "note": "OpenMP over systems in the neighbor build only"}}
+        out["cpu_baseline"] = {"value": v1, "unit": "atom-steps/s", "cores": c1, "kind": "port",
+                               "sample": f"first {sample_boxes} boxes ({n_s} atoms) of the same workload, {cpu_steps} steps "
+                                         "(VV + cell-list build + LJ + VV), C oracle -O3",
+                               "all_cores": {"value": va, "cores": ca,
+                                             "note": "OpenMP over systems in the neighbor build only"}}
+    del batch, dyn
+    torch.cuda.empty_cache()
+    return out
+
+
+# steps and warm-up of the configurations that ride along with the default run (kept short: the whole default
+# command stays well within a few minutes)
+OTHER_CONFIG_STEPS = {2: (100, 20), 4: (40, 10), 5: (10, 3)}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--config", type=int, default=3, choices=(2, 3, 4, 5),
+                    help="BASELINE configuration (3 = the 1M-atom liquid the metric is quoted on)")
+    ap.add_argument("--boxes", type=int, default=256, help="configuration 3: number of 3900-atom boxes (256 = the quoted workload)")
+    ap.add_argument("--relax-steps", type=int, default=50)
+    ap.add_argument("--skin", type=float, default=0.0,
+                    help="configuration 3: Verlet skin of the neighbor hook (0 = rebuild every step, the quoted workload)")
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="the timed region of exactly --steps steps is run this many times; the median one is reported")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default run only: do not append the short runs of configurations 2, 4 and 5")
+    ap.add_argument("--no-stage-events", action="store_true", help="do not record per-stage HIP events")
+    ap.add_argument("--stage-every", type=int, default=None,
+                    help="record per-stage HIP events on every n-th timed step (one entry point per sampled step, in "
+                         "turn: an event between two kernels costs the device about 4 us); default: every 8th step "
+                         "of 32 or more, every 4th of 8 or more")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+    if args.steps is None:
+        args.steps = 30 if args.config == 5 else 200
+    if args.warmup is None:
+        args.warmup = 5 if args.config == 5 else 20
+    args.repeats = max(1, args.repeats)
+
+    import torch
+
+    from nvalchemi_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm device", file=sys.stderr)
+        return 2
+    _lib.library()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    timer = None if args.no_stage_events else StageTimer()
+    m = measure(args.config, args, dev, args.steps, args.warmup, args.repeats, timer, not args.no_cpu_baseline)
+    stages = m["stages"]
+    result = {
+        "metric": "atom-steps/s",
+        "value": m["value"],
+        "unit": "atom-steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": m["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": m["what"], "baseline_config": args.config,
+                   "n_atoms": m["N"], "n_systems": m["B"], "edges": m["E"], "max_neighbors": m["K"], "seed": 0},
+        "repeats": {"n": args.repeats, "reported": "median", "ms_per_step": m["repeat_ms_per_step"]},
+        "edges_per_s": (m["E"] / (stages["nl"]["ms"] * 1e-3)) if stages else None,
+    }
+    if stages:
+        nl = stages["nl"]
+        result["roofline"] = {"bound": "hbm", "achieved": nl["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                              "frac": nl["frac"],
+                              "traffic": MEASURED_TRAFFIC_BYTES["nl"] if m["quoted"] else None,
+                              "traffic_source": ("profiles/hbm_traffic_lj_liquid_1M.txt: rocprofv3 --pmc FETCH_SIZE and "
+                                                 "WRITE_SIZE runs of this command, not measured in this run") if m["quoted"] else None,
+                              "kernel": "neighbor build (nvamd_nl_build)",
+                              "alg_bytes_per_launch": nl["alg_bytes"], "ms_per_launch": nl["ms"]}
+        result["stages"] = stages
+        result["stage_events"] = {"sampled_steps": m["sampled_steps"], "every": m["stage_every"],
+                                  "entry_points_per_sampled_step": 1}
+    if "cpu_baseline" in m:
+        result["cpu_baseline"] = m["cpu_baseline"]
+    if args.config == 3 and m["quoted"] and not args.no_other_configs:
+        # the other configurations of the baseline, shorter, same measurement (no CPU baseline)
+        others = {}
+        for cfg, (st, wu) in OTHER_CONFIG_STEPS.items():
+            o = measure(cfg, args, dev, st, wu, 3, timer, False)
+            others[str(cfg)] = {"workload": o["what"], "n_atoms": o["N"], "n_systems": o["B"], "steps": st, "warmup": wu,
+                                "ms_per_step": o["ms_per_step"], "atom_steps_per_s": o["value"],
+                                "repeat_ms_per_step": o["repeat_ms_per_step"], "stages": o["stages"],
+                                "edges": o["E"], "K": o["K"], "finite": o["finite"]}
+        result["other_configs"] = others
     print(json.dumps(result))
     return 0
 
