@@ -263,7 +263,10 @@ int32_t nvamd_segment_fmax(const float* forces, const int32_t* batch_idx, int32_
  *   Every listed pair is then closer than that; in a system whose cell has all three perpendicular widths
  *   above twice it, no pair has two listed images, the listed image is the nearest one, and the kernel
  *   derives the shift from the positions instead of reading neighbor_matrix_shifts (12 of the 16 bytes per
- *   pair).  A matrix that holds pairs beyond this cutoff makes the results wrong: pass 0 when in doubt. */
+ *   pair).  With a cutoff given, the matrix is taken to be what nvamd_nl_build wrote: in such a system the
+ *   entries below a row's count are not checked one by one for being atoms of the row's own system (reads
+ *   stay inside the arrays whatever the entries hold).  A matrix that holds pairs beyond this cutoff, or
+ *   entries of other systems or padding below the counts, makes the results wrong: pass 0 when in doubt. */
 int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells,
                                       const int32_t* neighbor_matrix,
                                       const int32_t* neighbor_matrix_shifts,

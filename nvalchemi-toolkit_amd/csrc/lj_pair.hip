@@ -94,6 +94,7 @@ __device__ __forceinline__ double group_sum(double v) {
 constexpr int kSysSlots = 8;      // consecutive systems a workgroup accumulates in LDS
 constexpr int kLdsAtoms = 4096;   // positions of this many consecutive atoms fit the LDS stage
 constexpr int kBlockFull = 512;   // workgroup size of the full-list kernel
+constexpr int kStageLoads = 12;   // loads a thread keeps in flight while it stages positions
 
 // How the images of a system's listed pairs are found.
 struct LjSysImage {
@@ -171,12 +172,14 @@ template <bool VIRIAL, bool SWITCH>
 __device__ __forceinline__ void pair_terms(const LjArgs& a, double r2, double d0, double d1, double d2, double& e,
                                            double& fx, double& fy, double& fz, double& w0, double& w1, double& w2,
                                            double& w3, double& w4, double& w5) {
+    // with q6 = (sigma^2 / r^2)^3:  u = 4 eps q6 (q6 - 1),  u'(r)/r = 4 eps q6 (6 - 12 q6) / r^2
+    // (one per-launch constant per instruction, the others are literals: nothing to move into vector registers)
     const double ir2 = reciprocal(r2);
-    double q2 = a.sig2 * ir2;
-    double q6 = q2 * q2 * q2;
-    double q12 = q6 * q6;
-    double uu = a.c4eps * (q12 - q6);
-    double gg = -(a.c24eps * (2.0 * q12 - q6)) * ir2;  // u'(r)/r
+    const double q2 = a.sig2 * ir2;
+    const double q6 = (q2 * q2) * q2;
+    const double aq = a.c4eps * q6;
+    double uu = __builtin_fma(aq, q6, -aq);
+    double gg = (aq * ir2) * __builtin_fma(q6, -12.0, 6.0);
     if (SWITCH) apply_switch(a, r2, uu, gg);
     e += 0.5 * uu;
     fx += gg * d0;
@@ -221,6 +224,10 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
             hdi[k] = uniform_double(s_diag + 3 + k);
         }
     }
+    // Images derived from the positions (IMG != 0) are only taken on the promise that the matrix is the neighbor
+    // build's own (neighbor_list_cutoff > 0): entries below a row's count are then atoms of the row's system and
+    // are not checked one by one.
+    constexpr bool TRUST = IMG != 0;
     constexpr int G = kBlockFull / LPR;
     const int g = threadIdx.x / LPR;
     const int sub = threadIdx.x % LPR;
@@ -247,6 +254,9 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
         for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
             int jj[UNROLL], s0[UNROLL], s1[UNROLL], s2[UNROLL];
             float xj[UNROLL], yj[UNROLL], zj[UNROLL];
+            // TRUST: entry u of this lane's chunk is a listed pair iff u < n_mine (the other entries are kept
+            // out by this number alone: their indices are never looked at)
+            const int n_mine = VEC ? cnt - (k0 + UNROLL * sub) : (cnt - k0 - sub + LPR - 1) / LPR;
             if (VEC) {
                 // each lane owns four consecutive entries: one 16-byte load of indices and three
                 // of shifts, so a row is read as contiguous 256 + 768 byte runs (K % 4 == 0)
@@ -270,9 +280,11 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
 #pragma unroll
                     for (int u = 0; u < UNROLL; ++u) s0[u] = s1[u] = s2[u] = 0;
                 }
+                if (!TRUST) {
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u)
-                    if (kb + u >= cnt) jj[u] = -1;
+                    for (int u = 0; u < UNROLL; ++u)
+                        if (kb + u >= cnt) jj[u] = -1;
+                }
             } else {
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
@@ -286,10 +298,33 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                     s1[u] = srow[3 * kq + 1];
                     s2[u] = srow[3 * kq + 2];
                 }
-                if (k >= cnt) jj[u] = -1;
+                if (!TRUST && k >= cnt) jj[u] = -1;
             }
             }
-            if (LDS_POS) {
+            if (TRUST && LDS_POS) {
+                // indices below the count are atoms of the row's own system (the list is the neighbor
+                // build's): the staged span holds them all.  The clamp keeps the reads of the slots
+                // beyond the count, and of a list that breaks the promise, inside the stage.
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    unsigned at = (unsigned)(jj[u] - span0);
+                    at = at < (unsigned)(span_n - 1) ? at : (unsigned)(span_n - 1);
+                    at = __umul24(at, 3u);  // (a full-rate multiply: the stage holds fewer than 2^24 atoms)
+                    xj[u] = s_pos[at + 0];
+                    yj[u] = s_pos[at + 1];
+                    zj[u] = s_pos[at + 2];
+                }
+            } else if (TRUST) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    unsigned j = (unsigned)jj[u];
+                    j = j < (unsigned)(a.n_atoms - 1) ? j : (unsigned)(a.n_atoms - 1);
+                    const float* pj = a.pos + 3 * (size_t)j;
+                    xj[u] = pj[0];
+                    yj[u] = pj[1];
+                    zj[u] = pj[2];
+                }
+            } else if (LDS_POS) {
                 // every lane reads the stage (a neighbor outside the staged span reads the span's first atom for
                 // now); the lanes with such a neighbor, if there are any at all, fetch it from memory afterwards
                 unsigned outside = 0;
@@ -335,7 +370,7 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                 if (IMG == 2) {
                     double d0, d1, d2;
                     const double r2 = pair_d2_nearest_diagonal(xi, yi, zi, xj[u], yj[u], zj[u], hd, hdi, d0, d1, d2);
-                    if (jj[u] < 0 || !(r2 < a.rc2)) continue;
+                    if (u >= n_mine || !(r2 < a.rc2)) continue;
                     pair_terms<VIRIAL, SWITCH>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
                     continue;
                 }
@@ -352,13 +387,13 @@ __device__ __forceinline__ void lj_rows(const LjArgs& a, int row0, int row_end, 
                         t0 = t[0];
                         t1 = t[1];
                         t2 = t[2];
-                    } else if (jj[u] >= 0) {
+                    } else if (TRUST ? u < n_mine : jj[u] >= 0) {
                         shift_vector(cell_row, s0[u], s1[u], s2[u], t0, t1, t2);
                     }
                 }
                 double d0, d1, d2;
                 double r2 = pair_d2_shifted(xi, yi, zi, xj[u], yj[u], zj[u], t0, t1, t2, d0, d1, d2);
-                if (jj[u] < 0 || !(r2 < a.rc2)) continue;
+                if ((TRUST ? u >= n_mine : jj[u] < 0) || !(r2 < a.rc2)) continue;
                 pair_terms<VIRIAL, SWITCH>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
             }
         }
@@ -447,8 +482,24 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
         int tid = threadIdx.x;
         asm volatile("" : "+v"(tid));
         if (staged) {
+            // kStageLoads loads of a thread are in flight together (clamped rather than branched over, so that
+            // none of them waits for a condition): a copy with one load outstanding per thread costs a round trip
+            // to memory per 512 words, which for a system of a few thousand atoms is most of a workgroup's life
             const float* src = a.pos + 3 * (size_t)span0;
-            for (int t = tid; t < 3 * span_n; t += kBlockFull) s_pos[t] = src[t];
+            const int n_words = 3 * span_n;
+            for (int base = 0; base < n_words; base += kStageLoads * kBlockFull) {
+                float v[kStageLoads];
+#pragma unroll
+                for (int k = 0; k < kStageLoads; ++k) {
+                    const int t = base + k * kBlockFull + tid;
+                    v[k] = src[t < n_words ? t : n_words - 1];
+                }
+#pragma unroll
+                for (int k = 0; k < kStageLoads; ++k) {
+                    const int t = base + k * kBlockFull + tid;
+                    if (t < n_words) s_pos[t] = v[k];
+                }
+            }
         }
         if (SHIFTS && tid < 27) {
             const int t = tid;
