@@ -339,9 +339,11 @@ __device__ __forceinline__ void choose_grid(NlSys& s, const NlArgs& a, const uin
     // largest cell-local coordinate the search can meet
     const double reach = (s.R[0] + 1) * len[0] + (s.R[1] + 1) * len[1] + (s.R[2] + zr) * len[2];
     s.tol = (float)(2.0e-6 * (reach / a.rc + 1.0));
-    // |q|^2 - 2 p.q against rc^2 - |p|^2 in float32: ten roundings of terms no larger than 3 reach^2
-    // (three for |q|^2, three fused multiply-adds, four for the threshold), 2^-24 relative each
-    s.tol_scan = (float)((double)s.tol + 1.6e-6 * (reach / a.rc) * (reach / a.rc));
+    // |q|^2 - 2 p.q against rc^2 - |p|^2 in float32, |p| and |q| at most reach: |q|^2 takes three roundings of
+    // values up to reach^2, the three fused multiply-adds round values up to 3 reach^2 (|q|^2 + 2 |p.q|), the
+    // threshold takes four roundings of values up to reach^2: (3 + 9 + 4) 2^-24 reach^2 = 0.96e-6 reach^2 in
+    // all; the constant leaves nearly a factor of two
+    s.tol_scan = (float)((double)s.tol + 1.8e-6 * (reach / a.rc) * (reach / a.rc));
 }
 
 __device__ __forceinline__ NlSearchSys search_view(const NlSys& s) {

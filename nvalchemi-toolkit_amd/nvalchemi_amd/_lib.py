@@ -183,8 +183,15 @@ class _Workspaces:
         key = (device.index, _stream(device), purpose)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
+            old = buf
             buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
-            buf[:256].zero_()  # (the neighbor build keeps status bits in its workspace's header from build to build)
+            # The neighbor build keeps status bits in its workspace's header from build to build: a fresh buffer
+            # starts with a zero header, a regrown one takes over the header of the buffer it replaces (so that an
+            # overflow recorded through the smaller buffer is still reported by nvamd_nl_status).
+            if old is None:
+                buf[:256].zero_()
+            else:
+                buf[:256].copy_(old[:256])
             self._bufs[key] = buf
         return buf
 

@@ -14,7 +14,9 @@ updates" (nvalchemi/dynamics/_ops/fire.py:270-272):
 
 All atoms of a system see the same pre-update scalars.  The reference's own step is in a kernel
 library outside its tree, so what its sentences leave open (the side of ``vf == 0``, ``>`` against
-``>=`` for ``n_min``, the Euler form) is this library's choice.  Only the vanilla branch exists:
+``>=`` for ``n_min``, the Euler form) is this library's choice, and the whole step is unpinned
+against the reference's output.  With the sums taken at entry and the mixing applied to the kicked
+velocity, the step is less damped than a mix-then-integrate FIRE.  Only the vanilla branch exists:
 ``fire_step`` raises ``NotImplementedError`` for a non-zero ``uphill_flag``.
 """
 

@@ -2,7 +2,13 @@
 nvalchemi/dynamics/optimizers/fire.py:79-290).  Defaults: ``maxstep=0.2, n_min=5, f_dec=0.5,
 f_inc=1.1, alpha_start=0.1, f_alpha=0.99``, ``dt_max = 10 dt``, ``dt_min = 0.02 dt``; ``dt`` is
 used as given (it is not converted from femtoseconds).  ``pre_update`` performs the whole
-FIRE step with the forces of the previous evaluation; ``post_update`` does nothing."""
+FIRE step with the forces of the previous evaluation; ``post_update`` does nothing.
+
+The order of the step (MD integration, then velocity mixing, then the parameter update, with the
+sums taken at entry) is the one the reference's sentences give; its kernel is in a library outside
+its tree, so the step is not pinned against the reference's output.  This order damps the first
+kicks less than mixing before integrating would: from a start with pairs far up the repulsive
+wall (a random gas) give ``maxstep`` a value well below the nearest-neighbor distance."""
 
 from __future__ import annotations
 

@@ -185,3 +185,36 @@ def test_rows_that_overflow_after_the_first_build_leave_a_flag():
         assert not h.overflowed()  # (read and cleared)
     h(ctx(b), stage())
     assert h.overflowed() == (int(h._num_neighbors.max()) > K)
+
+
+def test_status_bits_survive_a_regrown_workspace(monkeypatch):
+    """The accumulated status bits live in the header of the per-stream workspace.  A larger build makes the
+    package replace that buffer: the new one takes the old header over, so an overflow recorded through the
+    smaller buffer is still reported afterwards."""
+    from nvalchemi_amd import _lib
+
+    monkeypatch.setattr(_lib, "workspaces", _lib._Workspaces())
+    dev = torch.device(DEV)
+
+    def build(n, K, box):
+        g = torch.Generator().manual_seed(n)
+        pos = (torch.rand(n, 3, generator=g) * box).to(dev)
+        cell = (torch.eye(3) * box).reshape(1, 3, 3).to(dev)
+        pbc = torch.ones(1, 3, dtype=torch.bool, device=dev)
+        ptr = torch.tensor([0, n], dtype=torch.int32, device=dev)
+        bidx = torch.zeros(n, dtype=torch.int32, device=dev)
+        nm = torch.full((n, K), n, dtype=torch.int32, device=dev)
+        nn = torch.zeros(n, dtype=torch.int32, device=dev)
+        sh = torch.zeros(n, K, 3, dtype=torch.int32, device=dev)
+        _lib.nl_build(pos, cell, pbc, ptr, bidx, None, 2.5, K, False, 0, nm, nn, sh)
+        return nn
+
+    _lib.nl_status(64, 1, dev, clear=True)
+    nn = build(64, 4, 4.0)  # 64 atoms in a 4 A box: far more than 4 neighbors each
+    assert int(nn.max()) > 4
+    small = _lib.workspaces.get(dev, "nl", 1).numel()
+    nn = build(20000, 64, 60.0)  # a dilute box through a much larger workspace: no overflow of its own
+    assert int(nn.max()) <= 64
+    assert _lib.workspaces.get(dev, "nl", 1).numel() > small
+    st = _lib.nl_status(20000, 1, dev).tolist()
+    assert st[0] == 0 and st[1] & 2  # NVAMD_NL_STATUS_ROW_OVERFLOW of the earlier build

@@ -37,6 +37,28 @@ def test_workspace_sizes_are_host_computations():
     assert _lib.nl_workspace_bytes(0, 0) > 0
 
 
+def test_static_scratch_macro_is_the_workspace_of_its_largest_case(tmp_path):
+    """NVAMD_LJ_STATIC_SCRATCH_BYTES in the header must equal what the pair kernel carves for
+    NVAMD_LJ_STATIC_MAX_SYSTEMS systems (full list: the size does not depend on the number of atoms), so the
+    macro cannot drift from the carving.  The header is read by a C compiler, as a C caller would."""
+    import ctypes
+    import subprocess
+
+    from nvalchemi_amd import _lib
+
+    src = tmp_path / "m.c"
+    src.write_text('#include <stdio.h>\n#include "nvalchemi_amd.h"\nint main(void) { printf("%d %zu\\n", '
+                   "(int)NVAMD_LJ_STATIC_MAX_SYSTEMS, (size_t)NVAMD_LJ_STATIC_SCRATCH_BYTES); return 0; }\n")
+    exe = tmp_path / "m"
+    subprocess.run(["gcc", "-std=c99", "-I", str(ROOT / "include"), str(src), "-o", str(exe)], check=True)
+    max_systems, scratch = map(int, subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split())
+    assert max_systems == _lib.LJ_STATIC_MAX_SYSTEMS
+    for n_atoms in (0, 1, 10_000_000):
+        out = ctypes.c_size_t(0)
+        assert _lib.library().nvamd_lj_workspace_bytes(n_atoms, max_systems, 0, ctypes.byref(out)) == 0
+        assert out.value == scratch
+
+
 def test_error_codes_and_messages_cross_the_boundary():
     import ctypes
 
