@@ -172,10 +172,10 @@ __device__ __forceinline__ bool wave_segmented_max(int seg, float& v) {
 constexpr float kFireVmax = 3.0e38f;
 
 struct FireScratch {
-    double* acc;   // (M,3): sum F.v, sum v.v, sum F.F
-    float* mix_a;  // (M) factor on v
-    float* mix_b;  // (M) factor on F
-    float* dt_use; // (M) time step of the MD sub-step
+    double* acc;     // (M,3): sum F.v, sum v.v, sum F.F
+    float* alpha0;   // (M) mixing parameter of before the update
+    float* dt0;      // (M) time step of before the update (the MD sub-step integrates with it)
+    float* spare;    // (M)
 };
 
 __global__ __launch_bounds__(kBlock) void fire_clear_kernel(double* acc, int n) {
@@ -183,131 +183,185 @@ __global__ __launch_bounds__(kBlock) void fire_clear_kernel(double* acc, int n) 
     if (t < n) acc[t] = 0.0;
 }
 
-// A workgroup takes kFireChunks chunks of kBlock atoms.  Inside a wave the atoms of one system are summed
-// with shuffles; the sums of the first kFireSlots systems a workgroup meets are then collected in LDS and
-// go to memory once per workgroup (a system of a few thousand atoms otherwise receives one atomic per wave
-// on the same three addresses, which is what this kernel then waits for).
-constexpr int kFireChunks = 4;
+// Before the sums.  The accumulators start at zero (or at the caller's sums, compute_reductions = 0), and the
+// mixing parameter and the time step of before the update are set aside: the update kernel's per-atom threads
+// read them there while its per-system threads write the new ones into the caller's arrays.
+__global__ __launch_bounds__(kBlock) void fire_prepare_kernel(const float* __restrict__ alpha,
+                                                              const float* __restrict__ dt,
+                                                              const float* __restrict__ vf,
+                                                              const float* __restrict__ vv,
+                                                              const float* __restrict__ ff, FireScratch ws,
+                                                              int import_sums, int m) {
+    int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    ws.acc[3 * s + 0] = import_sums ? (double)vf[s] : 0.0;
+    ws.acc[3 * s + 1] = import_sums ? (double)vv[s] : 0.0;
+    ws.acc[3 * s + 2] = import_sums ? (double)ff[s] : 0.0;
+    ws.alpha0[s] = alpha[s];
+    ws.dt0[s] = dt[s];
+}
+
+// A workgroup takes kFireQuad * kBlock atoms, a thread kFireQuad consecutive ones (read as 16-byte words when the
+// arrays allow it); a thread's atoms are nearly always of one system, so they are summed in registers first.
+// Inside a wave the threads of one system are then summed with shuffles; the sums of the first kFireSlots systems
+// a workgroup meets are collected in LDS and go to memory once per workgroup (a system of a few thousand atoms
+// otherwise receives one atomic per wave on the same three addresses, which is what this kernel then waits for).
+constexpr int kFireQuad = 4;
 constexpr int kFireSlots = 8;
 
+template <bool VEC>
 __global__ __launch_bounds__(kBlock) void fire_reduce_kernel(const float* __restrict__ vel,
                                                              const float* __restrict__ frc,
                                                              const int32_t* __restrict__ bidx,
-                                                             double* __restrict__ acc, int n_atoms) {
+                                                             double* __restrict__ acc, int n_atoms,
+                                                             int chunks_per_block) {
     __shared__ double s_acc[kFireSlots][3];
-    const int first = (int)blockIdx.x * (kFireChunks * kBlock);  // (below n_atoms: the grid is sized so)
+    // a workgroup takes chunks_per_block consecutive chunks of kFireQuad * kBlock atoms
+    const int block_first = (int)blockIdx.x * chunks_per_block * (kFireQuad * kBlock);  // (below n_atoms: the grid is sized so)
     if (threadIdx.x < kFireSlots * 3) (&s_acc[0][0])[threadIdx.x] = 0.0;
-    const int seg_lo = bidx[first];
+    const int seg_lo = bidx[block_first];
     __syncthreads();
-    for (int c = 0; c < kFireChunks; ++c) {  // (every lane takes every turn: the sums use shuffles)
-        const int i = first + c * kBlock + (int)threadIdx.x;
-        double v[3] = {0.0, 0.0, 0.0};
-        int seg = -1 - (i - n_atoms);  // distinct negative ids past the end: never merged
-        if (i < n_atoms) {
-            seg = bidx[i];
+    auto deposit = [&](int seg, const double* v) {
+        const unsigned slot = (unsigned)(seg - seg_lo);
+        if (slot < (unsigned)kFireSlots) {
+            atomicAdd(&s_acc[slot][0], v[0]);
+            atomicAdd(&s_acc[slot][1], v[1]);
+            atomicAdd(&s_acc[slot][2], v[2]);
+        } else {
+            atomic_add_f64(acc + 3 * (size_t)seg + 0, v[0]);
+            atomic_add_f64(acc + 3 * (size_t)seg + 1, v[1]);
+            atomic_add_f64(acc + 3 * (size_t)seg + 2, v[2]);
+        }
+    };
+    for (int chunk = 0; chunk < chunks_per_block; ++chunk) {
+    const int first = block_first + chunk * (kFireQuad * kBlock);
+    if (first >= n_atoms) break;
+    const int i0 = first + kFireQuad * (int)threadIdx.x;
+    double v[3] = {0.0, 0.0, 0.0};
+    int seg = -1 - (int)threadIdx.x;  // distinct negative ids for threads past the end: never merged
+    if (i0 < n_atoms) {
+        const int n = (n_atoms - i0) < kFireQuad ? (n_atoms - i0) : kFireQuad;
+        seg = bidx[i0];
+        float x[3 * kFireQuad], f[3 * kFireQuad];
+        if (VEC && n == kFireQuad) {
+            const float4* xv = reinterpret_cast<const float4*>(vel + 3 * (size_t)i0);
+            const float4* fv = reinterpret_cast<const float4*>(frc + 3 * (size_t)i0);
 #pragma unroll
-            for (int a = 0; a < 3; ++a) {
-                double vv = (double)vel[3 * (size_t)i + a], ff = (double)frc[3 * (size_t)i + a];
-                v[0] += ff * vv;
-                v[1] += vv * vv;
-                v[2] += ff * ff;
+            for (int q = 0; q < 3; ++q) {
+                const float4 a = xv[q], b = fv[q];
+                x[4 * q + 0] = a.x; x[4 * q + 1] = a.y; x[4 * q + 2] = a.z; x[4 * q + 3] = a.w;
+                f[4 * q + 0] = b.x; f[4 * q + 1] = b.y; f[4 * q + 2] = b.z; f[4 * q + 3] = b.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 3 * kFireQuad; ++k) {
+                const bool in = k < 3 * n;
+                x[k] = in ? vel[3 * (size_t)i0 + k] : 0.f;
+                f[k] = in ? frc[3 * (size_t)i0 + k] : 0.f;
             }
         }
-        const bool head = wave_segmented_sum<3>(seg, v);
-        if (head && i < n_atoms) {
-            const unsigned slot = (unsigned)(seg - seg_lo);
-            if (slot < (unsigned)kFireSlots) {
-                atomicAdd(&s_acc[slot][0], v[0]);
-                atomicAdd(&s_acc[slot][1], v[1]);
-                atomicAdd(&s_acc[slot][2], v[2]);
-            } else {
-                atomic_add_f64(acc + 3 * (size_t)seg + 0, v[0]);
-                atomic_add_f64(acc + 3 * (size_t)seg + 1, v[1]);
-                atomic_add_f64(acc + 3 * (size_t)seg + 2, v[2]);
+#pragma unroll
+        for (int q = 0; q < kFireQuad; ++q) {
+            double w[3] = {0.0, 0.0, 0.0};
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                const double vv = (double)x[3 * q + c], ff = (double)f[3 * q + c];
+                w[0] += ff * vv;
+                w[1] += vv * vv;
+                w[2] += ff * ff;
+            }
+            const int sq = q < n ? bidx[i0 + q] : seg;
+            if (sq == seg) {
+                v[0] += w[0]; v[1] += w[1]; v[2] += w[2];
+            } else if (q < n) {
+                deposit(sq, w);  // (an atom of the next system inside a thread's four: rare)
             }
         }
+    }
+    const bool head = wave_segmented_sum<3>(seg, v);
+    if (head && seg >= 0) deposit(seg, v);
     }
     __syncthreads();
     if (threadIdx.x < kFireSlots * 3) {
         // (a slot that no atom touched is still zero and names a system that may not exist)
-        const double v = (&s_acc[0][0])[threadIdx.x];
-        if (v != 0.0) atomic_add_f64(acc + 3 * (size_t)seg_lo + threadIdx.x, v);
+        const double t = (&s_acc[0][0])[threadIdx.x];
+        if (t != 0.0) atomic_add_f64(acc + 3 * (size_t)seg_lo + threadIdx.x, t);
     }
 }
 
-// caller-supplied vf/vv/ff (compute_reductions = 0): widen them into the accumulator
-__global__ __launch_bounds__(kBlock) void fire_import_kernel(const float* vf, const float* vv,
-                                                             const float* ff, double* acc, int m) {
-    int s = blockIdx.x * kBlock + threadIdx.x;
-    if (s >= m) return;
-    acc[3 * s + 0] = (double)vf[s];
-    acc[3 * s + 1] = (double)vv[s];
-    acc[3 * s + 2] = (double)ff[s];
+void launch_fire_reduce(const float* velocities, const float* forces, const int32_t* batch_idx, double* acc,
+                        int n_atoms, hipStream_t st) {
+    // about three workgroups per compute unit at most: every workgroup ends with atomics on its systems' sums,
+    // which for one large system are the same three addresses for all of them
+    const int n_chunks = (n_atoms + kFireQuad * kBlock - 1) / (kFireQuad * kBlock);
+    const int per = n_chunks > 1024 ? (n_chunks + 767) / 768 : 1;
+    const dim3 grid_r((n_chunks + per - 1) / per), blk(kBlock);
+    if (aligned16(velocities) && aligned16(forces))
+        hipLaunchKernelGGL(fire_reduce_kernel<true>, grid_r, blk, 0, st, velocities, forces, batch_idx, acc, n_atoms, per);
+    else
+        hipLaunchKernelGGL(fire_reduce_kernel<false>, grid_r, blk, 0, st, velocities, forces, batch_idx, acc, n_atoms, per);
 }
 
-__global__ __launch_bounds__(kBlock) void fire_params_kernel(
-    float* __restrict__ alpha, float* __restrict__ dt, const float* __restrict__ alpha_start,
-    const float* __restrict__ f_alpha, const float* __restrict__ dt_min,
+// The update: blocks below n_atom_blocks take one atom per thread, the blocks after them one system per thread.
+//   per atom   : MD step with the time step of before the update, then the mixing with the parameter of before
+//                the update (both set aside by fire_prepare_kernel) and the sums of entry
+//   per system : the sums go out, n+, dt and alpha are updated in the caller's arrays
+__global__ __launch_bounds__(kBlock) void fire_update_kernel(
+    float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
+    const float* __restrict__ masses, const float* __restrict__ maxstep, const int32_t* __restrict__ bidx,
+    const uint8_t* __restrict__ active, float* __restrict__ alpha, float* __restrict__ dt,
+    const float* __restrict__ alpha_start, const float* __restrict__ f_alpha, const float* __restrict__ dt_min,
     const float* __restrict__ dt_max, int32_t* __restrict__ n_pos, const int32_t* __restrict__ n_min,
     const float* __restrict__ f_dec, const float* __restrict__ f_inc, float* __restrict__ vf,
-    float* __restrict__ vv, float* __restrict__ ff, const uint8_t* __restrict__ active,
-    FireScratch ws, int write_reductions, int m) {
-    int s = blockIdx.x * kBlock + threadIdx.x;
-    if (s >= m) return;
-    double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
-    if (write_reductions) {
-        vf[s] = (float)P;
-        vv[s] = (float)VV;
-        ff[s] = (float)FF;
-    }
-    const float h_stored = dt[s];  // the MD sub-step integrates with the time step of before the update
-    float h = h_stored;
-    float ma = 1.0f, mb = 0.0f;
-    if (!active || active[s]) {
+    float* __restrict__ vv, float* __restrict__ ff, FireScratch ws, int write_reductions, int n_atoms,
+    int n_atom_blocks, int m) {
+    if ((int)blockIdx.x >= n_atom_blocks) {
+        const int s = ((int)blockIdx.x - n_atom_blocks) * kBlock + (int)threadIdx.x;
+        if (s >= m) return;
+        const double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+        if (write_reductions) {
+            vf[s] = (float)P;
+            vv[s] = (float)VV;
+            ff[s] = (float)FF;
+        }
+        if (active && !active[s]) return;
+        float h = ws.dt0[s];
         if (P >= 0.0) {
-            float al = alpha[s];
-            ma = 1.0f - al;
-            mb = (FF > 0.0) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
-            int np = n_pos[s] + 1;
+            const int np = n_pos[s] + 1;
             n_pos[s] = np;
             if (np > n_min[s]) {
-                float nd = h * f_inc[s];
-                float cap = dt_max[s];
+                const float nd = h * f_inc[s];
+                const float cap = dt_max[s];
                 h = nd < cap ? nd : cap;
-                alpha[s] = al * f_alpha[s];
+                alpha[s] = ws.alpha0[s] * f_alpha[s];
             }
         } else {
-            ma = 0.0f;
-            mb = 0.0f;
             n_pos[s] = 0;
-            float nd = h * f_dec[s];
-            float lo = dt_min[s];
+            const float nd = h * f_dec[s];
+            const float lo = dt_min[s];
             h = nd > lo ? nd : lo;
             alpha[s] = alpha_start[s];
         }
         dt[s] = h;
+        return;
     }
-    ws.mix_a[s] = ma;
-    ws.mix_b[s] = mb;
-    ws.dt_use[s] = h_stored;
-}
-
-__global__ __launch_bounds__(kBlock) void fire_update_kernel(
-    float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
-    const float* __restrict__ masses, const float* __restrict__ maxstep,
-    const int32_t* __restrict__ bidx, const uint8_t* __restrict__ active, FireScratch ws,
-    int n_atoms) {
-    int i = blockIdx.x * kBlock + threadIdx.x;
+    const int i = (int)blockIdx.x * kBlock + (int)threadIdx.x;
     if (i >= n_atoms) return;
-    int s = bidx[i];
+    const int s = bidx[i];
     if (active && !active[s]) return;
-    float ma = ws.mix_a[s], mb = ws.mix_b[s], h = ws.dt_use[s], ms = maxstep[s], m = masses[i];
+    const double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+    const float al = ws.alpha0[s], h = ws.dt0[s], ms = maxstep[s], m_i = masses[i];
+    float ma = 0.0f, mb = 0.0f;
+    if (P >= 0.0) {
+        ma = 1.0f - al;
+        mb = (FF > 0.0) ? (float)((double)al * sqrt(VV / FF)) : 0.0f;
+    }
     size_t b = 3 * (size_t)i;
     float v[3], dr[3], f[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
         f[a] = frc[b + a];
-        float acc = f[a] / m;
+        float acc = f[a] / m_i;
         v[a] = vel[b + a] + (h * acc);
         v[a] = fminf(fmaxf(v[a], -kFireVmax), kFireVmax);  // keep dr finite
         dr[a] = h * v[a];
@@ -556,30 +610,25 @@ NVAMD_EXPORT int32_t nvamd_fire_step(float* positions, float* velocities, const 
     FireScratch ws;
     ws.acc = reinterpret_cast<double*>(w);
     w += align_up(m * 3 * sizeof(double));
-    ws.mix_a = reinterpret_cast<float*>(w);
+    ws.alpha0 = reinterpret_cast<float*>(w);
     w += align_up(m * sizeof(float));
-    ws.mix_b = reinterpret_cast<float*>(w);
+    ws.dt0 = reinterpret_cast<float*>(w);
     w += align_up(m * sizeof(float));
-    ws.dt_use = reinterpret_cast<float*>(w);
+    ws.spare = reinterpret_cast<float*>(w);
     hipStream_t st = static_cast<hipStream_t>(stream);
     dim3 blk(kBlock);
     dim3 grid_m((n_systems + kBlock - 1) / kBlock);
-    dim3 grid_n((n_atoms + kBlock - 1) / kBlock);
-    if (compute_reductions) {
-        int n3 = 3 * n_systems;
-        hipLaunchKernelGGL(fire_clear_kernel, dim3((n3 + kBlock - 1) / kBlock), blk, 0, st, ws.acc, n3);
-        if (n_atoms > 0)
-            hipLaunchKernelGGL(fire_reduce_kernel, dim3((n_atoms + kFireChunks * kBlock - 1) / (kFireChunks * kBlock)), blk,
-                               0, st, velocities, forces, batch_idx, ws.acc, n_atoms);
-    } else {
-        hipLaunchKernelGGL(fire_import_kernel, grid_m, blk, 0, st, vf, vv, ff, ws.acc, n_systems);
+    // three launches: prepare (per system), sums (per four atoms), update (per atom and per system)
+    hipLaunchKernelGGL(fire_prepare_kernel, grid_m, blk, 0, st, alpha, dt, vf, vv, ff, ws, compute_reductions ? 0 : 1,
+                       n_systems);
+    if (compute_reductions && n_atoms > 0) {
+        launch_fire_reduce(velocities, forces, batch_idx, ws.acc, n_atoms, st);
     }
-    hipLaunchKernelGGL(fire_params_kernel, grid_m, blk, 0, st, alpha, dt, alpha_start, f_alpha, dt_min,
-                       dt_max, n_steps_positive, n_min, f_dec, f_inc, vf, vv, ff, active, ws,
-                       compute_reductions ? 1 : 0, n_systems);
-    if (n_atoms > 0)
-        hipLaunchKernelGGL(fire_update_kernel, grid_n, blk, 0, st, positions, velocities, forces, masses,
-                           maxstep, batch_idx, active, ws, n_atoms);
+    const int n_atom_blocks = (n_atoms + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL(fire_update_kernel, dim3(n_atom_blocks + (n_systems + kBlock - 1) / kBlock), blk, 0, st, positions,
+                       velocities, forces, masses, maxstep, batch_idx, active, alpha, dt, alpha_start, f_alpha, dt_min,
+                       dt_max, n_steps_positive, n_min, f_dec, f_inc, vf, vv, ff, ws, compute_reductions ? 1 : 0,
+                       n_atoms, n_atom_blocks, n_systems);
     NVAMD_LAUNCH_CHECK("fire launch");
     return NVAMD_OK;
 }
@@ -627,9 +676,9 @@ NVAMD_EXPORT int32_t nvamd_fire2_step(float* positions, float* velocities, const
     const dim3 blk(kBlock), grid_m((n_systems + kBlock - 1) / kBlock), grid_n((n_atoms + kBlock - 1) / kBlock);
     const int n3 = 3 * n_systems;
     hipLaunchKernelGGL(fire_clear_kernel, dim3((n3 + kBlock - 1) / kBlock), blk, 0, st, ws.acc, n3);
-    if (n_atoms > 0)
-        hipLaunchKernelGGL(fire_reduce_kernel, dim3((n_atoms + kFireChunks * kBlock - 1) / (kFireChunks * kBlock)), blk, 0, st,
-                           velocities, forces, batch_idx, ws.acc, n_atoms);
+    if (n_atoms > 0) {
+        launch_fire_reduce(velocities, forces, batch_idx, ws.acc, n_atoms, st);
+    }
     hipLaunchKernelGGL(fire2_params_kernel, grid_m, blk, 0, st, alpha, dt, nsteps_inc, vf, v_sumsq, f_sumsq, active,
                        ws, p, n_systems);
     if (n_atoms > 0) {

@@ -195,6 +195,18 @@ class _Workspaces:
             self._bufs[key] = buf
         return buf
 
+    def share(self, device: torch.device, from_stream: int, to_stream: int) -> None:
+        """Let ``to_stream`` use the buffers of ``from_stream`` (raw stream handles).  For a capture stream whose
+        graph will be replayed into ``from_stream``: the two never run side by side."""
+        for (dev, stream, purpose), buf in list(self._bufs.items()):
+            if dev == device.index and stream == from_stream:
+                self._bufs[(dev, to_stream, purpose)] = buf
+
+    def unshare(self, device: torch.device, stream: int) -> None:
+        """Forget every entry of ``stream`` (the buffers stay with whoever else holds them)."""
+        for key in [k for k in self._bufs if k[0] == device.index and k[1] == stream]:
+            del self._bufs[key]
+
 
 workspaces = _Workspaces()
 

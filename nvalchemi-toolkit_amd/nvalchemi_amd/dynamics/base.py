@@ -550,6 +550,90 @@ class BaseDynamics(HookRegistryMixin):
     def _masked_post_update(self, batch, mask: torch.Tensor) -> None:
         self._run_masked(batch, mask, False, True)
 
+    # ---- steady-state steps replayed from a captured HIP graph ---------------------------------------
+    #: ``run`` replays a captured step when nothing in the step needs the host (see ``_graph_eligible``);
+    #: set to False on an instance or a subclass to always step eagerly
+    graph_replay: bool = True
+    #: eager steps taken with an unchanged batch before a capture is attempted (the first steps size
+    #: workspaces and settle the neighbor hook's row width, which involves the host)
+    _GRAPH_WARM_STEPS = 2
+
+    def _graph_eligible(self, batch) -> bool:
+        """A step can be captured once and replayed when every step enqueues the same kernels on the same
+        buffers and no decision is taken on the host: no convergence criterion (its result ends the run), no
+        sampler, the plain ``step`` of this class, and only hooks that run on every step and declare
+        ``graph_safe`` (their work is kernels on persistent buffers: the neighbor hook after its first build)."""
+        if not self.graph_replay or self.convergence_hook is not None or self.sampler is not None:
+            return False
+        if type(self).step is not BaseDynamics.step or not torch.cuda.is_available():
+            return False
+        pos = getattr(batch, "positions", None)
+        if not isinstance(pos, torch.Tensor) or pos.device.type != "cuda":
+            return False
+        if getattr(batch, "status", None) is not None and not self._honors_active_mask:
+            return False  # (the save / restore of inactive systems indexes with masks: a host synchronisation)
+        for hook in self.hooks:
+            if getattr(hook, "frequency", 1) != 1 or not getattr(hook, "graph_safe", False):
+                return False
+        return True
+
+    def _graph_key(self, batch) -> tuple:
+        """What a captured step is tied to: the batch's tensors (a replay writes to the addresses it was
+        captured with), its sizes, and whatever the hooks say their buffers are."""
+        key: list = [id(batch), batch.num_nodes, batch.num_graphs, torch.cuda.current_stream().cuda_stream]
+        for name in ("positions", "velocities", "forces", "energy", "atomic_masses", "batch_idx", "cell", "status"):
+            t = getattr(batch, name, None)
+            key.append((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None)
+        for hook in self.hooks:
+            fn = getattr(hook, "graph_key", None)
+            key.append((id(hook), fn() if callable(fn) else None))
+        return tuple(key)
+
+    def _graph_step(self, batch) -> bool:
+        """One step by graph replay.  False: not possible now (the caller takes the step eagerly)."""
+        if not self._graph_eligible(batch):
+            self._graph_state = None
+            return False
+        key = self._graph_key(batch)
+        st = getattr(self, "_graph_state", None)
+        if st is None or st["key"] != key:
+            st = self._graph_state = {"key": key, "warm": 0, "graph": None, "failed": False}
+        if st["failed"]:
+            return False
+        if st["graph"] is None:
+            if st["warm"] < self._GRAPH_WARM_STEPS:
+                st["warm"] += 1
+                return False
+            from .. import _lib
+
+            graph = torch.cuda.CUDAGraph()
+            current = torch.cuda.current_stream()
+            side = torch.cuda.Stream(device=current.device)
+            # the captured kernels use the workspaces of the stream the eager steps ran on: replays are
+            # launched into that stream, in order with its other work
+            _lib.workspaces.share(current.device, current.cuda_stream, side.cuda_stream)
+            count, converged = self.step_count, self._last_converged
+            side.wait_stream(current)
+            try:
+                with torch.cuda.stream(side):
+                    with torch.cuda.graph(graph, stream=side):
+                        self.step(batch)
+            except Exception:  # something in the step needs the host after all: stay eager for this batch
+                st["failed"] = True
+                return False
+            finally:
+                current.wait_stream(side)
+                _lib.workspaces.unshare(current.device, side.cuda_stream)
+                self.step_count, self._last_converged = count, converged  # (the capture ran nothing)
+            if self._graph_key(batch) != key:  # the step replaced a buffer: what was captured is already stale
+                st["failed"] = True
+                return False
+            st["graph"] = graph
+        st["graph"].replay()
+        self._last_converged = None
+        self.step_count += 1
+        return True
+
     def run(self, batch, n_steps: int | None = None):
         resolved = n_steps if n_steps is not None else self.n_steps
         if resolved is None:
@@ -558,6 +642,8 @@ class BaseDynamics(HookRegistryMixin):
         self._open_hooks()
         try:
             for _ in range(resolved):
+                if self._graph_step(batch):
+                    continue
                 batch, converged = self.step(batch)
                 if self.sampler is None and converged is not None and converged.numel() == batch.num_graphs:
                     break

@@ -147,6 +147,22 @@ class NeighborListHook:
             format=NeighborListFormat.COO if self._neighbor_list_flag else NeighborListFormat.MATRIX,
             cutoff=self.config.cutoff, search_cutoff=None if self.config.half_list else cutoff)
 
+    # ---- for a dynamics that replays captured steps ---------------------------------------------------
+    @property
+    def graph_safe(self) -> bool:
+        """After the first build (which sizes the rows with the host's help) a call of this hook is kernels
+        on persistent buffers only: it can be captured in a HIP graph and replayed."""
+        return self._neighbor_matrix is not None and not self._first_build and \
+            (self.skin <= 0.0 or self._ref_positions is not None)
+
+    def graph_key(self) -> tuple:
+        """The buffers a captured call is tied to."""
+        def ptr(t):
+            return None if t is None else (t.data_ptr(), tuple(t.shape))
+
+        return (ptr(self._neighbor_matrix), ptr(self._num_neighbors), ptr(self._neighbor_matrix_shifts),
+                ptr(self._ref_positions), ptr(self._rebuild_flags), ptr(getattr(self, "_atom_order", None)))
+
     def overflowed(self, clear: bool = True) -> bool:
         """Whether any build since the last call left an atom with more neighbors than the rows hold
         (the reference never notices this after its first build, nvalchemi/hooks/neighbor_list.py:351-355;

@@ -45,6 +45,9 @@ class WrapPeriodicHook:
     """Wrap ``batch.positions`` into the cell every ``frequency`` steps
     (``DynamicsStage.AFTER_POST_UPDATE`` in the reference's examples)."""
 
+    #: a call is one kernel on the batch's own tensors: a dynamics may capture it in a HIP graph
+    graph_safe = True
+
     def __init__(self, frequency: int = 1, stage: Enum | None = None) -> None:
         self.frequency = frequency
         self.stage = stage

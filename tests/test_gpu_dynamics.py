@@ -304,6 +304,67 @@ def test_one_md_step_replays_from_a_captured_graph():
     assert float(scratch) == float(scratch)
 
 
+def test_run_replays_captured_steps_bit_equal_to_eager_steps():
+    """``run`` takes the steady-state steps of a plain NVE (no convergence criterion, hooks that are kernels
+    only) by replaying one captured step.  100 steps that way, in two calls with unrelated eager work and
+    synchronisations in between, against 100 eager steps of a second copy: positions, velocities and forces
+    equal to the bit (per-system energies are float64 atomics summed in an order that varies from run to run:
+    compared at the usual bar)."""
+    from nvalchemi_amd.dynamics import NVE, DynamicsStage
+    from nvalchemi_amd.hooks import WrapPeriodicHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=0, n_boxes=4, reps=3, a=3.6)
+    N = len(P)
+    rng = np.random.default_rng(1)
+    M = np.full(N, 63.546, dtype=np.float32)
+    V = rng.normal(0, 0.02, (N, 3)).astype(np.float32)
+    Z = np.full(N, 29, dtype=np.int64)
+    sig = float((3.6 / np.sqrt(2)) / 2 ** (1 / 6))
+
+    def make(replay, skin):
+        batch = make_batch(P, Z, M, C, pb, ptr, V)
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=sig, cutoff=5.0)
+        model.model_config.neighbor_config.skin = skin
+        dyn = NVE(model, dt=1.0, hooks=model.make_neighbor_hooks() + [WrapPeriodicHook(stage=DynamicsStage.AFTER_POST_UPDATE)])
+        dyn.graph_replay = replay
+        return batch, dyn
+
+    for skin in (0.0, 0.4):
+        eager_batch, eager = make(False, skin)
+        graph_batch, graphed = make(True, skin)
+        eager.run(eager_batch, n_steps=100)
+        graphed.run(graph_batch, n_steps=40)
+        assert graphed._graph_state is not None and graphed._graph_state["graph"] is not None  # it was captured
+        assert not graphed._graph_state["failed"]
+        scratch = torch.randn(4096, device=DEV).square().sum()  # unrelated eager work between the two runs
+        torch.cuda.synchronize()
+        graphed.run(graph_batch, n_steps=60)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(scratch))
+        assert eager.step_count == graphed.step_count == 100
+        assert getattr(eager, "_graph_state", None) is None
+        for name in ("positions", "velocities", "forces"):
+            assert torch.equal(getattr(graph_batch, name), getattr(eager_batch, name)), (skin, name)
+        close(graph_batch.energy, eager_batch.energy.cpu().numpy(), "energy")
+        assert torch.equal(graph_batch.num_neighbors, eager_batch.num_neighbors)
+
+
+def test_run_steps_eagerly_when_a_step_needs_the_host():
+    """A convergence criterion ends a run from the host: such a dynamics is never captured."""
+    from nvalchemi_amd.dynamics import FIRE, ConvergenceHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=2, n_boxes=2, reps=3, a=3.6)
+    N = len(P)
+    batch = make_batch(P, np.full(N, 29, dtype=np.int64), np.full(N, 63.546, dtype=np.float32), C, pb, ptr,
+                       np.zeros_like(P))
+    model = LennardJonesModelWrapper(epsilon=0.01, sigma=float((3.6 / np.sqrt(2)) / 2 ** (1 / 6)), cutoff=5.0)
+    dyn = FIRE(model, dt=0.5, hooks=model.make_neighbor_hooks(), convergence_hook=ConvergenceHook.from_fmax(1e-3))
+    dyn.run(batch, n_steps=10)
+    assert getattr(dyn, "_graph_state", None) is None
+
+
 def test_hook_leaves_the_cell_order_for_large_systems_and_the_model_uses_it():
     from nvalchemi_amd.hooks import HookContext
     from nvalchemi_amd.models import LennardJonesModelWrapper

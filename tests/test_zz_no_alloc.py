@@ -103,7 +103,8 @@ def test_static_scratch_entry_at_its_largest_number_of_systems():
     for k in ("es", "w"):
         assert np.all(np.abs(got[k] - want[k]) <= 1e-6 + 1e-5 * np.abs(want[k])), k
     # a dimer's energy is the pair energy, half of it on each atom
-    r = bond.norm(dim=1).double().numpy()
+    p64 = pos.cpu().double().reshape(B, 2, 3)  # (the float32 positions the kernel saw)
+    r = (p64[:, 1] - p64[:, 0]).norm(dim=1).numpy()
     u = 4.0 * (r ** -12 - r ** -6)
     assert np.allclose(got["es"], u, rtol=1e-5, atol=1e-6)
 
