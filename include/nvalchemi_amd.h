@@ -278,6 +278,26 @@ int32_t nvamd_lj_energy_forces_hinted(const float* positions, const float* cells
                                       float* system_energies, void* workspace, size_t workspace_bytes,
                                       void* stream);
 
+/* nvamd_lj_energy_forces_hinted (full list) for a caller that evaluates the same batch again and again (an MD
+ * loop).  No counterpart in the reference.  The pair kernel's per-system tables in the workspace (first and
+ * last atom of each system, how the images of its pairs are found) depend on batch_idx, cells,
+ * neighbor_list_cutoff, n_atoms and n_systems only.  reuse_tables = 0: they are computed, as the other entry
+ * points do on every call.  reuse_tables = 1: the caller promises that nothing else has written the workspace
+ * since the previous call of this library's pair kernel through it, that this previous call had the same
+ * batch_idx, cells (contents included), neighbor_list_cutoff, n_atoms, n_systems and the same choice of
+ * virials / system_energies outputs, and was a full-list call: the tables are used as they stand, one launch
+ * fewer.  (Every full-list call leaves the workspace's accumulators at zero for the next one.) */
+int32_t nvamd_lj_energy_forces_repeat(const float* positions, const float* cells,
+                                      const int32_t* neighbor_matrix,
+                                      const int32_t* neighbor_matrix_shifts,
+                                      const int32_t* num_neighbors, const int32_t* batch_idx,
+                                      const int32_t* row_order, double neighbor_list_cutoff, int32_t n_atoms,
+                                      int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
+                                      double epsilon, double sigma, double cutoff, double switch_width,
+                                      int32_t reuse_tables, float* atomic_energies, float* forces, float* virials,
+                                      float* system_energies, void* workspace, size_t workspace_bytes,
+                                      void* stream);
+
 /* nvamd_lj_energy_forces_hinted for callers that cannot allocate device memory or carry a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
  * the reference.  The scratch of the pair kernel (per-system float64 accumulators, first and last atom of

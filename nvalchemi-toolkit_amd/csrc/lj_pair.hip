@@ -624,20 +624,34 @@ __global__ __launch_bounds__(kBlock) void clear_f64_kernel(double* p, size_t n) 
     if (t < n) p[t] = 0.0;
 }
 
-__global__ __launch_bounds__(kBlock) void lj_sys_finish_kernel(const double* __restrict__ sys_acc,
-                                                               float* __restrict__ sys_e,
-                                                               float* __restrict__ virials, int m) {
-    int t = blockIdx.x * kBlock + threadIdx.x;
-    if (t >= m * 10) return;
-    int s = t / 10, k = t % 10;
-    double v = sys_acc[t];
+// The per-system sums leave as float32 (the symmetric half of the virial was accumulated: it is mirrored), and the
+// accumulators go back to zero, so that a call that reuses the workspace's tables (and with them skips the kernel
+// that clears the accumulators) starts from zero.
+__global__ __launch_bounds__(kBlock) void lj_sys_finish_clear_kernel(double* __restrict__ sys_acc,
+                                                                     float* __restrict__ sys_e,
+                                                                     float* __restrict__ virials, int m) {
+    __shared__ double s_v[kBlock / 10 * 10];
+    // a workgroup takes whole systems (25 of them): the mirrored reads stay inside its own slice
+    constexpr int kPer = kBlock / 10;
+    const int s0 = (int)blockIdx.x * kPer;
+    const int t = (int)threadIdx.x;
+    const bool on = t < kPer * 10 && s0 + t / 10 < m;
+    const size_t at = 10 * (size_t)s0 + (size_t)t;
+    double v = 0.0;
+    if (on) {
+        v = sys_acc[at];
+        s_v[t] = v;
+    }
+    __syncthreads();
+    if (!on) return;
+    sys_acc[at] = 0.0;
+    const int s = s0 + t / 10, k = t % 10;
     if (k == 0) {
         if (sys_e) sys_e[s] = (float)v;
     } else if (virials) {
-        // the symmetric half was accumulated: mirror it
-        int c = k - 1;
-        int r = c / 3, q = c % 3;
-        if (r > q) v = sys_acc[10 * (size_t)s + 1 + 3 * q + r];
+        const int c = k - 1;
+        const int r = c / 3, q = c % 3;
+        if (r > q) v = s_v[t - k + 1 + 3 * q + r];
         virials[9 * (size_t)s + c] = (float)v;
     }
 }
@@ -735,7 +749,8 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
                                      int32_t n_atoms, int32_t max_neighbors, int32_t n_systems, int32_t fill_value,
                                      double epsilon, double sigma, double cutoff, double switch_width,
                                      int32_t half_list, float* atomic_energies, float* forces, float* virials,
-                                     float* system_energies, void* workspace, size_t workspace_bytes, void* stream) {
+                                     float* system_energies, void* workspace, size_t workspace_bytes, void* stream,
+                                     int32_t reuse_tables = 0) {
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
     if (!(switch_width >= 0.0) || switch_width > cutoff)
@@ -798,10 +813,12 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
     // the full-list path clears the accumulators in its range kernel when there are at least as many atoms
     // as accumulator words
     const bool clear_with_ranges = !half_list && (size_t)n_atoms >= (size_t)n_systems * 10;
+    // the tables (and the cleared accumulators) of the previous call stand: full list only
+    const bool reuse = reuse_tables && !half_list && n_atoms > 0;
     if (want_sys && n_systems > 0) {
         a.sys_acc = reinterpret_cast<double*>(w);
         size_t n = (size_t)n_systems * 10;
-        if (!clear_with_ranges)
+        if (!clear_with_ranges && !reuse)
             hipLaunchKernelGGL(clear_f64_kernel, dim3((unsigned)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                                st, a.sys_acc, n);
     }
@@ -824,9 +841,10 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
         } else {
             const bool vir = virials != nullptr;
             const bool sys = a.sys_acc != nullptr;
-            hipLaunchKernelGGL(lj_sys_range_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
-                               batch_idx, n_atoms, shifts ? cells : nullptr, a.list_rc, sys_first, sys_last, sys_image,
-                               clear_with_ranges ? a.sys_acc : nullptr, n_systems * 10);
+            if (!reuse)
+                hipLaunchKernelGGL(lj_sys_range_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+                                   batch_idx, n_atoms, shifts ? cells : nullptr, a.list_rc, sys_first, sys_last, sys_image,
+                                   clear_with_ranges ? a.sys_acc : nullptr, n_systems * 10);
             a.sys_first = sys_first;
             a.sys_last = sys_last;
             a.sys_image = sys_image;
@@ -839,8 +857,9 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
         }
     }
     if (want_sys && n_systems > 0) {
-        int n = n_systems * 10;
-        hipLaunchKernelGGL(lj_sys_finish_kernel, dim3((n + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+        // (the accumulators are left at zero for a call that reuses the tables)
+        constexpr int kPer = kBlock / 10;
+        hipLaunchKernelGGL(lj_sys_finish_clear_kernel, dim3((n_systems + kPer - 1) / kPer), dim3(kBlock), 0, st,
                            a.sys_acc, system_energies, virials, n_systems);
     }
     NVAMD_LAUNCH_CHECK("lj launch");
@@ -862,6 +881,22 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_hinted(const float* positions, const
                                  row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
                                  sigma, cutoff, switch_width, half_list, atomic_energies, forces, virials,
                                  system_energies, workspace, workspace_bytes, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_repeat(const float* positions, const float* cells,
+                                                    const int32_t* neighbor_matrix,
+                                                    const int32_t* neighbor_matrix_shifts,
+                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
+                                                    const int32_t* row_order, double neighbor_list_cutoff,
+                                                    int32_t n_atoms, int32_t max_neighbors, int32_t n_systems,
+                                                    int32_t fill_value, double epsilon, double sigma, double cutoff,
+                                                    double switch_width, int32_t reuse_tables, float* atomic_energies,
+                                                    float* forces, float* virials, float* system_energies,
+                                                    void* workspace, size_t workspace_bytes, void* stream) {
+    return lj_energy_forces_impl(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors, batch_idx,
+                                 row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
+                                 sigma, cutoff, switch_width, /*half_list=*/0, atomic_energies, forces, virials,
+                                 system_energies, workspace, workspace_bytes, stream, reuse_tables ? 1 : 0);
 }
 
 // ---- the variant that allocates nothing ------------------------------------------------------

@@ -55,6 +55,7 @@ _SIGNATURES = {
     "nvamd_fire_step": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_lj_energy_forces_hinted": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
+    "nvamd_lj_energy_forces_repeat": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_static": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_vp] * 5),
     "nvamd_nl_atom_order": (_i32, [_vp, _c.c_size_t, _vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_segment_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
@@ -201,11 +202,15 @@ class _Workspaces:
         for (dev, stream, purpose), buf in list(self._bufs.items()):
             if dev == device.index and stream == from_stream:
                 self._bufs[(dev, to_stream, purpose)] = buf
+        # (what is known about the contents of a shared buffer goes with it)
+        if (device.index, from_stream) in _lj_tables:
+            _lj_tables[(device.index, to_stream)] = _lj_tables[(device.index, from_stream)]
 
     def unshare(self, device: torch.device, stream: int) -> None:
         """Forget every entry of ``stream`` (the buffers stay with whoever else holds them)."""
         for key in [k for k in self._bufs if k[0] == device.index and k[1] == stream]:
             del self._bufs[key]
+        _lj_tables.pop((device.index, stream), None)
 
 
 workspaces = _Workspaces()
@@ -351,6 +356,32 @@ def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, 
         return
     need = _size(lib.nvamd_lj_workspace_bytes, N, B, int(bool(half_list)))
     ws = workspaces.get(positions.device, "lj", need)
+    if not half_list:
+        # The per-system tables that the pair kernel keeps in this workspace depend on batch_idx, cells and the
+        # list's cutoff only: while those stand as they were at the previous call through the same buffer (same
+        # storage, no in-place write since: Torch's version counters), that call's tables are used again.
+        tables = (ws.data_ptr(), batch_idx.data_ptr(), batch_idx._version, cells.data_ptr(), cells._version, N, K, B,
+                  float(neighbor_list_cutoff), neighbor_matrix_shifts is None, virials is None, system_energies is None)
+        state = (positions.device.index, _stream(positions.device))
+        reuse = _lj_tables.get(state) == tables
+        _lj_tables[state] = tables
+        _check(lib.nvamd_lj_energy_forces_repeat(
+            _dev(positions, "positions", torch.float32, (N, 3)),
+            _dev(cells, "cells", torch.float32, (B, 3, 3)),
+            _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+            _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+            _dev(num_neighbors, "num_neighbors", torch.int32, (N,)),
+            _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+            _opt(row_order, "row_order", torch.int32, (N,)), float(neighbor_list_cutoff),
+            N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), float(switch_width),
+            int(reuse),
+            _dev(atomic_energies, "atomic_energies", torch.float32, (N,)),
+            _dev(forces, "forces", torch.float32, (N, 3)),
+            _opt(virials, "virials", torch.float32, (B, 9)),
+            _opt(system_energies, "system_energies", torch.float32, (B,)),
+            ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_repeat")
+        return
+    _lj_tables.pop((positions.device.index, _stream(positions.device)), None)  # (a half-list call writes the workspace its own way)
     _check(lib.nvamd_lj_energy_forces_hinted(
         _dev(positions, "positions", torch.float32, (N, 3)),
         _dev(cells, "cells", torch.float32, (B, 3, 3)),
@@ -367,6 +398,9 @@ def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, 
         _opt(system_energies, "system_energies", torch.float32, (B,)),
         ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_hinted")
 
+
+#: per (device, stream): what the pair kernel's tables in the "lj" workspace were last computed for
+_lj_tables: dict[tuple, tuple] = {}
 
 LJ_STATIC_MAX_SYSTEMS = 16384
 

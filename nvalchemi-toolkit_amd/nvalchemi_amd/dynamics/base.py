@@ -584,6 +584,9 @@ class BaseDynamics(HookRegistryMixin):
         for name in ("positions", "velocities", "forces", "energy", "atomic_masses", "batch_idx", "cell", "status"):
             t = getattr(batch, name, None)
             key.append((t.data_ptr(), tuple(t.shape)) if isinstance(t, torch.Tensor) else None)
+        for name in ("batch_idx", "cell"):  # (kernels keep tables derived from these: an in-place edit ends the replay)
+            t = getattr(batch, name, None)
+            key.append(t._version if isinstance(t, torch.Tensor) else None)
         for hook in self.hooks:
             fn = getattr(hook, "graph_key", None)
             key.append((id(hook), fn() if callable(fn) else None))

@@ -672,3 +672,61 @@ def test_fire2_step_matches_oracle_over_many_steps(masked):
         sel = bi == 2
         assert np.array_equal(tp.cpu().numpy()[sel], P[sel]) and np.array_equal(tv.cpu().numpy()[sel], V[sel])
         assert tdt.cpu().numpy()[2] == np.float32(0.02) and tcnt.cpu().numpy()[2] == 0
+
+
+def test_lj_tables_are_reused_while_the_batch_stands_and_recomputed_when_it_changes():
+    """An MD loop calls the pair kernel with the same batch_idx and cells step after step: the package then tells
+    the library to keep the per-system tables of the previous call (``nvamd_lj_energy_forces_repeat`` with
+    ``reuse_tables = 1``).  With positions that move from call to call, with the cells then edited in place, and
+    with another batch in between, every call must equal a call that computes its tables itself."""
+    from nvalchemi_amd import _lib
+
+    rc, eps, sig = 2.5, 1.0, 1.0
+    P, C, pb, ptr = periodic_batch(61, 5, 200, 500, 0.8)
+    bi = oracle.batch_idx_from_ptr(ptr)
+    N, B = len(P), len(ptr) - 1
+    rng = np.random.default_rng(8)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)  # noqa: E731
+    pos, cells, bidx, tptr, tpb = t(P), t(C), t(bi), t(ptr), t(pb)
+    K = 96
+    nm = torch.full((N, K), N, dtype=torch.int32, device=DEV)
+    nn = torch.zeros(N, dtype=torch.int32, device=DEV)
+    sh = torch.zeros(N, K, 3, dtype=torch.int32, device=DEV)
+
+    def both(hint):
+        _lib.nl_build(pos, cells, tpb, tptr, bidx, None, rc, K, False, 0, nm, nn, sh)
+        assert int(nn.max()) < K
+        out = []
+        for fn in (_lib.lj_energy_forces, _lib.lj_energy_forces_static):
+            e, f = torch.empty(N, device=DEV), torch.empty(N, 3, device=DEV)
+            es, w = torch.empty(B, device=DEV), torch.empty(B, 9, device=DEV)
+            kw = dict(half_list=False) if fn is _lib.lj_energy_forces else {}
+            fn(pos, cells, nm, sh, nn, bidx, N, eps, sig, rc, 0.0, **kw, atomic_energies=e, forces=f, virials=w,
+               system_energies=es, neighbor_list_cutoff=hint)
+            out.append((e.cpu(), f.cpu(), es.cpu(), w.cpu()))
+        (e1, f1, s1, w1), (e2, f2, s2, w2) = out
+        assert torch.equal(e1, e2) and torch.equal(f1, f2)
+        assert torch.allclose(s1, s2, rtol=1e-5, atol=1e-6) and torch.allclose(w1, w2, rtol=1e-5, atol=1e-5)
+
+    state = (torch.device(DEV).index, _lib._stream(torch.device(DEV)))
+    for hint in (rc, 0.0):
+        both(hint)
+        key = _lib._lj_tables[state]
+        for _ in range(3):  # positions move, the batch stands: the tables stand
+            pos.add_(torch.from_numpy(rng.normal(0, 0.02, P.shape).astype(np.float32)).to(DEV))
+            both(hint)
+            assert _lib._lj_tables[state] == key
+        cells.mul_(1.01)  # an in-place edit of the cells: the image decisions are made again
+        pos.mul_(1.01)
+        both(hint)
+        assert _lib._lj_tables[state] != key
+        # another batch through the same workspace in between
+        P2, C2, pb2, ptr2 = periodic_batch(62, 3, 100, 200, 0.8)
+        nm2, nn2, sh2 = oracle.nl_cell(P2, C2, pb2, ptr2, rc, 96)
+        bi2 = oracle.batch_idx_from_ptr(ptr2)
+        ref = oracle.lj_matrix(P2, C2, nm2, sh2, nn2, bi2, len(P2), eps, sig, rc)
+        got = gpu_lj(P2, C2, nm2, sh2, nn2, bi2, eps, sig, rc)
+        assert_close(got, ref, "other batch")
+        both(hint)
+        cells.div_(1.01)
+        pos.div_(1.01)
