@@ -49,12 +49,22 @@ class NeighborListHook:
         Stage the hook fires at (assigned at registration when ``None``).
     method : str | None
         Accepted for compatibility with the reference's strategy names.
+    min_image_skin : bool
+        How far an atom has moved since its system's last build.  ``False`` (default): the plain
+        displacement, so an atom that a wrap hook has moved by a lattice vector counts as moved and its
+        system is rebuilt (the rows that are kept hold integer shifts that belong to the coordinates they
+        were built from).  ``True``: the displacement reduced to the nearest image, as the reference does
+        (nvalchemi/hooks/neighbor_list.py:295-311): a wrap then triggers nothing, and the stored shifts of a
+        wrapped atom's pairs are stale until its system's next build.  Only for a consumer that does not
+        read the stored shifts of such systems (the pair kernel of this package derives them from the
+        positions where every width of the cell exceeds twice the search radius).
     """
 
     def __init__(self, config: NeighborConfig, skin: float = 0.0, max_neighbors: int | None = None,
-                 stage: Enum | None = None, method: str | None = None) -> None:
+                 stage: Enum | None = None, method: str | None = None, min_image_skin: bool = False) -> None:
         self.config = config
         self.skin = skin
+        self.min_image_skin = bool(min_image_skin)
         self.stage = stage
         self.method = method
         self._max_neighbors_override = max_neighbors
@@ -116,7 +126,7 @@ class NeighborListHook:
                 reference_positions=self._ref_positions, current_positions=positions,
                 batch_idx=batch.batch_idx, rebuild_flags=self._rebuild_flags,
                 skin_distance_threshold=self.skin / 2, update_reference_positions=True,
-                cell=None, pbc=None)
+                cell=cell if self.min_image_skin else None, pbc=pbc if self.min_image_skin else None)
 
         cutoff = self.config.cutoff + self.skin
         self._build(batch, cutoff, cell, pbc,

@@ -280,3 +280,48 @@ def test_skin_and_wrap_together_on_cells_whose_shifts_are_read():
         assert np.abs(a - b).max() < tol, (key, np.abs(a - b).max())
     d = (res[True].positions - res[False].positions).cpu().numpy().astype(np.float64) / 7.2
     assert np.abs(d - np.round(d)).max() < 1e-4
+
+
+def test_min_image_skin_keeps_lists_through_wraps_on_cells_whose_shifts_are_derived():
+    """Cells wider than twice the search radius (the pair kernel derives the shifts from the positions there)
+    with a Verlet skin, the wrap hook and ``min_image_skin=True``: a wrap is no displacement, so the lists are
+    kept through it (far fewer rebuilds than with the plain displacement), and the run is still the run without
+    the wrap, up to lattice vectors."""
+    from nvalchemi_amd.dynamics import NVE
+    from nvalchemi_amd.dynamics.base import DynamicsStage
+    from nvalchemi_amd.hooks import WrapPeriodicHook
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=4, n_boxes=3, reps=4, a=3.6)  # 14.4 wide: more than 2 (4.5 + 0.5)
+    N = len(P)
+    M = np.full(N, 63.546, dtype=np.float32)
+    V = np.tile(np.array([[0.35, -0.25, 0.15]], np.float32), (N, 1))  # a drift that carries atoms across the faces
+    V += np.random.default_rng(5).normal(0, 0.01, (N, 3)).astype(np.float32)
+    Z = np.full(N, 29, dtype=np.int64)
+    sig = float((3.6 / np.sqrt(2)) / 2 ** (1 / 6))
+    res, rebuilt = {}, {}
+    for mode in ("no wrap", "plain", "min image"):
+        batch = make_batch(P, Z, M, C, pb, ptr, V)
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=sig, cutoff=4.5)
+        hooks = model.make_neighbor_hooks()
+        for h in hooks:
+            h.skin = 0.5
+            h.min_image_skin = mode == "min image"
+        if mode != "no wrap":
+            hooks.append(WrapPeriodicHook(frequency=1, stage=DynamicsStage.AFTER_POST_UPDATE))
+        dyn = NVE(model, dt=2.0, hooks=hooks)
+        dyn.graph_replay = False
+        n = 0
+        for _ in range(100):
+            dyn.run(batch, n_steps=1)
+            n += int(hooks[0]._rebuild_flags.sum())
+        res[mode], rebuilt[mode] = batch, n
+    assert rebuilt["min image"] <= rebuilt["no wrap"] + 3 and rebuilt["plain"] > rebuilt["min image"] + 30
+    assert np.abs(res["no wrap"].positions.cpu().numpy() / 14.4).max() > 1.1  # atoms did leave the box
+    for mode in ("plain", "min image"):
+        for key, tol in (("forces", 2e-4), ("velocities", 2e-5)):
+            a = getattr(res[mode], key).cpu().numpy().astype(np.float64)
+            b = getattr(res["no wrap"], key).cpu().numpy().astype(np.float64)
+            assert np.abs(a - b).max() < tol, (mode, key, np.abs(a - b).max())
+        d = (res[mode].positions - res["no wrap"].positions).cpu().numpy().astype(np.float64) / 14.4
+        assert np.abs(d - np.round(d)).max() < 1e-4
