@@ -36,6 +36,13 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kTile = 1088;       // candidates staged in LDS at a time
 constexpr int kStencilBatch = 64; // stencil cells enumerated at a time (one per lane of a wave)
 constexpr int kCenterChunk = 72;  // centre atoms of a run of cells handled per pass
+#ifndef NVAMD_NL_CHUNK
+#define NVAMD_NL_CHUNK(n) center_chunk_for(n)
+#endif
+inline int center_chunk_for(int n_atoms) {
+    int c = n_atoms / 4096 / 8 * 8;
+    return c < 16 ? 16 : (c > kCenterChunk ? kCenterChunk : c);
+}
 constexpr int kMaxRun = 4;        // a workgroup's unit of work: up to this many cells in a row along z
 constexpr int kHitCap = 256;      // per-wave list of accepted candidates before it is written out
 constexpr int kPackOverflow = 1 << 15;
@@ -90,7 +97,7 @@ struct __attribute__((aligned(32))) NlUnit {
     int nc_pack;      // cells per axis minus one, 10 bits each: (nc0-1) | (nc1-1) << 10 | (nc2-1) << 20
     int rper_pack;    // stencil radii, 6 bits each, then the periodic flags: R0 | R1 << 6 | R2 << 12 | per << 18
     int cell_offset;  // first cell of the system
-    int first_centre; // the unit covers centre atoms first_centre .. +kCenterChunk of the run; -1: all of them
+    int first_centre; // -1: the unit covers all centre atoms of the run; else count << 24 | first: `count` of them from `first`
 };
 static_assert(sizeof(NlUnit) == 32, "read as two 16-byte words");
 static_assert(kMaxStencilRadius < 64, "stencil radii are packed 6 bits each");
@@ -168,6 +175,7 @@ struct NlArgs {
     const uint8_t* rebuild;
     int n_atoms, n_systems, K, half, tail_mode;
     int unit_group;  // units are dealt to the XCDs in groups of this many (a power of two)
+    int center_chunk;  // centre atoms per unit of work at most (<= kCenterChunk; smaller for small batches: more units)
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -328,7 +336,7 @@ __device__ __forceinline__ void choose_grid(NlSys& s, const NlArgs& a, const uin
             const int entries = (cand + 2 * s.R[2]) * e01;
             if (entries > kStencilBatch) break;
             if (entries * per_cell + kWave > (double)kTile) break;
-            if (cand * per_cell > (double)kCenterChunk) break;
+            if (cand * per_cell > (double)a.center_chunk) break;
             zr = cand;
         }
         const int runs = (s.nc[2] + zr - 1) / zr;
@@ -711,13 +719,14 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         auto first_atom = [&](int lc) {
             return in_lds ? s_hist[lc] : __hip_atomic_load(&g_start[lc], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         };
-        auto passes_of = [&](const NlUnit& u) {
+        auto centres_of = [&](const NlUnit& u) {
             const int lc0 = u.c0 - cell_base;
             const int n_centre = first_atom(lc0 + u.run_len) - first_atom(lc0);
-            return (n_centre + kCenterChunk - 1) / kCenterChunk;
+            return n_centre;
         };
+        auto passes_for = [&](int n_centre) { return (n_centre + a.center_chunk - 1) / a.center_chunk; };
         int mine_units = 0;
-        for (int lu = tid; lu < n_runs; lu += kSortBlock) mine_units += passes_of(make_unit(q, lu, runs, t));
+        for (int lu = tid; lu < n_runs; lu += kSortBlock) mine_units += passes_for(centres_of(make_unit(q, lu, runs, t)));
         int total;
         const int before = block_exclusive_scan(mine_units, s_part, &total);
         // a contiguous piece of the unit list, wherever the counter stands (the order of the
@@ -727,9 +736,11 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         NlUnit* out = ws.units + s_unit0 + before;
         for (int lu = tid; lu < n_runs; lu += kSortBlock) {
             NlUnit u = make_unit(q, lu, runs, t);
-            const int passes = passes_of(u);
+            const int n_centre = centres_of(u);
+            const int passes = passes_for(n_centre);
+            const int share = passes > 0 ? (n_centre + passes - 1) / passes : 0;  // equal shares, not full chunks and a rest
             for (int k = 0; k < passes; ++k) {
-                u.first_centre = passes > 1 ? k * kCenterChunk : -1;
+                u.first_centre = passes > 1 ? ((share << 24) | (k * share)) : -1;
                 *out++ = u;
             }
         }
@@ -939,8 +950,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
 
         // the run's centre atoms, one pass at a time; or the one pass this unit stands for
         const int first_centre = __builtin_amdgcn_readfirstlane(grid.w);
-        const int cc_begin = first_centre >= 0 ? first_centre : 0;
-        const int cc_end = (first_centre >= 0 && first_centre + kCenterChunk < n_center) ? first_centre + kCenterChunk : n_center;
+        const int cc_begin = first_centre >= 0 ? (first_centre & 0xffffff) : 0;
+        const int cc_share = first_centre >= 0 ? (first_centre >> 24) : n_center;
+        const int cc_end = (cc_begin + cc_share) < n_center ? (cc_begin + cc_share) : n_center;
         for (int cc0 = cc_begin; cc0 < cc_end; cc0 += kCenterChunk) {
             const int n_cc = (cc_end - cc0) < kCenterChunk ? (cc_end - cc0) : kCenterChunk;
             int pad_end = 0;
@@ -1350,6 +1362,8 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     a.tail_mode = tail_mode ? 1 : 0;
     a.unit_group = 1;
     while (a.unit_group < 64 && (long long)a.unit_group * 8192 <= (long long)n_atoms) a.unit_group *= 2;
+    // A small batch does not fill the chip with units of kCenterChunk centre atoms: smaller units, about 4096 of them
+    a.center_chunk = NVAMD_NL_CHUNK(n_atoms);
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
