@@ -330,7 +330,7 @@ int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells
  * double on the float64 positions.  The pair kernel's per-system energy is the sum of the float64 atomic
  * energies.  nvamd_f64_workspace_bytes(n_systems) serves nvamd_fire_step_f64, nvamd_segment_fmax_f64 and
  * nvamd_lj_energy_forces_f64 (which needs it only with virials or system_energies); the neighbor build uses
- * nvamd_nl_workspace_bytes.  Not built for float64: the Verlet-skin test, the wrap, the thermostats, FIRE 2.0.
+ * nvamd_nl_workspace_bytes.  Not built for float64: the thermostats, FIRE 2.0.
  * ---------------------------------------------------------------------------------------- */
 int32_t nvamd_nl_build_f64(const double* positions, const double* cell, const uint8_t* pbc,
                            const int32_t* batch_ptr, const int32_t* batch_idx, const uint8_t* rebuild_flags,
@@ -362,6 +362,12 @@ int32_t nvamd_fire_step_f64(double* positions, double* velocities, const double*
                             void* stream);
 int32_t nvamd_segment_fmax_f64(const double* forces, const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
                                double* fmax, void* workspace, size_t workspace_bytes, void* stream);
+int32_t nvamd_nl_rebuild_check_f64(double* reference_positions, const double* current_positions,
+                                   const int32_t* batch_idx, const double* cell, const uint8_t* pbc,
+                                   int32_t n_atoms, int32_t n_systems, double threshold,
+                                   int32_t update_reference, uint8_t* rebuild_flags, void* stream);
+int32_t nvamd_wrap_positions_f64(double* positions, const double* cell, const uint8_t* pbc,
+                                 const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems, void* stream);
 
 /* What the neighbor builds through this workspace had to report.  No counterpart in the reference, whose
  * kernels report nothing (a caller there compares num_neighbors with max_neighbors on the host:

@@ -18,10 +18,13 @@ __global__ __launch_bounds__(kBlock) void clear_flags_kernel(uint8_t* flags, int
     if (t < n) flags[t] = 0;
 }
 
-__global__ __launch_bounds__(kBlock) void displacement_kernel(const float* __restrict__ ref,
-                                                              const float* __restrict__ cur,
+// T: the type the positions and cells are stored in; the arithmetic is double either way (float32 inputs
+// convert exactly), and a float64 result is stored as it is.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void displacement_kernel(const T* __restrict__ ref,
+                                                              const T* __restrict__ cur,
                                                               const int32_t* __restrict__ bidx,
-                                                              const float* __restrict__ cell,
+                                                              const T* __restrict__ cell,
                                                               const uint8_t* __restrict__ pbc, int n_atoms,
                                                               double thr2, uint8_t* flags) {
 #pragma clang fp contract(off)
@@ -53,8 +56,9 @@ __global__ __launch_bounds__(kBlock) void displacement_kernel(const float* __res
     if (r2 > thr2) flags[s] = 1;  // (every writer stores the same byte)
 }
 
-__global__ __launch_bounds__(kBlock) void refresh_reference_kernel(float* __restrict__ ref,
-                                                                   const float* __restrict__ cur,
+template <typename T>
+__global__ __launch_bounds__(kBlock) void refresh_reference_kernel(T* __restrict__ ref,
+                                                                   const T* __restrict__ cur,
                                                                    const int32_t* __restrict__ bidx,
                                                                    const uint8_t* __restrict__ flags, size_t n3) {
     size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -62,7 +66,8 @@ __global__ __launch_bounds__(kBlock) void refresh_reference_kernel(float* __rest
     if (flags[bidx[t / 3]]) ref[t] = cur[t];
 }
 
-__global__ __launch_bounds__(kBlock) void wrap_kernel(float* __restrict__ pos, const float* __restrict__ cell,
+template <typename T>
+__global__ __launch_bounds__(kBlock) void wrap_kernel(T* __restrict__ pos, const T* __restrict__ cell,
                                                       const uint8_t* __restrict__ pbc,
                                                       const int32_t* __restrict__ bidx, int n_atoms) {
 #pragma clang fp contract(off)
@@ -75,7 +80,7 @@ __global__ __launch_bounds__(kBlock) void wrap_kernel(float* __restrict__ pos, c
 #pragma unroll
     for (int k = 0; k < 9; ++k) h[k] = (double)cell[9 * (size_t)s + k];
     inv3(h, hinv);
-    float* r = pos + 3 * (size_t)i;
+    T* r = pos + 3 * (size_t)i;
     const double x = (double)r[0], y = (double)r[1], z = (double)r[2];
     double f0 = (x * hinv[0] + y * hinv[3]) + z * hinv[6];
     double f1 = (x * hinv[1] + y * hinv[4]) + z * hinv[7];
@@ -87,9 +92,9 @@ __global__ __launch_bounds__(kBlock) void wrap_kernel(float* __restrict__ pos, c
     const double wy = (f0 * h[1] + f1 * h[4]) + f2 * h[7];
     const double wz = (f0 * h[2] + f1 * h[5]) + f2 * h[8];
     // the reference keeps the old Cartesian component wherever that component's flag is clear
-    if (p[0]) r[0] = (float)wx;
-    if (p[1]) r[1] = (float)wy;
-    if (p[2]) r[2] = (float)wz;
+    if (p[0]) r[0] = (T)wx;
+    if (p[1]) r[1] = (T)wy;
+    if (p[2]) r[2] = (T)wz;
 }
 
 }  // namespace
@@ -97,10 +102,10 @@ __global__ __launch_bounds__(kBlock) void wrap_kernel(float* __restrict__ pos, c
 
 using namespace nvamd;
 
-NVAMD_EXPORT int32_t nvamd_nl_rebuild_check(float* reference_positions, const float* current_positions,
-                                            const int32_t* batch_idx, const float* cell, const uint8_t* pbc,
-                                            int32_t n_atoms, int32_t n_systems, double threshold,
-                                            int32_t update_reference, uint8_t* rebuild_flags, void* stream) {
+template <typename T>
+static int32_t rebuild_check_impl(T* reference_positions, const T* current_positions, const int32_t* batch_idx,
+                                  const T* cell, const uint8_t* pbc, int32_t n_atoms, int32_t n_systems,
+                                  double threshold, int32_t update_reference, uint8_t* rebuild_flags, void* stream) {
     if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "rebuild check: negative size");
     if (!(threshold >= 0.0)) return fail(NVAMD_ERR_INVALID_ARGUMENT, "rebuild check: threshold must not be negative");
     if (n_systems == 0) return NVAMD_OK;
@@ -113,12 +118,12 @@ NVAMD_EXPORT int32_t nvamd_nl_rebuild_check(float* reference_positions, const fl
     if (n_atoms > 0) {
         if (!reference_positions || !current_positions || !batch_idx)
             return fail(NVAMD_ERR_INVALID_ARGUMENT, "rebuild check: null buffer");
-        hipLaunchKernelGGL(displacement_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+        hipLaunchKernelGGL(displacement_kernel<T>, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
                            reference_positions, current_positions, batch_idx, cell, pbc, n_atoms,
                            threshold * threshold, rebuild_flags);
         if (update_reference) {
             const size_t n3 = 3 * (size_t)n_atoms;
-            hipLaunchKernelGGL(refresh_reference_kernel, dim3((unsigned)((n3 + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+            hipLaunchKernelGGL(refresh_reference_kernel<T>, dim3((unsigned)((n3 + kBlock - 1) / kBlock)), dim3(kBlock), 0,
                                st, reference_positions, current_positions, batch_idx, rebuild_flags, n3);
         }
     }
@@ -126,14 +131,42 @@ NVAMD_EXPORT int32_t nvamd_nl_rebuild_check(float* reference_positions, const fl
     return NVAMD_OK;
 }
 
-NVAMD_EXPORT int32_t nvamd_wrap_positions(float* positions, const float* cell, const uint8_t* pbc,
-                                          const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
-                                          void* stream) {
+template <typename T>
+static int32_t wrap_impl(T* positions, const T* cell, const uint8_t* pbc, const int32_t* batch_idx, int32_t n_atoms,
+                         int32_t n_systems, void* stream) {
     if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "wrap: negative size");
     if (n_atoms == 0 || n_systems == 0) return NVAMD_OK;
     if (!positions || !cell || !pbc || !batch_idx) return fail(NVAMD_ERR_INVALID_ARGUMENT, "wrap: null buffer");
-    hipLaunchKernelGGL(wrap_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0,
+    hipLaunchKernelGGL(wrap_kernel<T>, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0,
                        static_cast<hipStream_t>(stream), positions, cell, pbc, batch_idx, n_atoms);
     NVAMD_LAUNCH_CHECK("wrap launch");
     return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_rebuild_check(float* reference_positions, const float* current_positions,
+                                            const int32_t* batch_idx, const float* cell, const uint8_t* pbc,
+                                            int32_t n_atoms, int32_t n_systems, double threshold,
+                                            int32_t update_reference, uint8_t* rebuild_flags, void* stream) {
+    return rebuild_check_impl<float>(reference_positions, current_positions, batch_idx, cell, pbc, n_atoms, n_systems,
+                                     threshold, update_reference, rebuild_flags, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_rebuild_check_f64(double* reference_positions, const double* current_positions,
+                                                const int32_t* batch_idx, const double* cell, const uint8_t* pbc,
+                                                int32_t n_atoms, int32_t n_systems, double threshold,
+                                                int32_t update_reference, uint8_t* rebuild_flags, void* stream) {
+    return rebuild_check_impl<double>(reference_positions, current_positions, batch_idx, cell, pbc, n_atoms, n_systems,
+                                      threshold, update_reference, rebuild_flags, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_wrap_positions(float* positions, const float* cell, const uint8_t* pbc,
+                                          const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
+                                          void* stream) {
+    return wrap_impl<float>(positions, cell, pbc, batch_idx, n_atoms, n_systems, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_wrap_positions_f64(double* positions, const double* cell, const uint8_t* pbc,
+                                              const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems,
+                                              void* stream) {
+    return wrap_impl<double>(positions, cell, pbc, batch_idx, n_atoms, n_systems, stream);
 }

@@ -63,6 +63,8 @@ _SIGNATURES = {
     "nvamd_kinetic_energy": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_nl_rebuild_check": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_nl_rebuild_check_f64": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
+    "nvamd_wrap_positions_f64": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_langevin_half_step": (_i32, [_vp] * 7 + [_c.c_uint64, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_fire2_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_fire2_step": (_i32, [_vp] * 11 + [_i32] + [_c.c_double] * 7 + [_vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
@@ -527,11 +529,13 @@ def nl_rebuild_check(reference_positions, current_positions, batch_idx, rebuild_
     M = rebuild_flags.shape[0]
     if (cell is None) != (pbc is None):
         cell = pbc = None  # the displacement is plain unless both are given
-    _check(library().nvamd_nl_rebuild_check(
-        _dev(reference_positions, "reference_positions", torch.float32, (N, 3)),
-        _dev(current_positions, "current_positions", torch.float32, (N, 3)),
+    real = _real_dtype(current_positions, "current_positions")
+    entry = library().nvamd_nl_rebuild_check_f64 if real == torch.float64 else library().nvamd_nl_rebuild_check
+    _check(entry(
+        _dev(reference_positions, "reference_positions", real, (N, 3)),
+        _dev(current_positions, "current_positions", real, (N, 3)),
         _dev(batch_idx, "batch_idx", torch.int32, (N,)),
-        _opt(cell, "cell", torch.float32, (M, 3, 3)), _opt(_as_u8(pbc), "pbc", torch.uint8, (M, 3)),
+        _opt(cell, "cell", real, (M, 3, 3)), _opt(_as_u8(pbc), "pbc", torch.uint8, (M, 3)),
         N, M, float(threshold), int(bool(update_reference)),
         _dev(_as_u8(rebuild_flags), "rebuild_flags", torch.uint8, (M,)),
         _stream(current_positions.device)), "nvamd_nl_rebuild_check")
@@ -540,8 +544,10 @@ def nl_rebuild_check(reference_positions, current_positions, batch_idx, rebuild_
 def wrap_positions(positions, cell, pbc, batch_idx) -> None:
     N = positions.shape[0]
     M = cell.shape[0]
-    _check(library().nvamd_wrap_positions(
-        _dev(positions, "positions", torch.float32, (N, 3)), _dev(cell, "cell", torch.float32, (M, 3, 3)),
+    real = _real_dtype(positions, "positions")
+    entry = library().nvamd_wrap_positions_f64 if real == torch.float64 else library().nvamd_wrap_positions
+    _check(entry(
+        _dev(positions, "positions", real, (N, 3)), _dev(cell, "cell", real, (M, 3, 3)),
         _dev(_as_u8(pbc), "pbc", torch.uint8, (M, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         N, M, _stream(positions.device)), "nvamd_wrap_positions")
 

@@ -34,9 +34,9 @@ def _(positions, cell, pbc, batch_idx) -> None:
 def wrap_positions_into_cell(positions: torch.Tensor, cell: torch.Tensor, pbc: torch.Tensor,
                              batch_idx: torch.Tensor) -> torch.Tensor:
     """Wrap ``positions`` (V, 3) in place and return the same tensor."""
-    if positions.dtype != torch.float32:
-        raise TypeError("wrap_positions_into_cell: float32 positions only")
-    _wrap_positions_(positions, cell.to(torch.float32).contiguous(), pbc.to(torch.bool).contiguous(),
+    if positions.dtype not in (torch.float32, torch.float64):
+        raise TypeError("wrap_positions_into_cell: float32 or float64 positions")
+    _wrap_positions_(positions, cell.to(positions.dtype).contiguous(), pbc.to(torch.bool).contiguous(),
                      batch_idx.to(torch.int32))
     return positions
 

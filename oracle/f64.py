@@ -11,13 +11,22 @@ one IEEE operation per numpy operation (numpy does not fuse multiply-adds):
 * ``vv_pre/vv_post``  nvalchemi/dynamics/_ops/velocity_verlet.py:50-92, 102-138
 * ``fire_step``       nvalchemi/dynamics/_ops/fire.py:245-362, order of :270-272
 * ``fmax``            nvalchemi/dynamics/base.py:304-349
+* ``rebuild_check``   nvalchemi/dynamics/_ops/neighbor_list_rebuild.py:37-139 (flags cleared, then set for
+                      systems with an atom displaced by more than the threshold, strictly; nearest image on
+                      periodic axes when the cell is given; the whole flagged system's reference refreshed)
+* ``wrap_positions``  nvalchemi/hooks/periodic.py:42-114, 159-163 (fractional coordinates mod 1, back to
+                      Cartesian, per Cartesian component where that component's pbc flag is set)
 
 Pinned (tests/test_oracle_f64.py) against the float32 oracle on inputs that float32 holds exactly
 (where both must agree: to the bit for the neighbor sets, to float32 rounding elsewhere), against
 closed forms in double (the Lennard-Jones dimer, F = -dE/dr by finite differences at 1e-9, the
 discrete harmonic oscillator), and by pairs that only double resolves around the cutoff.  What the
 float32 oracle leaves unpinned against the reference (FIRE's order beyond the reference's sentences,
-the switching polynomial, the energy at the cutoff) is unpinned here in the same way.
+the switching polynomial, the energy at the cutoff; for the skin test: strictness, the nearest-image form,
+the whole-system refresh) is unpinned here in the same way.  ``rebuild_check`` and ``wrap_positions`` are
+pinned against the float32 oracle on inputs float32 holds exactly and by what the definitions fix (a wrapped
+position lies in the cell and differs from the old one by whole lattice vectors; a displacement of
+``threshold (1 +- 1e-12)``, which float32 cannot tell from the threshold, lands on the right side).
 """
 
 from __future__ import annotations
@@ -215,3 +224,71 @@ def fmax(forces, batch_idx, n_systems: int) -> np.ndarray:
     out = np.full(n_systems, -np.inf)
     np.maximum.at(out, np.asarray(batch_idx).astype(np.int64), n)
     return out
+
+
+def _inv3(h):
+    """The adjugate-over-determinant inverse in the operation order of oracle/md_oracle.c (orc_inv3)."""
+    m = np.asarray(h, dtype=np.float64).reshape(9)
+    c00 = m[4] * m[8] - m[5] * m[7]
+    c01 = m[5] * m[6] - m[3] * m[8]
+    c02 = m[3] * m[7] - m[4] * m[6]
+    det = m[0] * c00 + m[1] * c01 + m[2] * c02
+    i = 1.0 / det
+    return np.array([c00 * i, (m[2] * m[7] - m[1] * m[8]) * i, (m[1] * m[5] - m[2] * m[4]) * i,
+                     c01 * i, (m[0] * m[8] - m[2] * m[6]) * i, (m[2] * m[3] - m[0] * m[5]) * i,
+                     c02 * i, (m[1] * m[6] - m[0] * m[7]) * i, (m[0] * m[4] - m[1] * m[3]) * i])
+
+
+def rebuild_check(reference_positions, current_positions, batch_idx, n_systems: int, threshold: float,
+                  update_reference: bool = False, cell=None, pbc=None) -> np.ndarray:
+    """Flags ``(M,) uint8``; ``reference_positions`` (float64, C-contiguous) is refreshed in place for the atoms
+    of flagged systems when ``update_reference``."""
+    ref = reference_positions
+    assert ref.dtype == np.float64
+    cur = np.asarray(current_positions, dtype=np.float64)
+    bi = np.asarray(batch_idx, dtype=np.int64)
+    flags = np.zeros(int(n_systems), dtype=np.uint8)
+    thr2 = float(threshold) * float(threshold)
+    for i in range(len(cur)):
+        s = bi[i]
+        d = cur[i] - ref[i]
+        if cell is not None and pbc is not None and np.any(pbc[s]):
+            h = np.asarray(cell[s], dtype=np.float64).reshape(9)
+            hv = _inv3(h)
+            f = np.array([(d[0] * hv[0] + d[1] * hv[3]) + d[2] * hv[6],
+                          (d[0] * hv[1] + d[1] * hv[4]) + d[2] * hv[7],
+                          (d[0] * hv[2] + d[1] * hv[5]) + d[2] * hv[8]])
+            for k in range(3):
+                if pbc[s][k]:
+                    f[k] -= np.rint(f[k])
+            d = np.array([(f[0] * h[0] + f[1] * h[3]) + f[2] * h[6],
+                          (f[0] * h[1] + f[1] * h[4]) + f[2] * h[7],
+                          (f[0] * h[2] + f[1] * h[5]) + f[2] * h[8]])
+        if (d[0] * d[0] + d[1] * d[1]) + d[2] * d[2] > thr2:
+            flags[s] = 1
+    if update_reference:
+        hit = flags[bi] != 0
+        ref[hit] = cur[hit]
+    return flags
+
+
+def wrap_positions(positions, cell, pbc, batch_idx) -> np.ndarray:
+    """Wrapped copy of ``positions`` (float64)."""
+    pos = np.array(positions, dtype=np.float64)
+    bi = np.asarray(batch_idx, dtype=np.int64)
+    for i in range(len(pos)):
+        s = bi[i]
+        if not np.any(pbc[s]):
+            continue
+        h = np.asarray(cell[s], dtype=np.float64).reshape(9)
+        hv = _inv3(h)
+        x, y, z = pos[i]
+        f = np.array([(x * hv[0] + y * hv[3]) + z * hv[6], (x * hv[1] + y * hv[4]) + z * hv[7],
+                      (x * hv[2] + y * hv[5]) + z * hv[8]])
+        f -= np.floor(f)
+        w = np.array([(f[0] * h[0] + f[1] * h[3]) + f[2] * h[6], (f[0] * h[1] + f[1] * h[4]) + f[2] * h[7],
+                      (f[0] * h[2] + f[1] * h[5]) + f[2] * h[8]])
+        for k in range(3):
+            if pbc[s][k]:
+                pos[i, k] = w[k]
+    return pos

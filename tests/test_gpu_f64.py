@@ -215,3 +215,44 @@ def test_a_float64_batch_runs_through_the_package_api():
         if k == 0:
             e0 = b2.energy.clone()
     assert b2.energy.dtype == F64 and bool((b2.energy < e0).all())
+
+
+def test_skin_test_and_wrap_on_float64_arrays():
+    """The Verlet-skin displacement test and the periodic wrap on float64 arrays against the float64 oracle:
+    flags and refreshed references to the bit, wrapped positions to the bit (both sides compute in double, one
+    operation at a time), and a displacement of threshold (1 +- 1e-12) on the right side."""
+    from nvalchemi_amd import _lib
+    from nvalchemi_amd.hooks.periodic import wrap_positions_into_cell
+
+    P, C, pb, ptr = periodic_batch(7, 3, 30, 60, 0.05, triclinic=True)
+    pb = pb.copy()
+    pb[1] = [1, 0, 1]
+    bi = oracle.batch_idx_from_ptr(ptr)
+    B = len(ptr) - 1
+    rng = np.random.default_rng(7)
+    P64 = P.astype(np.float64) + rng.normal(0, 1e-9, P.shape)       # values float32 does not hold
+    C64 = C.astype(np.float64) * (1 + 1e-10)
+    cur = P64.copy()
+    moved = bi != 2
+    cur[moved] += rng.normal(0, 0.08, (int(moved.sum()), 3))
+    cur[0] += 2 * C64[0][0] - C64[0][1]
+    for cell, pbc in ((None, None), (C64, pb)):
+        for thr in (0.05, 0.2, 0.6):
+            ref = P64.copy()
+            want = f64.rebuild_check(ref, cur, bi, B, thr, update_reference=True, cell=cell, pbc=pbc)
+            ref_t, flags = T(P64), torch.ones(B, dtype=torch.bool, device=DEV)
+            _lib.nl_rebuild_check(ref_t, T(cur), T(bi), flags, thr, True, None if cell is None else T(C64),
+                                  None if pbc is None else T(pb).bool())
+            assert np.array_equal(flags.cpu().numpy(), want.astype(bool))
+            assert np.array_equal(ref_t.cpu().numpy(), ref)
+    thr = 0.25
+    for eps, want in ((+1e-12, True), (-1e-12, False)):
+        c2 = np.zeros((2, 3))
+        c2[1] = np.array([0.6, 0.0, 0.8]) * thr * (1 + eps)
+        flags = torch.zeros(1, dtype=torch.bool, device=DEV)
+        _lib.nl_rebuild_check(T(np.zeros((2, 3))), T(c2), T(np.zeros(2, dtype=np.int32)), flags, thr, False)
+        assert bool(flags[0]) == want
+    far = cur * 3.0 - 5.0
+    want = f64.wrap_positions(far, C64, pb, bi)
+    got = wrap_positions_into_cell(T(far), T(C64), T(pb).bool(), T(bi))
+    assert got.dtype == torch.float64 and np.array_equal(got.cpu().numpy(), want)

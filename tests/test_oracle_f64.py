@@ -138,3 +138,68 @@ def test_fmax_in_double():
     f = np.array([[3.0, 4.0, 0.0], [0.0, 0.0, 1e-200], [1.0, 2.0, 2.0]])
     out = f64.fmax(f, np.array([0, 0, 2], np.int32), 3)
     assert out[0] == 5.0 and out[1] == -np.inf and out[2] == 3.0
+
+
+def _skin_case(seed=7):
+    """Three triclinic boxes with mixed periodic flags, float32-exact values: a reference, a current
+    configuration with a few atoms pushed across faces, one system left as it was."""
+    P, C, pb, ptr = periodic_batch(seed, 3, 30, 60, 0.05, triclinic=True)
+    pb = pb.copy()
+    pb[1] = [1, 0, 1]
+    bi = oracle.batch_idx_from_ptr(ptr)
+    rng = np.random.default_rng(seed)
+    cur = P.copy()
+    moved = bi != 2
+    cur[moved] += rng.normal(0, 0.08, (int(moved.sum()), 3)).astype(np.float32)
+    cur[0] += (2 * C[0][0] - C[0][1]).astype(np.float32)  # a lattice translation: no displacement on periodic axes
+    return P, cur, C, pb, ptr, bi
+
+
+def test_skin_test_in_double_equals_the_float32_oracle_on_float32_inputs():
+    P, cur, C, pb, ptr, bi = _skin_case()
+    B = len(ptr) - 1
+    for cell, pbc in ((None, None), (C, pb)):
+        for thr in (0.05, 0.2, 0.5):
+            f32, ref32 = oracle.rebuild_check(P, cur, bi, B, thr, update_reference=True, cell=cell, pbc=pbc)
+            ref64 = P.astype(np.float64)
+            got = f64.rebuild_check(ref64, cur.astype(np.float64), bi, B, thr, update_reference=True,
+                                    cell=None if cell is None else cell.astype(np.float64), pbc=pbc)
+            assert np.array_equal(got.astype(bool), f32)
+            assert np.array_equal(ref64, ref32.astype(np.float64))  # the same systems were refreshed
+    # with the cell, the lattice translation of atom 0 does not flag system 0 at a threshold above the jitter
+    assert f64.rebuild_check(P.astype(np.float64), cur.astype(np.float64), bi, B, 0.6, cell=C.astype(np.float64), pbc=pb)[0] == 0
+    assert f64.rebuild_check(P.astype(np.float64), cur.astype(np.float64), bi, B, 0.6)[0] == 1
+
+
+def test_skin_test_resolves_what_only_double_resolves():
+    """A displacement of threshold (1 +- 1e-12): float32 cannot tell either from the threshold."""
+    ref = np.zeros((2, 3))
+    thr = 0.25
+    for eps, want in ((+1e-12, 1), (-1e-12, 0)):
+        cur = ref.copy()
+        cur[1] = np.array([0.6, 0.0, 0.8]) * thr * (1 + eps)
+        assert f64.rebuild_check(ref.copy(), cur, [0, 0], 1, thr)[0] == want
+
+
+def test_wrap_in_double():
+    P, cur, C, pb, ptr, bi = _skin_case(9)
+    far = (cur.astype(np.float64) * 3.0 - 5.0)  # well outside the cells
+    W = f64.wrap_positions(far, C.astype(np.float64), pb, bi)
+    for s in range(len(ptr) - 1):
+        a, b = ptr[s], ptr[s + 1]
+        H = C[s].astype(np.float64)
+        moved = (W[a:b] - far[a:b]) @ np.linalg.inv(H)
+        if pb[s].all():
+            frac = W[a:b] @ np.linalg.inv(H)
+            assert frac.min() > -1e-12 and frac.max() < 1 + 1e-12          # inside the cell
+            assert np.abs(moved - np.round(moved)).max() < 1e-9            # moved by whole lattice vectors
+    # float32-exact inputs: the float32 oracle's result is this one rounded once
+    W32 = oracle.wrap_positions(cur, C, pb, bi)
+    W64 = f64.wrap_positions(cur.astype(np.float64), C.astype(np.float64), pb, bi)
+    assert np.array_equal(W64.astype(np.float32), W32)
+    # an open system is left alone; a Cartesian component whose flag is clear is kept
+    pb0 = pb.copy()
+    pb0[2] = 0
+    W0 = f64.wrap_positions(far, C.astype(np.float64), pb0, bi)
+    assert np.array_equal(W0[ptr[2]:ptr[3]], far[ptr[2]:ptr[3]])
+    assert np.array_equal(W[ptr[1]:ptr[2], 1], far[ptr[1]:ptr[2], 1])
