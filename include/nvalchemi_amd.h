@@ -298,6 +298,26 @@ int32_t nvamd_lj_energy_forces_repeat(const float* positions, const float* cells
                                       float* system_energies, void* workspace, size_t workspace_bytes,
                                       void* stream);
 
+/* nvamd_lj_energy_forces_repeat with the outputs of nvamd_nl_pair_hints for the same positions (all three
+ * given, or all three null: then this is nvamd_lj_energy_forces_repeat).  No counterpart in the reference.
+ * The rows are walked in row_order, 64 at a time; where a round has a hint, the atoms of its slices are read
+ * from ordered_positions (contiguous reads) into a table in LDS keyed by atom index, and the pair arithmetic
+ * finds its neighbors there instead of gathering each from memory.  Used for batches of more than 4096 atoms
+ * per system on average, in cells without off-diagonal terms that are wider than twice neighbor_list_cutoff;
+ * everything else takes the paths of the other entry points.  Results are those of the other entry points. */
+int32_t nvamd_lj_energy_forces_rounds(const float* positions, const float* cells,
+                                      const int32_t* neighbor_matrix,
+                                      const int32_t* neighbor_matrix_shifts,
+                                      const int32_t* num_neighbors, const int32_t* batch_idx,
+                                      const int32_t* row_order, const float* ordered_positions,
+                                      const int32_t* round_segments, const int32_t* round_counts,
+                                      double neighbor_list_cutoff, int32_t n_atoms, int32_t max_neighbors,
+                                      int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
+                                      double cutoff, double switch_width, int32_t reuse_tables,
+                                      float* atomic_energies, float* forces, float* virials,
+                                      float* system_energies, void* workspace, size_t workspace_bytes,
+                                      void* stream);
+
 /* nvamd_lj_energy_forces_hinted for callers that cannot allocate device memory or carry a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
  * the reference.  The scratch of the pair kernel (per-system float64 accumulators, first and last atom of
@@ -391,6 +411,24 @@ int32_t nvamd_nl_status(void* workspace, size_t workspace_bytes, int32_t n_atoms
 int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
                             const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
                             int32_t* atom_order, void* stream);
+
+/* What the pair kernel can take over from a neighbor build for systems too large for it to stage whole (more
+ * than 4096 atoms per system on average: only then does a build keep what this call reads; otherwise every
+ * count comes back as -1).  No counterpart in the reference.  From the build that last used this workspace with
+ * the same n_atoms / n_systems:
+ *   atom_order (N) i32             as nvamd_nl_atom_order
+ *   ordered_positions (N,4) f32    the float32 coordinates of atom_order[k] as the build read them, and the
+ *                                  bits of atom_order[k] in the fourth word
+ *   round_counts (R) i32, round_segments (R, NVAMD_PAIR_ROUND_SEGMENTS, 2) i32, R = ceil(N / 64):
+ *                                  for round w, the rows 64 w .. 64 w + 63 of the cell order, round_counts[w]
+ *                                  pairs (first, length) of slices of that order which together hold every atom
+ *                                  in the stencil of the round's cells, hence every neighbor of the round's
+ *                                  atoms within the build's cutoff; -1: no hint for this round
+ * Valid for the positions of that build only. */
+#define NVAMD_PAIR_ROUND_SEGMENTS 40
+int32_t nvamd_nl_pair_hints(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
+                            int32_t n_atoms, int32_t n_systems, int32_t* atom_order, float* ordered_positions,
+                            int32_t* round_segments, int32_t* round_counts, void* stream);
 
 /* Per-system reductions of a per-atom float32 vector: replace the Warp launches behind
  * nvalchemi_hooks::segmented_sum / _max / _min / _mean (nvalchemi/dynamics/hooks/_utils.py:58-136;

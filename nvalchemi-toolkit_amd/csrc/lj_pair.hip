@@ -21,6 +21,9 @@
 #include "common.h"
 #include "geom.h"
 
+#ifndef NVAMD_LJ_HASH_ROWS
+#define NVAMD_LJ_HASH_ROWS 512
+#endif
 #ifndef NVAMD_LJ_UNROLL
 #define NVAMD_LJ_UNROLL 4
 #endif
@@ -543,6 +546,293 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
     }
 }
 
+// ---- systems too large to stage: the neighborhood of a round of rows, staged by hash -----------------
+// A system that does not fit the LDS stage is walked in the cell order of the neighbor build (row_order), 64 rows
+// to a round: atoms of a few adjacent cells, whose neighbors all lie in the stencil of those cells.  The build
+// names that stencil per round as a few slices of the cell order (nvamd_nl_pair_hints) and leaves the atoms'
+// coordinates in that order, so a round reads its whole neighborhood with contiguous loads, enters each atom into
+// a hash table in LDS under its index (open addressing), and the pair arithmetic finds its neighbors there:
+// no gather from memory per listed pair (which fetches a cache line for twelve bytes, from all over the array).
+// Cells without off-diagonal terms whose images follow from the positions (img == 2) only; any other system, a
+// round without a hint, and a round whose neighborhood overflows the table take the unstaged row loop.
+constexpr int kHashSlots = 4096;   // keys (16 KB) and xyz (48 KB), in buckets of four slots
+constexpr int kHashBuckets = kHashSlots / 4;
+constexpr int kHashProbes = 12;    // buckets looked at before the table is taken to be as good as full
+constexpr int kHashLpr = 8;        // lanes per row
+constexpr int kHashRows = kBlockFull / kHashLpr;  // rows of a round
+constexpr int kHashStage = 4;      // atoms of the neighborhood a thread has in flight at a time
+static_assert(kHashRows == 64, "nvamd_nl_pair_hints describes rounds of 64 rows");
+
+__device__ __forceinline__ unsigned hash_bucket(int j) { return ((unsigned)j * 0x9E3779B1u) >> 22; }
+static_assert(kHashBuckets == 1 << 10, "the hash keeps the top ten bits");
+
+struct LjRounds {
+    const float4* ordered;   // (N) coordinates in row order + atom index bits
+    const int2* segments;    // (R, NVAMD_PAIR_ROUND_SEGMENTS)
+    const int32_t* counts;   // (R)
+};
+
+template <bool VIRIAL, bool SYS>
+__global__ __launch_bounds__(kBlockFull, 4) void lj_hashed_kernel(
+    LjArgs a, LjRounds hints, const int32_t* __restrict__ bidx_ro, const int32_t* __restrict__ order_ro,
+    const int32_t* __restrict__ first_ro, const int32_t* __restrict__ last_ro, const float* __restrict__ cells_ro,
+    const LjSysImage* __restrict__ image_ro) {
+    constexpr int NV = VIRIAL ? 7 : 1;
+    constexpr int LPR = kHashLpr, G = kHashRows, UNROLL = 8;
+    __shared__ double s_acc[kSysSlots][NV];
+    __shared__ __align__(16) int s_keys[kHashSlots];  // atom index per slot, -1: free; a bucket is four consecutive slots
+    __shared__ float s_xyz[3 * kHashSlots];
+    __shared__ int s_seg_first[64];
+    __shared__ int s_seg_prefix[65];
+    __shared__ double s_shift[27][3];
+    __shared__ int s_overflow;
+
+    const unsigned lb = xcd_contiguous_block(blockIdx.x, a.n_blocks);
+    if (lb >= a.n_blocks) return;
+    const int row0 = (int)lb * a.rows_per_block;
+    const int row_end = (row0 + a.rows_per_block) < a.n_atoms ? (row0 + a.rows_per_block) : a.n_atoms;
+    if (row0 >= row_end) return;
+    const int sys_lo = bidx_ro[order_ro[row0]];
+    if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
+    const int g = threadIdx.x / LPR, sub = threadIdx.x % LPR;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+
+    for (int r = row0; r < row_end;) {
+        const int sys = bidx_ro[order_ro[r]];
+        const int span0 = first_ro[sys], span_end = last_ro[sys];
+        const bool range_ok = span0 <= r && r < span_end;
+        const int seg_end = (range_ok && span_end < row_end) ? span_end : row_end;
+        const LjSysImage& image = image_ro[sys];
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        if (tid < 27) {
+            const int t = tid;
+            shift_vector(cells_ro + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
+                         s_shift[t][2]);
+        }
+        if (image.img != 2) {
+            // (not this kernel's case: the row loop of the staged kernel, without a stage)
+            __syncthreads();
+            if (image.img == 1)
+                lj_rows<LPR, VIRIAL, true, SYS, false, true, 1, false>(a, r, seg_end, sys_lo, nullptr, 0, 0, s_shift, sys,
+                                                                       image.hinv, image.diag, s_acc);
+            else
+                lj_rows<LPR, VIRIAL, true, SYS, false, true, 0, false>(a, r, seg_end, sys_lo, nullptr, 0, 0, s_shift, sys,
+                                                                       image.hinv, image.diag, s_acc);
+            r = seg_end;
+            if (r < row_end) __syncthreads();
+            continue;
+        }
+        double hd[3], hdi[3];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            hd[k] = uniform_double(image.diag + k);
+            hdi[k] = uniform_double(image.diag + 3 + k);
+        }
+        // rounds are the 64-slot windows of the row order, cut at the ends of the system's rows in this workgroup
+        for (int round0 = r; round0 < seg_end;) {
+            const int window = round0 / G;
+            const int round_end = ((window + 1) * G) < seg_end ? ((window + 1) * G) : seg_end;
+            const int n_seg = hints.counts[window];
+            // ---- an empty table, and where each of the round's slices begins in the flat numbering of its atoms
+            for (int t = tid; t < kHashSlots; t += kBlockFull) s_keys[t] = -1;
+            if (tid == 0) s_overflow = n_seg < 0 ? 1 : 0;
+            if (wave == 0) {
+                int2 piece = make_int2(0, 0);
+                if (lane < n_seg) piece = hints.segments[(size_t)window * NVAMD_PAIR_ROUND_SEGMENTS + lane];
+                int incl = piece.y;
+#pragma unroll
+                for (int o = 1; o < kWave; o <<= 1) {
+                    const int up = __shfl_up(incl, o, kWave);
+                    if (lane >= o) incl += up;
+                }
+                s_seg_first[lane] = piece.x;
+                s_seg_prefix[lane] = incl - piece.y;
+                if (lane == kWave - 1) s_seg_prefix[kWave] = incl;
+            }
+            __syncthreads();
+            // ---- the neighborhood into the table: a thread takes atoms t, t + 512, ... of the flat numbering, with
+            //      kHashStage loads in flight before the first of them is entered
+            const int n_hood = s_seg_prefix[kWave];
+            for (int base = 0; base < n_hood; base += kHashStage * kBlockFull) {
+                float4 p[kHashStage];
+#pragma unroll
+                for (int q = 0; q < kHashStage; ++q) {
+                    const int flat = base + q * kBlockFull + tid;
+                    const int f = flat < n_hood ? flat : n_hood - 1;
+                    int sg = 0;  // the slice that holds flat atom f
+#pragma unroll
+                    for (int step = kWave / 2; step > 0; step >>= 1)
+                        if (s_seg_prefix[sg + step] <= f) sg += step;
+                    p[q] = hints.ordered[s_seg_first[sg] + (f - s_seg_prefix[sg])];
+                }
+#pragma unroll
+                for (int q = 0; q < kHashStage; ++q) {
+                    if (base + q * kBlockFull + tid >= n_hood) continue;
+                    const int j = __float_as_int(p[q].w);
+                    unsigned b = hash_bucket(j);
+                    bool placed = false;
+                    for (int probes = 0; probes < kHashProbes && !placed; ++probes) {
+#pragma unroll
+                        for (int k = 0; k < 4 && !placed; ++k) {
+                            const int old = atomicCAS(&s_keys[4 * b + k], -1, j);
+                            if (old == -1) {
+                                float* at = s_xyz + 3 * (4 * b + k);
+                                at[0] = p[q].x; at[1] = p[q].y; at[2] = p[q].z;
+                                placed = true;
+                            } else if (old == j) {
+                                placed = true;  // (the same atom through two slices: it is there already)
+                            }
+                        }
+                        b = (b + 1) & (kHashBuckets - 1);
+                    }
+                    if (!placed) s_overflow = 1;
+                }
+            }
+            __syncthreads();
+            if (s_overflow) {
+                // no hint, or more atoms than the table takes: this round's neighbors straight from memory
+                lj_rows<LPR, VIRIAL, true, SYS, false, true, 2, false>(a, round0, round_end, sys_lo, nullptr, 0, 0, s_shift,
+                                                                       sys, image.hinv, image.diag, s_acc);
+                __syncthreads();
+                round0 = round_end;
+                continue;
+            }
+            // ---- the pair arithmetic, neighbors through the table
+            const int k_row = round0 + g;
+            if (k_row < round_end) {
+                const float4 me = hints.ordered[k_row];
+                const int i = __float_as_int(me.w);
+                int cnt = a.nn[i];
+                cnt = cnt < a.K ? cnt : a.K;
+                const int32_t* row = a.nm + (size_t)i * a.K;
+                const int last_quad = cnt > 0 ? ((cnt - 1) & ~3) : 0;
+                double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
+                double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;
+                for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
+                    const int kb = k0 + UNROLL * sub;
+                    const int n_mine = cnt - kb;
+                    int jj[UNROLL];
+                    float4 pj[UNROLL];
+#pragma unroll
+                    for (int v = 0; v < UNROLL / 4; ++v) {
+                        const int kv = kb + 4 * v;
+                        const int4 j4 = *reinterpret_cast<const int4*>(row + (kv < last_quad ? kv : last_quad));
+                        jj[4 * v + 0] = j4.x; jj[4 * v + 1] = j4.y; jj[4 * v + 2] = j4.z; jj[4 * v + 3] = j4.w;
+                    }
+                    // the home buckets of all entries side by side (four keys in one read): nearly every neighbor is there
+                    int at[UNROLL];
+                    unsigned missed = 0;
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) {
+                        const unsigned b = hash_bucket(jj[u]);
+                        const int4 k4 = *reinterpret_cast<const int4*>(&s_keys[4 * b]);
+                        const int j = jj[u];
+                        const int k = k4.x == j ? 0 : (k4.y == j ? 1 : (k4.z == j ? 2 : (k4.w == j ? 3 : -1)));
+                        at[u] = 4 * (int)b + (k < 0 ? 0 : k);
+                        if (k < 0 && u < n_mine) missed |= 1u << u;
+                    }
+                    if (__builtin_expect(__builtin_amdgcn_ballot_w64(missed != 0) != 0, 0)) {
+                        // a neighbor whose home bucket was full when it came lives further on; one that is nowhere (a
+                        // list that is not this library's) is fetched from memory below
+#pragma unroll
+                        for (int u = 0; u < UNROLL; ++u) {
+                            if (!(missed & (1u << u))) continue;
+                            unsigned b = hash_bucket(jj[u]);
+                            for (int probes = 1; probes < kHashProbes; ++probes) {
+                                b = (b + 1) & (kHashBuckets - 1);
+                                const int4 k4 = *reinterpret_cast<const int4*>(&s_keys[4 * b]);
+                                const int j = jj[u];
+                                const int k = k4.x == j ? 0 : (k4.y == j ? 1 : (k4.z == j ? 2 : (k4.w == j ? 3 : -1)));
+                                if (k >= 0) {
+                                    at[u] = 4 * (int)b + k;
+                                    missed &= ~(1u << u);
+                                    break;
+                                }
+                                if (k4.w == -1) break;  // (a bucket with room ends the chain)
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) {
+                        const float* q = s_xyz + 3 * at[u];
+                        pj[u].x = q[0]; pj[u].y = q[1]; pj[u].z = q[2];
+                    }
+                    if (__builtin_expect(__builtin_amdgcn_ballot_w64(missed != 0) != 0, 0)) {
+#pragma unroll
+                        for (int u = 0; u < UNROLL; ++u) {
+                            if (missed & (1u << u)) {
+                                unsigned j = (unsigned)jj[u];
+                                j = j < (unsigned)(a.n_atoms - 1) ? j : (unsigned)(a.n_atoms - 1);
+                                const float* q = a.pos + 3 * (size_t)j;
+                                pj[u].x = q[0]; pj[u].y = q[1]; pj[u].z = q[2];
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) {
+                        double d0, d1, d2;
+                        const double r2 = pair_d2_nearest_diagonal(me.x, me.y, me.z, pj[u].x, pj[u].y, pj[u].z, hd, hdi, d0, d1,
+                                                                   d2);
+                        if (u >= n_mine || !(r2 < a.rc2)) continue;
+                        pair_terms<VIRIAL, false>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
+                    }
+                }
+                e = group_sum<LPR>(e);
+                fx = group_sum<LPR>(fx);
+                fy = group_sum<LPR>(fy);
+                fz = group_sum<LPR>(fz);
+                if (VIRIAL) {
+                    w0 = group_sum<LPR>(w0); w1 = group_sum<LPR>(w1); w2 = group_sum<LPR>(w2);
+                    w3 = group_sum<LPR>(w3); w4 = group_sum<LPR>(w4); w5 = group_sum<LPR>(w5);
+                }
+                if (sub == 0) {
+                    const float ef = (float)e;
+                    a.e_atom[i] = ef;
+                    float* fo = a.forces + 3 * (size_t)i;
+                    fo[0] = (float)fx;
+                    fo[1] = (float)fy;
+                    fo[2] = (float)fz;
+                    if (SYS) {
+                        const int slot = sys - sys_lo;
+                        if (slot >= 0 && slot < kSysSlots) {
+                            atomicAdd(&s_acc[slot][0], (double)ef);
+                            if (VIRIAL) {
+                                atomicAdd(&s_acc[slot][1], w0); atomicAdd(&s_acc[slot][2], w1);
+                                atomicAdd(&s_acc[slot][3], w2); atomicAdd(&s_acc[slot][4], w3);
+                                atomicAdd(&s_acc[slot][5], w4); atomicAdd(&s_acc[slot][6], w5);
+                            }
+                        } else {
+                            double* out = a.sys_acc + 10 * (size_t)sys;
+                            atomic_add_f64(out + 0, (double)ef);
+                            if (VIRIAL) {
+                                atomic_add_f64(out + 1, w0); atomic_add_f64(out + 2, w1);
+                                atomic_add_f64(out + 3, w2); atomic_add_f64(out + 5, w3);
+                                atomic_add_f64(out + 6, w4); atomic_add_f64(out + 9, w5);
+                            }
+                        }
+                    }
+                }
+            }
+            __syncthreads();  // (the table is cleared next)
+            round0 = round_end;
+        }
+        r = seg_end;
+    }
+
+    if (SYS) {
+        __syncthreads();
+        if (threadIdx.x < kSysSlots * NV) {
+            const int slot = threadIdx.x / NV, k = threadIdx.x % NV;
+            const double v = s_acc[slot][k];
+            if (v != 0.0 && sys_lo + slot < a.n_systems) {
+                const int where = (k == 0) ? 0 : (k <= 3 ? k : (k <= 5 ? k + 1 : 9));
+                atomic_add_f64(a.sys_acc + 10 * (size_t)(sys_lo + slot) + where, v);
+            }
+        }
+    }
+}
+
 // Half list: each pair once, both atoms updated.  Accumulates in fp64 scratch through
 // atomics; one lane per row.  Not tuned: the reference's LJ default is the full list
 // (nvalchemi/models/lj.py:115).
@@ -750,7 +1040,8 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
                                      double epsilon, double sigma, double cutoff, double switch_width,
                                      int32_t half_list, float* atomic_energies, float* forces, float* virials,
                                      float* system_energies, void* workspace, size_t workspace_bytes, void* stream,
-                                     int32_t reuse_tables = 0) {
+                                     int32_t reuse_tables = 0, const float* ordered_positions = nullptr,
+                                     const int32_t* round_segments = nullptr, const int32_t* round_counts = nullptr) {
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
     if (!(switch_width >= 0.0) || switch_width > cutoff)
@@ -848,6 +1139,26 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
             a.sys_first = sys_first;
             a.sys_last = sys_last;
             a.sys_image = sys_image;
+            // large systems walked in the neighbor build's cell order with that build's hints, images derived, rows of
+            // 16-byte words, per-system sums wanted: the kernel that stages a round's neighborhood by hash
+            const bool hashed = a.order && ordered_positions && round_segments && round_counts && a.list_rc > 0.0 &&
+                                shifts && sys && a.inv_sw == 0.0 && n_systems > 0 && n_atoms / n_systems > kLdsAtoms &&
+                                max_neighbors >= 4 && max_neighbors % 4 == 0 && aligned16(a.nm) &&
+                                aligned16(ordered_positions);
+            if (hashed) {
+                LjArgs b = a;
+                b.rows_per_block = NVAMD_LJ_HASH_ROWS;
+                b.n_blocks = (unsigned)((n_atoms + b.rows_per_block - 1) / b.rows_per_block);
+                dim3 grid((b.n_blocks + 7) / 8 * 8), blk(kBlockFull);
+                const LjRounds hints{reinterpret_cast<const float4*>(ordered_positions),
+                                     reinterpret_cast<const int2*>(round_segments), round_counts};
+                if (vir)
+                    hipLaunchKernelGGL((lj_hashed_kernel<true, true>), grid, blk, 0, st, b, hints, b.bidx, b.order,
+                                       b.sys_first, b.sys_last, b.cells, b.sys_image);
+                else
+                    hipLaunchKernelGGL((lj_hashed_kernel<false, true>), grid, blk, 0, st, b, hints, b.bidx, b.order,
+                                       b.sys_first, b.sys_last, b.cells, b.sys_image);
+            } else
             switch (lanes_per_row(max_neighbors)) {
                 case 8: launch_full<8>(a, vir, shifts, sys, st); break;
                 case 16: launch_full<16>(a, vir, shifts, sys, st); break;
@@ -897,6 +1208,29 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_repeat(const float* positions, const
                                  row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
                                  sigma, cutoff, switch_width, /*half_list=*/0, atomic_energies, forces, virials,
                                  system_energies, workspace, workspace_bytes, stream, reuse_tables ? 1 : 0);
+}
+
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_rounds(const float* positions, const float* cells,
+                                                    const int32_t* neighbor_matrix,
+                                                    const int32_t* neighbor_matrix_shifts,
+                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
+                                                    const int32_t* row_order, const float* ordered_positions,
+                                                    const int32_t* round_segments, const int32_t* round_counts,
+                                                    double neighbor_list_cutoff, int32_t n_atoms, int32_t max_neighbors,
+                                                    int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
+                                                    double cutoff, double switch_width, int32_t reuse_tables,
+                                                    float* atomic_energies, float* forces, float* virials,
+                                                    float* system_energies, void* workspace, size_t workspace_bytes,
+                                                    void* stream) {
+    const int given = (ordered_positions ? 1 : 0) + (round_segments ? 1 : 0) + (round_counts ? 1 : 0);
+    if (given != 0 && (given != 3 || !row_order))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT,
+                    "lj: ordered_positions, round_segments and round_counts come together, with the row_order they belong to");
+    return lj_energy_forces_impl(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors, batch_idx,
+                                 row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
+                                 sigma, cutoff, switch_width, /*half_list=*/0, atomic_energies, forces, virials,
+                                 system_energies, workspace, workspace_bytes, stream, reuse_tables ? 1 : 0,
+                                 ordered_positions, round_segments, round_counts);
 }
 
 // ---- the variant that allocates nothing ------------------------------------------------------

@@ -51,6 +51,9 @@ constexpr int kMaxCellsPerAxis = 1024;
 static_assert(kMaxCellsPerAxis <= 1024, "a search unit's cell coordinates are packed 10 bits each");
 constexpr int kMinCellCap = 8;    // a system may use at least this many cells
 constexpr int kMaxStencilRadius = 32;  // cells searched per axis and direction, at most
+constexpr int kPairStageAtoms = 4096;  // the pair kernel stages the positions of systems up to this size whole
+constexpr int kRoundRows = 64;         // rows of the pair kernel's rounds over large systems
+constexpr int kRoundSegments = NVAMD_PAIR_ROUND_SEGMENTS;  // slices of the sorted arrays named per round, at most
 
 struct NlSys {
     double h[9];       // rows = lattice vectors (identity without a cell)
@@ -107,7 +110,8 @@ struct NlHeader {
     int error;   // of the build in hand: NVAMD_NL_STATUS_* bits
     int total_units;
     int sticky;  // the bits of all earlier builds through this workspace since they were last cleared
-    int pad[12];
+    int kept_xyz;  // the build in hand left the atoms' own coordinates in cell order (sorted_xyz)
+    int pad[11];
 };
 
 struct NlWorkspace {
@@ -124,6 +128,7 @@ struct NlWorkspace {
     int* block_sums;     // scan partials
     float4* sorted_pos;  // (N) cell-local xyz + original index bits
     int4* sorted_aux;    // (N) wrap integers
+    float4* sorted_xyz;  // (N) the atoms' own float32 coordinates + original index bits, in cell order (large systems only)
     int max_cells;
     int n_scan_blocks;
 };
@@ -157,6 +162,7 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
     p = take((nsb + 1) * sizeof(int)); if (ws) ws->block_sums = reinterpret_cast<int*>(p);
     p = take(N * sizeof(float4)); if (ws) ws->sorted_pos = reinterpret_cast<float4*>(p);
     p = take(N * sizeof(int4)); if (ws) ws->sorted_aux = reinterpret_cast<int4*>(p);
+    p = take(N * sizeof(float4)); if (ws) ws->sorted_xyz = reinterpret_cast<float4*>(p);
     if (ws) {
         ws->max_cells = (int)C;
         ws->n_scan_blocks = (int)nsb;
@@ -176,6 +182,7 @@ struct NlArgs {
     int n_atoms, n_systems, K, half, tail_mode;
     int unit_group;  // units are dealt to the XCDs in groups of this many (a power of two)
     int center_chunk;  // centre atoms per unit of work at most (<= kCenterChunk; smaller for small batches: more units)
+    int keep_xyz;      // also leave the atoms' own coordinates in cell order (for the pair kernel of large systems)
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -244,6 +251,7 @@ __global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspac
     if (t == 0) {
         ws.hdr->sticky |= ws.hdr->error;
         ws.hdr->error = 0;
+        ws.hdr->kept_xyz = a.keep_xyz;
     }
     if (t >= a.n_systems) return;
     NlSys s;
@@ -525,6 +533,10 @@ __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspac
     int slot = ws.cell_start[b.cell] + ws.atom_rank[i];
     ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
     ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
+    if (a.keep_xyz) {
+        const Pos3 r = load_pos(a, (size_t)i);
+        ws.sorted_xyz[slot] = make_float4((float)r.x, (float)r.y, (float)r.z, __int_as_float(i));
+    }
 }
 
 // ---- per-system path: 1-6 in one workgroup per system -----------------------------------------
@@ -698,6 +710,10 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         const int slot = start + rank;
         ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
         ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
+        if (a.keep_xyz) {
+            const Pos3 r = load_pos(a, (size_t)i);
+            ws.sorted_xyz[slot] = make_float4((float)r.x, (float)r.y, (float)r.z, __int_as_float(i));
+        }
     };
     if (kept) {
 #pragma unroll
@@ -748,11 +764,12 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
 }
 
 // Before nl_system_sort_kernel: the unit counter and the error flag start at zero.
-__global__ void nl_reset_kernel(NlWorkspace ws) {
+__global__ void nl_reset_kernel(NlWorkspace ws, int keep_xyz) {
     ws.hdr->total_units = 0;
     ws.hdr->total_cells = 0;  // not used on the per-system path: cell ids are not dense
     ws.hdr->sticky |= ws.hdr->error;
     ws.hdr->error = 0;
+    ws.hdr->kept_xyz = keep_xyz;
 }
 
 // ---- 7 search -------------------------------------------------------------------------------
@@ -1263,6 +1280,93 @@ __global__ __launch_bounds__(kBlock) void nl_atom_order_kernel(const float4* __r
     order[k] = __float_as_int(sorted_pos[k].w);
 }
 
+// ---- what the pair kernel of large systems takes over from a build -----------------------------------------
+// The atoms in cell order with their own coordinates (a copy out of the workspace, which the next build overwrites) ...
+__global__ __launch_bounds__(kBlock) void nl_ordered_positions_kernel(NlWorkspace ws, int n_atoms,
+                                                                      int32_t* __restrict__ order,
+                                                                      float4* __restrict__ ordered) {
+    const int k = blockIdx.x * kBlock + threadIdx.x;
+    if (k >= n_atoms) return;
+    const bool kept = ws.hdr->kept_xyz != 0;
+    const float4 p = kept ? ws.sorted_xyz[k] : ws.sorted_pos[k];
+    order[k] = __float_as_int(p.w);
+    ordered[k] = p;  // (without kept coordinates the rounds below all say "no hint": nobody reads the xyz)
+}
+
+// ... and, for every round of kRoundRows consecutive slots of the cell order, the slices of that order that hold
+// every atom within the stencil of the round's cells: a handful of (first slot, length) pairs, because a column of
+// cells along axis 2 is one slice.  A count of -1 says "no hint" (the round spans two systems, its system was not
+// built with kept coordinates, or it needs more slices than the table has room for).
+__global__ __launch_bounds__(kBlock) void nl_pair_rounds_kernel(NlWorkspace ws, const int32_t* __restrict__ bidx,
+                                                                int n_atoms, int n_rounds, int2* __restrict__ segments,
+                                                                int32_t* __restrict__ counts) {
+    const int w = blockIdx.x * kBlock + threadIdx.x;
+    if (w >= n_rounds) return;
+    const int s_lo = w * kRoundRows, s_hi = (s_lo + kRoundRows < n_atoms ? s_lo + kRoundRows : n_atoms) - 1;
+    const int sidx = bidx[s_lo];
+    int n = -1;
+    if (ws.hdr->kept_xyz && bidx[s_hi] == sidx) {
+        const NlSys& S = ws.sys[sidx];
+        const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
+        const int* start = ws.cell_start + S.cell_offset;  // S.n_cells + 1 entries
+        auto cell_of = [&](int slot) {  // the last cell that begins at or before the slot
+            int lo = 0, hi = S.n_cells;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (start[mid] <= slot) lo = mid; else hi = mid;
+            }
+            return lo;
+        };
+        if (S.n_cells > 0) {
+            const int c_a = cell_of(s_lo), c_b = cell_of(s_hi);
+            const int col_a = c_a / nc2, col_b = c_b / nc2;
+            int2* out = segments + (size_t)w * kRoundSegments;
+            n = 0;
+            for (int col = col_a; col <= col_b && n >= 0; ++col) {
+                const int z_lo = (col == col_a ? c_a - col_a * nc2 : 0) - S.R[2];
+                const int z_hi = (col == col_b ? c_b - col_b * nc2 : nc2 - 1) + S.R[2];
+                const int cx = col / nc1, cy = col - cx * nc1;
+                for (int dx = -S.R[0]; dx <= S.R[0] && n >= 0; ++dx) {
+                    int gx = cx + dx;
+                    if (S.per[0]) gx -= floordiv(gx, nc0) * nc0; else if (gx < 0 || gx >= nc0) continue;
+                    for (int dy = -S.R[1]; dy <= S.R[1] && n >= 0; ++dy) {
+                        int gy = cy + dy;
+                        if (S.per[1]) gy -= floordiv(gy, nc1) * nc1; else if (gy < 0 || gy >= nc1) continue;
+                        const int base = (gx * nc1 + gy) * nc2;
+                        // the range of cells along axis 2, in one piece or (through the periodic boundary) in two
+                        int p_lo[2], p_hi[2], pieces = 1;
+                        p_lo[0] = z_lo; p_hi[0] = z_hi;
+                        if (!S.per[2]) {
+                            p_lo[0] = z_lo < 0 ? 0 : z_lo;
+                            p_hi[0] = z_hi > nc2 - 1 ? nc2 - 1 : z_hi;
+                        } else if (z_hi - z_lo + 1 >= nc2) {
+                            p_lo[0] = 0; p_hi[0] = nc2 - 1;
+                        } else if (z_lo < 0) {
+                            // (z_lo > -nc2 here: the span is shorter than the axis)
+                            pieces = 2;
+                            p_lo[0] = z_lo + nc2; p_hi[0] = nc2 - 1;
+                            p_lo[1] = 0; p_hi[1] = z_hi;
+                        } else if (z_hi > nc2 - 1) {
+                            pieces = 2;
+                            p_lo[0] = z_lo; p_hi[0] = nc2 - 1;
+                            p_lo[1] = 0; p_hi[1] = z_hi - nc2;
+                        }
+                        for (int k = 0; k < pieces; ++k) {
+                            if (p_hi[k] < p_lo[k]) continue;
+                            const int first = start[base + p_lo[k]];
+                            const int len = start[base + p_hi[k] + 1] - first;
+                            if (len <= 0) continue;
+                            if (n >= kRoundSegments) { n = -1; break; }
+                            out[n++] = make_int2(first, len);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    counts[w] = n;
+}
+
 }  // namespace
 }  // namespace nvamd
 
@@ -1282,6 +1386,29 @@ NVAMD_EXPORT int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace
     hipLaunchKernelGGL(nl_atom_order_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0,
                        static_cast<hipStream_t>(stream), ws.sorted_pos, batch_idx, rebuild_flags, n_atoms, atom_order);
     NVAMD_LAUNCH_CHECK("atom order launch");
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_pair_hints(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
+                                         int32_t n_atoms, int32_t n_systems, int32_t* atom_order,
+                                         float* ordered_positions, int32_t* round_segments, int32_t* round_counts,
+                                         void* stream) {
+    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "pair hints: negative size");
+    if (n_atoms == 0 || n_systems == 0) return NVAMD_OK;
+    if (!batch_idx || !atom_order || !ordered_positions || !round_segments || !round_counts)
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "pair hints: null buffer");
+    size_t need = carve(nullptr, nullptr, n_atoms, n_systems);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "pair hints: workspace %zu < %zu bytes", workspace_bytes, need);
+    NlWorkspace ws;
+    carve(&ws, static_cast<char*>(const_cast<void*>(workspace)), n_atoms, n_systems);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(nl_ordered_positions_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws,
+                       n_atoms, atom_order, reinterpret_cast<float4*>(ordered_positions));
+    const int n_rounds = (n_atoms + kRoundRows - 1) / kRoundRows;
+    hipLaunchKernelGGL(nl_pair_rounds_kernel, dim3((n_rounds + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws, batch_idx,
+                       n_atoms, n_rounds, reinterpret_cast<int2*>(round_segments), round_counts);
+    NVAMD_LAUNCH_CHECK("pair hints launch");
     return NVAMD_OK;
 }
 
@@ -1364,6 +1491,8 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     while (a.unit_group < 64 && (long long)a.unit_group * 8192 <= (long long)n_atoms) a.unit_group *= 2;
     // A small batch does not fill the chip with units of kCenterChunk centre atoms: smaller units, about 4096 of them
     a.center_chunk = NVAMD_NL_CHUNK(n_atoms);
+    // systems too large for the pair kernel to stage whole: their atoms' own coordinates stay behind in cell order
+    a.keep_xyz = (positions != nullptr && n_atoms / n_systems > kPairStageAtoms) ? 1 : 0;
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
@@ -1378,7 +1507,7 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
                                                             : (sort_path == NVAMD_NL_SORT_PER_SYSTEM);
     if (per_system) {
         // many small systems: set-up to scatter in one workgroup per system
-        hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws);
+        hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws, a.keep_xyz);
         hipLaunchKernelGGL(nl_system_sort_kernel, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
     } else {
         size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;

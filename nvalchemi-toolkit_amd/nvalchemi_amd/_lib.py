@@ -56,6 +56,8 @@ _SIGNATURES = {
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_lj_energy_forces_hinted": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_repeat": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
+    "nvamd_lj_energy_forces_rounds": (_i32, [_vp] * 10 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
+    "nvamd_nl_pair_hints": (_i32, [_vp, _c.c_size_t, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
     "nvamd_lj_energy_forces_static": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_vp] * 5),
     "nvamd_nl_atom_order": (_i32, [_vp, _c.c_size_t, _vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_segment_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
@@ -336,7 +338,9 @@ def nl_matrix_to_coo(neighbor_matrix, neighbor_matrix_shifts, edge_ptr, neighbor
 def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
                      batch_idx, fill_value, epsilon, sigma, cutoff, switch_width, half_list,
                      atomic_energies, forces, virials=None, system_energies=None, row_order=None,
-                     neighbor_list_cutoff: float = 0.0) -> None:
+                     neighbor_list_cutoff: float = 0.0, pair_hints=None) -> None:
+    """``pair_hints``: ``(ordered_positions (N,4) f32, round_segments, round_counts)`` of ``nl_pair_hints`` for the
+    positions in hand and the ``row_order`` given with them (full list only; ignored otherwise)."""
     lib = library()
     N = positions.shape[0]
     K = neighbor_matrix.shape[1]
@@ -367,6 +371,28 @@ def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, 
         state = (positions.device.index, _stream(positions.device))
         reuse = _lj_tables.get(state) == tables
         _lj_tables[state] = tables
+        if pair_hints is not None and row_order is not None:
+            ordered, segments, counts = pair_hints
+            R = (N + PAIR_ROUND_ROWS - 1) // PAIR_ROUND_ROWS
+            _check(lib.nvamd_lj_energy_forces_rounds(
+                _dev(positions, "positions", torch.float32, (N, 3)),
+                _dev(cells, "cells", torch.float32, (B, 3, 3)),
+                _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
+                _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+                _dev(num_neighbors, "num_neighbors", torch.int32, (N,)),
+                _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+                _dev(row_order, "row_order", torch.int32, (N,)),
+                _dev(ordered, "ordered_positions", torch.float32, (N, 4)),
+                _dev(segments, "round_segments", torch.int32, (R, PAIR_ROUND_SEGMENTS, 2)),
+                _dev(counts, "round_counts", torch.int32, (R,)), float(neighbor_list_cutoff),
+                N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), float(switch_width),
+                int(reuse),
+                _dev(atomic_energies, "atomic_energies", torch.float32, (N,)),
+                _dev(forces, "forces", torch.float32, (N, 3)),
+                _opt(virials, "virials", torch.float32, (B, 9)),
+                _opt(system_energies, "system_energies", torch.float32, (B,)),
+                ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_rounds")
+            return
         _check(lib.nvamd_lj_energy_forces_repeat(
             _dev(positions, "positions", torch.float32, (N, 3)),
             _dev(cells, "cells", torch.float32, (B, 3, 3)),
@@ -432,6 +458,25 @@ def lj_energy_forces_static(positions, cells, neighbor_matrix, neighbor_matrix_s
         _opt(virials, "virials", torch.float32, (B, 9)),
         _opt(system_energies, "system_energies", torch.float32, (B,)),
         _stream(positions.device)), "nvamd_lj_energy_forces_static")
+
+
+PAIR_ROUND_ROWS, PAIR_ROUND_SEGMENTS = 64, 40
+
+
+def nl_pair_hints(batch_idx, n_systems: int, atom_order, ordered_positions, round_segments, round_counts) -> None:
+    """What the pair kernel takes over from the last neighbor build on this device and stream (same sizes): the cell
+    order, the positions in that order, and per round of 64 rows the slices of the order that hold its neighborhood."""
+    lib = library()
+    N = batch_idx.shape[0]
+    R = (N + PAIR_ROUND_ROWS - 1) // PAIR_ROUND_ROWS
+    need = _size(lib.nvamd_nl_workspace_bytes, N, int(n_systems))
+    ws = workspaces.get(batch_idx.device, "nl", need)
+    _check(lib.nvamd_nl_pair_hints(
+        ws.data_ptr(), ws.numel(), _dev(batch_idx, "batch_idx", torch.int32, (N,)), N, int(n_systems),
+        _dev(atom_order, "atom_order", torch.int32, (N,)),
+        _dev(ordered_positions, "ordered_positions", torch.float32, (N, 4)),
+        _dev(round_segments, "round_segments", torch.int32, (R, PAIR_ROUND_SEGMENTS, 2)),
+        _dev(round_counts, "round_counts", torch.int32, (R,)), _stream(batch_idx.device)), "nvamd_nl_pair_hints")
 
 
 def nl_atom_order(batch_idx, n_systems: int, atom_order, rebuild_flags=None) -> None:

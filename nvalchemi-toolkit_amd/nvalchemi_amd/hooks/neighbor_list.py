@@ -171,7 +171,8 @@ class NeighborListHook:
             return None if t is None else (t.data_ptr(), tuple(t.shape))
 
         return (ptr(self._neighbor_matrix), ptr(self._num_neighbors), ptr(self._neighbor_matrix_shifts),
-                ptr(self._ref_positions), ptr(self._rebuild_flags), ptr(getattr(self, "_atom_order", None)))
+                ptr(self._ref_positions), ptr(self._rebuild_flags), ptr(getattr(self, "_atom_order", None)),
+                ptr(getattr(self, "_ordered_positions", None)))
 
     def overflowed(self, clear: bool = True) -> bool:
         """Whether any build since the last call left an atom with more neighbors than the rows hold
@@ -195,12 +196,34 @@ class NeighborListHook:
         if N == 0 or batch.max_num_nodes <= self._ROW_ORDER_MIN_ATOMS:
             if getattr(batch, "_neighbor_row_order", None) is not None:
                 object.__setattr__(batch, "_neighbor_row_order", None)
+            if getattr(batch, "_neighbor_pair_hints", None) is not None:
+                object.__setattr__(batch, "_neighbor_pair_hints", None)
             self._atom_order = None
             return
         fresh = (getattr(self, "_atom_order", None) is None or self._atom_order.shape[0] != N
                  or self._atom_order.device != batch.positions.device)
         if fresh:
             self._atom_order = torch.empty(N, dtype=torch.int32, device=batch.positions.device)
+        if self.skin <= 0.0 and batch.positions.dtype == torch.float32 and N // max(B, 1) > self._ROW_ORDER_MIN_ATOMS:
+            # Every call is a full build on the positions in hand: besides the order, the pair kernel can take the
+            # positions in that order and, per round of 64 rows, the slices of the order that hold the round's
+            # neighborhood (it then reads its neighbors with contiguous loads instead of one gather per pair).
+            R = (N + _lib.PAIR_ROUND_ROWS - 1) // _lib.PAIR_ROUND_ROWS
+            if fresh or getattr(self, "_ordered_positions", None) is None or self._ordered_positions.shape[0] != N:
+                dev = batch.positions.device
+                self._ordered_positions = torch.empty(N, 4, dtype=torch.float32, device=dev)
+                self._round_segments = torch.empty(R, _lib.PAIR_ROUND_SEGMENTS, 2, dtype=torch.int32, device=dev)
+                self._round_counts = torch.empty(R, dtype=torch.int32, device=dev)
+            _lib.nl_pair_hints(batch.batch_idx, B, self._atom_order, self._ordered_positions, self._round_segments,
+                               self._round_counts)
+            object.__setattr__(batch, "_neighbor_row_order", self._atom_order)
+            # (tied to the positions of this build: storage and version)
+            object.__setattr__(batch, "_neighbor_pair_hints",
+                               (self._ordered_positions, self._round_segments, self._round_counts,
+                                batch.positions.data_ptr(), batch.positions._version))
+            return
+        if getattr(batch, "_neighbor_pair_hints", None) is not None:
+            object.__setattr__(batch, "_neighbor_pair_hints", None)
         flags = None
         if not fresh and self.skin > 0.0 and self._ref_positions is not None:
             flags = self._rebuild_flags  # systems that were not rebuilt keep the order of their last build

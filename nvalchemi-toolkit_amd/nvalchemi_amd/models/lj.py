@@ -142,6 +142,16 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
         return None
 
     @staticmethod
+    def _pair_hints_of(data, positions: torch.Tensor):
+        """What the neighbor hook left for the pair kernel of large systems, if it was made from exactly these
+        positions (same storage, no write since)."""
+        hints = getattr(data, "_neighbor_pair_hints", None)
+        if (isinstance(hints, tuple) and len(hints) == 5 and hints[3] == positions.data_ptr()
+                and hints[4] == positions._version):
+            return hints[:3]
+        return None
+
+    @staticmethod
     def _search_cutoff_of(data, neighbor_matrix: torch.Tensor) -> float:
         """The radius the neighbor matrix in hand was searched with, if the builder left it on the
         batch for exactly this tensor; 0.0 (unknown) otherwise."""
@@ -192,7 +202,8 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             inp["batch_idx"].contiguous(), inp["fill_value"], self.epsilon, self.sigma, self.cutoff,
             self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs,
             row_order=self._row_order_of(data, N, positions.device),
-            neighbor_list_cutoff=self._search_cutoff_of(data, neighbor_matrix))
+            neighbor_list_cutoff=self._search_cutoff_of(data, neighbor_matrix),
+            pair_hints=self._pair_hints_of(data, inp["positions"]))
         if own_energy:
             sys_e = sys_e.clone()  # a fresh tensor for the caller, as in the reference (:482)
         model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
