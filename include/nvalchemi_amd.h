@@ -298,25 +298,27 @@ int32_t nvamd_lj_energy_forces_repeat(const float* positions, const float* cells
                                       float* system_energies, void* workspace, size_t workspace_bytes,
                                       void* stream);
 
-/* nvamd_lj_energy_forces_repeat with the outputs of nvamd_nl_pair_hints for the same positions (all three
- * given, or all three null: then this is nvamd_lj_energy_forces_repeat).  No counterpart in the reference.
- * The rows are walked in row_order, 64 at a time; where a round has a hint, the atoms of its slices are read
- * from ordered_positions (contiguous reads) into a table in LDS keyed by atom index, and the pair arithmetic
- * finds its neighbors there instead of gathering each from memory.  Used for batches of more than 4096 atoms
- * per system on average, in cells without off-diagonal terms that are wider than twice neighbor_list_cutoff;
- * everything else takes the paths of the other entry points.  Results are those of the other entry points. */
-int32_t nvamd_lj_energy_forces_rounds(const float* positions, const float* cells,
-                                      const int32_t* neighbor_matrix,
-                                      const int32_t* neighbor_matrix_shifts,
-                                      const int32_t* num_neighbors, const int32_t* batch_idx,
-                                      const int32_t* row_order, const float* ordered_positions,
-                                      const int32_t* round_segments, const int32_t* round_counts,
-                                      double neighbor_list_cutoff, int32_t n_atoms, int32_t max_neighbors,
-                                      int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
-                                      double cutoff, double switch_width, int32_t reuse_tables,
-                                      float* atomic_energies, float* forces, float* virials,
-                                      float* system_energies, void* workspace, size_t workspace_bytes,
-                                      void* stream);
+/* nvamd_lj_energy_forces_repeat over the tiles of nvamd_nl_build_tiles, for the positions that build read.  No
+ * counterpart in the reference.  The rows are walked unit by unit of the build's search; a unit's tile (the atoms
+ * of its stencil cells, a few hundred) is copied from ordered_positions into LDS with contiguous reads, laid out
+ * by the unit's record, and each listed pair finds its neighbor there through its 16-bit tile_index: no gather from
+ * memory per pair, and two bytes read per pair instead of four.  Meant for systems too large for the other entry
+ * points to stage whole (more than 4096 atoms).  Images are derived from the positions, so neighbor_list_cutoff
+ * must be the build's cutoff and every cell wider than twice that (systems where it is not, and units without a
+ * tile, take their neighbors from memory as the other entry points do).  Full list, no switching.
+ * neighbor_matrix / num_neighbors / row_order are those of the same build.  Results are those of the other entry
+ * points, bit for bit. */
+int32_t nvamd_lj_energy_forces_tiles(const float* positions, const float* cells,
+                                     const int32_t* neighbor_matrix,
+                                     const int32_t* neighbor_matrix_shifts,
+                                     const int32_t* num_neighbors, const int32_t* batch_idx,
+                                     const int32_t* row_order, const uint16_t* tile_index,
+                                     const float* ordered_positions, const int32_t* tile_records,
+                                     const int32_t* tile_count, double neighbor_list_cutoff, int32_t n_atoms,
+                                     int32_t max_neighbors, int32_t n_systems, int32_t fill_value, double epsilon,
+                                     double sigma, double cutoff, int32_t reuse_tables, float* atomic_energies,
+                                     float* forces, float* virials, float* system_energies, void* workspace,
+                                     size_t workspace_bytes, void* stream);
 
 /* nvamd_lj_energy_forces_hinted for callers that cannot allocate device memory or carry a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
@@ -412,23 +414,30 @@ int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const
                             const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
                             int32_t* atom_order, void* stream);
 
-/* What the pair kernel can take over from a neighbor build for systems too large for it to stage whole (more
- * than 4096 atoms per system on average: only then does a build keep what this call reads; otherwise every
- * count comes back as -1).  No counterpart in the reference.  From the build that last used this workspace with
- * the same n_atoms / n_systems:
- *   atom_order (N) i32             as nvamd_nl_atom_order
- *   ordered_positions (N,4) f32    the float32 coordinates of atom_order[k] as the build read them, and the
- *                                  bits of atom_order[k] in the fourth word
- *   round_counts (R) i32, round_segments (R, NVAMD_PAIR_ROUND_SEGMENTS, 2) i32, R = ceil(N / 64):
- *                                  for round w, the rows 64 w .. 64 w + 63 of the cell order, round_counts[w]
- *                                  pairs (first, length) of slices of that order which together hold every atom
- *                                  in the stencil of the round's cells, hence every neighbor of the round's
- *                                  atoms within the build's cutoff; -1: no hint for this round
- * Valid for the positions of that build only. */
-#define NVAMD_PAIR_ROUND_SEGMENTS 40
-int32_t nvamd_nl_pair_hints(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
-                            int32_t n_atoms, int32_t n_systems, int32_t* atom_order, float* ordered_positions,
-                            int32_t* round_segments, int32_t* round_counts, void* stream);
+/* nvamd_nl_build_path that also leaves behind what a pair kernel needs to walk the search's own tiles again
+ * (nvamd_lj_energy_forces_tiles).  No counterpart in the reference.  The search handles the atoms of a run of
+ * cells (a "unit") against one tile: the atoms of the run's stencil cells, staged in LDS in a fixed order.  Beyond
+ * the outputs of nvamd_nl_build_path:
+ *   tile_index (N, max_neighbors) u16    per listed pair, where the neighbor stood in the tile of the row's unit
+ *   ordered_positions (N, 4) f32         the atoms in cell order: float32 coordinates as read, and the bits of the
+ *                                        atom's index in the fourth word
+ *   tile_records (R, NVAMD_NL_TILE_RECORD_INTS) i32, R from nvamd_nl_tile_records: per unit
+ *                                        [first row, rows] (slots of the cell order), [system, atoms in the tile,
+ *                                        or -1: the unit's stencil is not one tile], then per stencil cell
+ *                                        [its first slot of the cell order, its offset in the tile]
+ *   tile_count (1) i32                   units of this build
+ * Float32 positions, full list, every system built (no rebuild_flags), max_neighbors a multiple of 8.  A tile holds
+ * at most NVAMD_NL_TILE_ATOMS atoms.  Valid for the positions of this build only. */
+#define NVAMD_NL_TILE_RECORD_INTS 132
+#define NVAMD_NL_TILE_ATOMS 1088
+int32_t nvamd_nl_tile_records(int32_t n_atoms, int32_t n_systems, size_t* records);
+int32_t nvamd_nl_build_tiles(const float* positions, const float* cell, const uint8_t* pbc,
+                             const int32_t* batch_ptr, const int32_t* batch_idx, int32_t n_atoms,
+                             int32_t n_systems, double cutoff, int32_t max_neighbors, int32_t tail_mode,
+                             int32_t sort_path, int32_t* neighbor_matrix, int32_t* num_neighbors,
+                             int32_t* neighbor_matrix_shifts, uint16_t* tile_index, float* ordered_positions,
+                             int32_t* tile_records, int32_t* tile_count, void* workspace, size_t workspace_bytes,
+                             void* stream);
 
 /* Per-system reductions of a per-atom float32 vector: replace the Warp launches behind
  * nvalchemi_hooks::segmented_sum / _max / _min / _mean (nvalchemi/dynamics/hooks/_utils.py:58-136;

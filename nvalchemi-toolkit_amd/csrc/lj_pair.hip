@@ -21,9 +21,6 @@
 #include "common.h"
 #include "geom.h"
 
-#ifndef NVAMD_LJ_HASH_ROWS
-#define NVAMD_LJ_HASH_ROWS 512
-#endif
 #ifndef NVAMD_LJ_UNROLL
 #define NVAMD_LJ_UNROLL 4
 #endif
@@ -546,289 +543,296 @@ __global__ __launch_bounds__(kBlockFull, (VIRIAL || SWITCH) ? 4 : 6) void lj_mat
     }
 }
 
-// ---- systems too large to stage: the neighborhood of a round of rows, staged by hash -----------------
-// A system that does not fit the LDS stage is walked in the cell order of the neighbor build (row_order), 64 rows
-// to a round: atoms of a few adjacent cells, whose neighbors all lie in the stencil of those cells.  The build
-// names that stencil per round as a few slices of the cell order (nvamd_nl_pair_hints) and leaves the atoms'
-// coordinates in that order, so a round reads its whole neighborhood with contiguous loads, enters each atom into
-// a hash table in LDS under its index (open addressing), and the pair arithmetic finds its neighbors there:
-// no gather from memory per listed pair (which fetches a cache line for twelve bytes, from all over the array).
-// Cells without off-diagonal terms whose images follow from the positions (img == 2) only; any other system, a
-// round without a hint, and a round whose neighborhood overflows the table take the unstaged row loop.
-constexpr int kHashSlots = 4096;   // keys (16 KB) and xyz (48 KB), in buckets of four slots
-constexpr int kHashBuckets = kHashSlots / 4;
-constexpr int kHashProbes = 12;    // buckets looked at before the table is taken to be as good as full
-constexpr int kHashLpr = 8;        // lanes per row
-constexpr int kHashRows = kBlockFull / kHashLpr;  // rows of a round
-constexpr int kHashStage = 4;      // atoms of the neighborhood a thread has in flight at a time
-static_assert(kHashRows == 64, "nvamd_nl_pair_hints describes rounds of 64 rows");
+// ---- systems too large to stage: the tiles of the neighbor search, walked again ---------------------------
+// The neighbor search (nvamd_nl_build_tiles) handles a unit of work, the atoms of a short run of cells, against one
+// tile: the atoms of the run's stencil cells in a fixed order in LDS.  It leaves behind the atoms' coordinates in
+// cell order, per unit a record that lays the tile out as slices of that order, and per listed pair the place of
+// the neighbor in the tile (16 bits).  A workgroup here takes a few consecutive units, copies their tiles into LDS
+// with contiguous reads, and the pair arithmetic finds every neighbor there by its tile index: no gather from
+// memory per pair (a cache line for twelve bytes, from all over the array, when atom numbers carry no locality).
+constexpr int kTileUnits = 4;        // consecutive units a workgroup takes at a time (about three rounds of 64 rows)
+constexpr int kTilePool = 4096;      // atoms of their tiles staged at a time (48 KB)
+constexpr int kTileCells = 64;       // stencil cells in a unit's record
+constexpr int kTileRecord = NVAMD_NL_TILE_RECORD_INTS / 2;  // 8-byte words per record
+static_assert(kTileRecord == 2 + kTileCells, "two words of header, one per stencil cell");
+static_assert(NVAMD_NL_TILE_ATOMS <= kTilePool, "one tile always fits the pool");
 
-__device__ __forceinline__ unsigned hash_bucket(int j) { return ((unsigned)j * 0x9E3779B1u) >> 22; }
-static_assert(kHashBuckets == 1 << 10, "the hash keeps the top ten bits");
-
-struct LjRounds {
-    const float4* ordered;   // (N) coordinates in row order + atom index bits
-    const int2* segments;    // (R, NVAMD_PAIR_ROUND_SEGMENTS)
-    const int32_t* counts;   // (R)
+struct LjTiles {
+    const uint16_t* index;   // (N, K)
+    const float4* xyz;       // (N) cell order
+    const int2* records;     // (units, kTileRecord)
+    const int32_t* count;    // (1)
 };
 
-template <bool VIRIAL, bool SYS>
-__global__ __launch_bounds__(kBlockFull, 4) void lj_hashed_kernel(
-    LjArgs a, LjRounds hints, const int32_t* __restrict__ bidx_ro, const int32_t* __restrict__ order_ro,
-    const int32_t* __restrict__ first_ro, const int32_t* __restrict__ last_ro, const float* __restrict__ cells_ro,
-    const LjSysImage* __restrict__ image_ro) {
-    constexpr int NV = VIRIAL ? 7 : 1;
-    constexpr int LPR = kHashLpr, G = kHashRows, UNROLL = 8;
-    __shared__ double s_acc[kSysSlots][NV];
-    __shared__ __align__(16) int s_keys[kHashSlots];  // atom index per slot, -1: free; a bucket is four consecutive slots
-    __shared__ float s_xyz[3 * kHashSlots];
-    __shared__ int s_seg_first[64];
-    __shared__ int s_seg_prefix[65];
-    __shared__ double s_shift[27][3];
-    __shared__ int s_overflow;
-
-    const unsigned lb = xcd_contiguous_block(blockIdx.x, a.n_blocks);
-    if (lb >= a.n_blocks) return;
-    const int row0 = (int)lb * a.rows_per_block;
-    const int row_end = (row0 + a.rows_per_block) < a.n_atoms ? (row0 + a.rows_per_block) : a.n_atoms;
-    if (row0 >= row_end) return;
-    const int sys_lo = bidx_ro[order_ro[row0]];
-    if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
-    const int g = threadIdx.x / LPR, sub = threadIdx.x % LPR;
-    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-
-    for (int r = row0; r < row_end;) {
-        const int sys = bidx_ro[order_ro[r]];
-        const int span0 = first_ro[sys], span_end = last_ro[sys];
-        const bool range_ok = span0 <= r && r < span_end;
-        const int seg_end = (range_ok && span_end < row_end) ? span_end : row_end;
-        const LjSysImage& image = image_ro[sys];
-        int tid = threadIdx.x;
-        asm volatile("" : "+v"(tid));
-        if (tid < 27) {
-            const int t = tid;
-            shift_vector(cells_ro + 9 * (size_t)sys, t / 9 - 1, (t / 3) % 3 - 1, t % 3 - 1, s_shift[t][0], s_shift[t][1],
-                         s_shift[t][2]);
-        }
-        if (image.img != 2) {
-            // (not this kernel's case: the row loop of the staged kernel, without a stage)
-            __syncthreads();
-            if (image.img == 1)
-                lj_rows<LPR, VIRIAL, true, SYS, false, true, 1, false>(a, r, seg_end, sys_lo, nullptr, 0, 0, s_shift, sys,
-                                                                       image.hinv, image.diag, s_acc);
-            else
-                lj_rows<LPR, VIRIAL, true, SYS, false, true, 0, false>(a, r, seg_end, sys_lo, nullptr, 0, 0, s_shift, sys,
-                                                                       image.hinv, image.diag, s_acc);
-            r = seg_end;
-            if (r < row_end) __syncthreads();
-            continue;
-        }
-        double hd[3], hdi[3];
+// rows [0, n_rows) of the staged units: row rr belongs to staged unit q with s_row0[q] <= rr < s_row0[q + 1]
+template <bool VIRIAL, bool SYS, int IMG>
+__device__ __forceinline__ void lj_tile_rows(const LjArgs& a, const LjTiles& t, int n_rows, const int4* s_unit,
+                                             const int* s_row0, const int* s_tile0, const float* __restrict__ s_pos,
+                                             const double (*s_shift)[3], const float* cells_sys, const float* s_hinv,
+                                             const double* s_diag, int sys, int sys_base,
+                                             double (*s_acc)[VIRIAL ? 7 : 1]) {
+    constexpr int LPR = 8, G = kBlockFull / LPR, UNROLL = 8;
+    float hi[9];
+    double hd[3], hdi[3];
+    if (IMG == 1) {
+#pragma unroll
+        for (int k = 0; k < 9; ++k) hi[k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(s_hinv[k])));
+    }
+    if (IMG == 2) {
 #pragma unroll
         for (int k = 0; k < 3; ++k) {
-            hd[k] = uniform_double(image.diag + k);
-            hdi[k] = uniform_double(image.diag + 3 + k);
+            hd[k] = uniform_double(s_diag + k);
+            hdi[k] = uniform_double(s_diag + 3 + k);
         }
-        // rounds are the 64-slot windows of the row order, cut at the ends of the system's rows in this workgroup
-        for (int round0 = r; round0 < seg_end;) {
-            const int window = round0 / G;
-            const int round_end = ((window + 1) * G) < seg_end ? ((window + 1) * G) : seg_end;
-            const int n_seg = hints.counts[window];
-            // ---- an empty table, and where each of the round's slices begins in the flat numbering of its atoms
-            for (int t = tid; t < kHashSlots; t += kBlockFull) s_keys[t] = -1;
-            if (tid == 0) s_overflow = n_seg < 0 ? 1 : 0;
-            if (wave == 0) {
-                int2 piece = make_int2(0, 0);
-                if (lane < n_seg) piece = hints.segments[(size_t)window * NVAMD_PAIR_ROUND_SEGMENTS + lane];
-                int incl = piece.y;
-#pragma unroll
-                for (int o = 1; o < kWave; o <<= 1) {
-                    const int up = __shfl_up(incl, o, kWave);
-                    if (lane >= o) incl += up;
-                }
-                s_seg_first[lane] = piece.x;
-                s_seg_prefix[lane] = incl - piece.y;
-                if (lane == kWave - 1) s_seg_prefix[kWave] = incl;
-            }
-            __syncthreads();
-            // ---- the neighborhood into the table: a thread takes atoms t, t + 512, ... of the flat numbering, with
-            //      kHashStage loads in flight before the first of them is entered
-            const int n_hood = s_seg_prefix[kWave];
-            for (int base = 0; base < n_hood; base += kHashStage * kBlockFull) {
-                float4 p[kHashStage];
-#pragma unroll
-                for (int q = 0; q < kHashStage; ++q) {
-                    const int flat = base + q * kBlockFull + tid;
-                    const int f = flat < n_hood ? flat : n_hood - 1;
-                    int sg = 0;  // the slice that holds flat atom f
-#pragma unroll
-                    for (int step = kWave / 2; step > 0; step >>= 1)
-                        if (s_seg_prefix[sg + step] <= f) sg += step;
-                    p[q] = hints.ordered[s_seg_first[sg] + (f - s_seg_prefix[sg])];
-                }
-#pragma unroll
-                for (int q = 0; q < kHashStage; ++q) {
-                    if (base + q * kBlockFull + tid >= n_hood) continue;
-                    const int j = __float_as_int(p[q].w);
-                    unsigned b = hash_bucket(j);
-                    bool placed = false;
-                    for (int probes = 0; probes < kHashProbes && !placed; ++probes) {
-#pragma unroll
-                        for (int k = 0; k < 4 && !placed; ++k) {
-                            const int old = atomicCAS(&s_keys[4 * b + k], -1, j);
-                            if (old == -1) {
-                                float* at = s_xyz + 3 * (4 * b + k);
-                                at[0] = p[q].x; at[1] = p[q].y; at[2] = p[q].z;
-                                placed = true;
-                            } else if (old == j) {
-                                placed = true;  // (the same atom through two slices: it is there already)
-                            }
-                        }
-                        b = (b + 1) & (kHashBuckets - 1);
-                    }
-                    if (!placed) s_overflow = 1;
-                }
-            }
-            __syncthreads();
-            if (s_overflow) {
-                // no hint, or more atoms than the table takes: this round's neighbors straight from memory
-                lj_rows<LPR, VIRIAL, true, SYS, false, true, 2, false>(a, round0, round_end, sys_lo, nullptr, 0, 0, s_shift,
-                                                                       sys, image.hinv, image.diag, s_acc);
-                __syncthreads();
-                round0 = round_end;
-                continue;
-            }
-            // ---- the pair arithmetic, neighbors through the table
-            const int k_row = round0 + g;
-            if (k_row < round_end) {
-                const float4 me = hints.ordered[k_row];
-                const int i = __float_as_int(me.w);
-                int cnt = a.nn[i];
-                cnt = cnt < a.K ? cnt : a.K;
-                const int32_t* row = a.nm + (size_t)i * a.K;
-                const int last_quad = cnt > 0 ? ((cnt - 1) & ~3) : 0;
-                double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
-                double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;
-                for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
-                    const int kb = k0 + UNROLL * sub;
-                    const int n_mine = cnt - kb;
-                    int jj[UNROLL];
-                    float4 pj[UNROLL];
-#pragma unroll
-                    for (int v = 0; v < UNROLL / 4; ++v) {
-                        const int kv = kb + 4 * v;
-                        const int4 j4 = *reinterpret_cast<const int4*>(row + (kv < last_quad ? kv : last_quad));
-                        jj[4 * v + 0] = j4.x; jj[4 * v + 1] = j4.y; jj[4 * v + 2] = j4.z; jj[4 * v + 3] = j4.w;
-                    }
-                    // the home buckets of all entries side by side (four keys in one read): nearly every neighbor is there
-                    int at[UNROLL];
-                    unsigned missed = 0;
-#pragma unroll
-                    for (int u = 0; u < UNROLL; ++u) {
-                        const unsigned b = hash_bucket(jj[u]);
-                        const int4 k4 = *reinterpret_cast<const int4*>(&s_keys[4 * b]);
-                        const int j = jj[u];
-                        const int k = k4.x == j ? 0 : (k4.y == j ? 1 : (k4.z == j ? 2 : (k4.w == j ? 3 : -1)));
-                        at[u] = 4 * (int)b + (k < 0 ? 0 : k);
-                        if (k < 0 && u < n_mine) missed |= 1u << u;
-                    }
-                    if (__builtin_expect(__builtin_amdgcn_ballot_w64(missed != 0) != 0, 0)) {
-                        // a neighbor whose home bucket was full when it came lives further on; one that is nowhere (a
-                        // list that is not this library's) is fetched from memory below
-#pragma unroll
-                        for (int u = 0; u < UNROLL; ++u) {
-                            if (!(missed & (1u << u))) continue;
-                            unsigned b = hash_bucket(jj[u]);
-                            for (int probes = 1; probes < kHashProbes; ++probes) {
-                                b = (b + 1) & (kHashBuckets - 1);
-                                const int4 k4 = *reinterpret_cast<const int4*>(&s_keys[4 * b]);
-                                const int j = jj[u];
-                                const int k = k4.x == j ? 0 : (k4.y == j ? 1 : (k4.z == j ? 2 : (k4.w == j ? 3 : -1)));
-                                if (k >= 0) {
-                                    at[u] = 4 * (int)b + k;
-                                    missed &= ~(1u << u);
-                                    break;
-                                }
-                                if (k4.w == -1) break;  // (a bucket with room ends the chain)
-                            }
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < UNROLL; ++u) {
-                        const float* q = s_xyz + 3 * at[u];
-                        pj[u].x = q[0]; pj[u].y = q[1]; pj[u].z = q[2];
-                    }
-                    if (__builtin_expect(__builtin_amdgcn_ballot_w64(missed != 0) != 0, 0)) {
-#pragma unroll
-                        for (int u = 0; u < UNROLL; ++u) {
-                            if (missed & (1u << u)) {
-                                unsigned j = (unsigned)jj[u];
-                                j = j < (unsigned)(a.n_atoms - 1) ? j : (unsigned)(a.n_atoms - 1);
-                                const float* q = a.pos + 3 * (size_t)j;
-                                pj[u].x = q[0]; pj[u].y = q[1]; pj[u].z = q[2];
-                            }
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < UNROLL; ++u) {
-                        double d0, d1, d2;
-                        const double r2 = pair_d2_nearest_diagonal(me.x, me.y, me.z, pj[u].x, pj[u].y, pj[u].z, hd, hdi, d0, d1,
-                                                                   d2);
-                        if (u >= n_mine || !(r2 < a.rc2)) continue;
-                        pair_terms<VIRIAL, false>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
-                    }
-                }
-                e = group_sum<LPR>(e);
-                fx = group_sum<LPR>(fx);
-                fy = group_sum<LPR>(fy);
-                fz = group_sum<LPR>(fz);
-                if (VIRIAL) {
-                    w0 = group_sum<LPR>(w0); w1 = group_sum<LPR>(w1); w2 = group_sum<LPR>(w2);
-                    w3 = group_sum<LPR>(w3); w4 = group_sum<LPR>(w4); w5 = group_sum<LPR>(w5);
-                }
-                if (sub == 0) {
-                    const float ef = (float)e;
-                    a.e_atom[i] = ef;
-                    float* fo = a.forces + 3 * (size_t)i;
-                    fo[0] = (float)fx;
-                    fo[1] = (float)fy;
-                    fo[2] = (float)fz;
-                    if (SYS) {
-                        const int slot = sys - sys_lo;
-                        if (slot >= 0 && slot < kSysSlots) {
-                            atomicAdd(&s_acc[slot][0], (double)ef);
-                            if (VIRIAL) {
-                                atomicAdd(&s_acc[slot][1], w0); atomicAdd(&s_acc[slot][2], w1);
-                                atomicAdd(&s_acc[slot][3], w2); atomicAdd(&s_acc[slot][4], w3);
-                                atomicAdd(&s_acc[slot][5], w4); atomicAdd(&s_acc[slot][6], w5);
-                            }
-                        } else {
-                            double* out = a.sys_acc + 10 * (size_t)sys;
-                            atomic_add_f64(out + 0, (double)ef);
-                            if (VIRIAL) {
-                                atomic_add_f64(out + 1, w0); atomic_add_f64(out + 2, w1);
-                                atomic_add_f64(out + 3, w2); atomic_add_f64(out + 5, w3);
-                                atomic_add_f64(out + 6, w4); atomic_add_f64(out + 9, w5);
-                            }
-                        }
-                    }
-                }
-            }
-            __syncthreads();  // (the table is cleared next)
-            round0 = round_end;
-        }
-        r = seg_end;
     }
-
-    if (SYS) {
-        __syncthreads();
-        if (threadIdx.x < kSysSlots * NV) {
-            const int slot = threadIdx.x / NV, k = threadIdx.x % NV;
-            const double v = s_acc[slot][k];
-            if (v != 0.0 && sys_lo + slot < a.n_systems) {
-                const int where = (k == 0) ? 0 : (k <= 3 ? k : (k <= 5 ? k + 1 : 9));
-                atomic_add_f64(a.sys_acc + 10 * (size_t)(sys_lo + slot) + where, v);
+    const int g = threadIdx.x / LPR, sub = threadIdx.x % LPR;
+    for (int rr = g; rr < n_rows; rr += G) {
+        int q = 0;
+#pragma unroll
+        for (int k = 1; k < kTileUnits; ++k) q += rr >= s_row0[k] ? 1 : 0;
+        const int4 un = s_unit[q];  // first row, rows, system, atoms in the tile (or -1)
+        const float4 me = t.xyz[un.x + (rr - s_row0[q])];
+        const int i = __float_as_int(me.w);
+        const float xi = me.x, yi = me.y, zi = me.z;
+        int cnt = a.nn[i];
+        cnt = cnt < a.K ? cnt : a.K;
+        const bool tiled = un.w > 0;
+        const int tile_last = tiled ? un.w - 1 : 0, tile0 = s_tile0[q];
+        const uint16_t* trow = t.index + (size_t)i * a.K;
+        const int32_t* row = a.nm + (size_t)i * a.K;
+        const int last_oct = cnt > 0 ? ((cnt - 1) & ~7) : 0;  // lanes beyond it re-read it: no extra lines
+        double e = 0.0, fx = 0.0, fy = 0.0, fz = 0.0;
+        double w0 = 0.0, w1 = 0.0, w2 = 0.0, w3 = 0.0, w4 = 0.0, w5 = 0.0;
+        for (int k0 = 0; k0 < cnt; k0 += UNROLL * LPR) {
+            const int kb = k0 + UNROLL * sub;
+            const int n_mine = cnt - kb;  // entry u of this lane's eight is a listed pair iff u < n_mine
+            const int kq = kb < last_oct ? kb : last_oct;
+            float xj[UNROLL], yj[UNROLL], zj[UNROLL];
+            if (__builtin_expect(tiled, 1)) {
+                const int4 w = *reinterpret_cast<const int4*>(trow + kq);
+                const unsigned packed[4] = {(unsigned)w.x, (unsigned)w.y, (unsigned)w.z, (unsigned)w.w};
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    // (the clamp keeps the reads of the slots beyond the count inside the tile)
+                    int at = (int)((u & 1) ? packed[u / 2] >> 16 : packed[u / 2] & 0xffffu);
+                    at = at < tile_last ? at : tile_last;
+                    at = (int)__umul24((unsigned)(at + tile0), 3u);
+                    xj[u] = s_pos[at + 0];
+                    yj[u] = s_pos[at + 1];
+                    zj[u] = s_pos[at + 2];
+                }
+            } else {
+                // a unit whose stencil is not one tile: its neighbors come from memory
+                const int4 ja = *reinterpret_cast<const int4*>(row + kq), jb = *reinterpret_cast<const int4*>(row + kq + 4);
+                const int jj[UNROLL] = {ja.x, ja.y, ja.z, ja.w, jb.x, jb.y, jb.z, jb.w};
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    unsigned j = (unsigned)jj[u];
+                    j = j < (unsigned)(a.n_atoms - 1) ? j : (unsigned)(a.n_atoms - 1);
+                    const float* pj = a.pos + 3 * (size_t)j;
+                    xj[u] = pj[0];
+                    yj[u] = pj[1];
+                    zj[u] = pj[2];
+                }
             }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                double d0, d1, d2, r2;
+                if (IMG == 2) {
+                    r2 = pair_d2_nearest_diagonal(xi, yi, zi, xj[u], yj[u], zj[u], hd, hdi, d0, d1, d2);
+                } else {
+                    const float dx = xj[u] - xi, dy = yj[u] - yi, dz = zj[u] - zi;
+                    const int s0 = -(int)__builtin_rintf(dx * hi[0] + dy * hi[3] + dz * hi[6]);
+                    const int s1 = -(int)__builtin_rintf(dx * hi[1] + dy * hi[4] + dz * hi[7]);
+                    const int s2 = -(int)__builtin_rintf(dx * hi[2] + dy * hi[5] + dz * hi[8]);
+                    const unsigned c0 = (unsigned)(s0 + 1), c1 = (unsigned)(s1 + 1), c2 = (unsigned)(s2 + 1);
+                    double t0 = 0.0, t1 = 0.0, t2 = 0.0;
+                    if (c0 < 3u && c1 < 3u && c2 < 3u) {
+                        const double* tv = s_shift[(c0 * 3 + c1) * 3 + c2];
+                        t0 = tv[0];
+                        t1 = tv[1];
+                        t2 = tv[2];
+                    } else if (u < n_mine) {
+                        shift_vector(cells_sys, s0, s1, s2, t0, t1, t2);
+                    }
+                    r2 = pair_d2_shifted(xi, yi, zi, xj[u], yj[u], zj[u], t0, t1, t2, d0, d1, d2);
+                }
+                if (u >= n_mine || !(r2 < a.rc2)) continue;
+                pair_terms<VIRIAL, false>(a, r2, d0, d1, d2, e, fx, fy, fz, w0, w1, w2, w3, w4, w5);
+            }
+        }
+        e = group_sum<LPR>(e);
+        fx = group_sum<LPR>(fx);
+        fy = group_sum<LPR>(fy);
+        fz = group_sum<LPR>(fz);
+        if (VIRIAL) {
+            w0 = group_sum<LPR>(w0); w1 = group_sum<LPR>(w1); w2 = group_sum<LPR>(w2);
+            w3 = group_sum<LPR>(w3); w4 = group_sum<LPR>(w4); w5 = group_sum<LPR>(w5);
+        }
+        if (sub == 0) {
+            const float ef = (float)e;
+            a.e_atom[i] = ef;
+            float* fo = a.forces + 3 * (size_t)i;
+            fo[0] = (float)fx;
+            fo[1] = (float)fy;
+            fo[2] = (float)fz;
+            if (SYS) {
+                const int slot = sys - sys_base;
+                if (slot >= 0 && slot < kSysSlots) {
+                    atomicAdd(&s_acc[slot][0], (double)ef);
+                    if (VIRIAL) {
+                        atomicAdd(&s_acc[slot][1], w0); atomicAdd(&s_acc[slot][2], w1);
+                        atomicAdd(&s_acc[slot][3], w2); atomicAdd(&s_acc[slot][4], w3);
+                        atomicAdd(&s_acc[slot][5], w4); atomicAdd(&s_acc[slot][6], w5);
+                    }
+                } else {
+                    double* out = a.sys_acc + 10 * (size_t)sys;
+                    atomic_add_f64(out + 0, (double)ef);
+                    if (VIRIAL) {
+                        atomic_add_f64(out + 1, w0); atomic_add_f64(out + 2, w1);
+                        atomic_add_f64(out + 3, w2); atomic_add_f64(out + 5, w3);
+                        atomic_add_f64(out + 6, w4); atomic_add_f64(out + 9, w5);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <bool VIRIAL, bool SYS>
+__global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_tiles_kernel(
+    LjArgs a, LjTiles t, const int2* __restrict__ records_ro, const int32_t* __restrict__ count_ro,
+    const float* __restrict__ cells_ro, const LjSysImage* __restrict__ image_ro) {
+    constexpr int NV = VIRIAL ? 7 : 1;
+    __shared__ double s_acc[kSysSlots][NV];
+    __shared__ float s_pos[3 * kTilePool];
+    __shared__ int2 s_cells[kTileUnits][kTileCells];  // per stencil cell: first slot of the cell order, offset in the tile
+    __shared__ int4 s_unit[kTileUnits];               // first row, rows, system, atoms in the tile (or -1)
+    __shared__ int4 s_staged[kTileUnits];             // the units staged together, renumbered from 0
+    __shared__ int s_row0[kTileUnits + 1];            // their first rows in the numbering of the rounds
+    __shared__ int s_tile0[kTileUnits + 1];           // where their tiles begin in the pool
+    __shared__ int s_plan[2];                         // how many units are staged together, and the system they share
+    __shared__ double s_shift[27][3];
+
+    // units are dealt to the 8 XCDs in contiguous eighths (consecutive workgroups go to the XCDs round-robin), so
+    // that the slices of the cell order that neighboring tiles share stay in one L2
+    const int total = count_ro[0];
+    const int n_groups = (total + kTileUnits - 1) / kTileUnits;
+    const int per_xcd = (n_groups + 7) / 8;
+    const int xcd = blockIdx.x % 8, slot0 = blockIdx.x / 8, stride = gridDim.x / 8;
+    if (SYS && threadIdx.x < kSysSlots * NV) (&s_acc[0][0])[threadIdx.x] = 0.0;
+
+    for (int gs = slot0; gs < per_xcd; gs += stride) {
+        // NOTE: every thread of the workgroup takes the same path through this loop body
+        const int grp = xcd * per_xcd + gs;
+        if (grp >= n_groups) break;
+        const int u0 = grp * kTileUnits;
+        const int nq = (total - u0) < kTileUnits ? (total - u0) : kTileUnits;
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        {
+            const int q = tid / kTileCells, c = tid % kTileCells;
+            if (q < nq) {
+                const int2* rec = records_ro + (size_t)(u0 + q) * kTileRecord;
+                const int2 rows = rec[0], what = rec[1];
+                if (c == 0) s_unit[q] = make_int4(rows.x, rows.y, what.x, rows.y > 0 ? what.y : -1);
+                if (what.y > 0) s_cells[q][c] = rec[2 + c];
+            }
+        }
+        __syncthreads();
+        const int sys_base = s_unit[0].z;
+        for (int q0 = 0; q0 < nq;) {
+            // units staged together: consecutive ones of one system whose tiles fit the pool
+            if (tid == 0) {
+                const int sys = s_unit[q0].z;
+                int q1 = q0, atoms = 0, rows = 0;
+                while (q1 < nq && s_unit[q1].z == sys) {
+                    const int4 un = s_unit[q1];
+                    const int n = un.w > 0 ? un.w : 0;
+                    if (atoms + n > kTilePool) break;
+                    s_staged[q1 - q0] = un;
+                    s_row0[q1 - q0] = rows;
+                    s_tile0[q1 - q0] = atoms;
+                    atoms += n;
+                    rows += un.y;
+                    ++q1;
+                }
+                for (int k = q1 - q0; k <= kTileUnits; ++k) {
+                    s_row0[k] = k == q1 - q0 ? rows : 0x7fffffff;
+                    s_tile0[k] = atoms;
+                }
+                s_plan[0] = q1 - q0;
+                s_plan[1] = sys;
+            }
+            if (tid < 27) {
+                const int sys = s_unit[q0].z;
+                shift_vector(cells_ro + 9 * (size_t)sys, tid / 9 - 1, (tid / 3) % 3 - 1, tid % 3 - 1, s_shift[tid][0],
+                             s_shift[tid][1], s_shift[tid][2]);
+            }
+            __syncthreads();
+            const int n_staged = s_plan[0], sys = s_plan[1];
+            const int n_rows = s_row0[n_staged], n_pool = s_tile0[n_staged];
+            // ---- the tiles into the pool: thread t takes atoms t, t + 512, ... of the pool, kTileLoads loads in flight
+            constexpr int kTileLoads = 4;
+            for (int base = 0; base < n_pool; base += kTileLoads * kBlockFull) {
+                float4 p[kTileLoads];
+#pragma unroll
+                for (int k = 0; k < kTileLoads; ++k) {
+                    const int at = base + k * kBlockFull + tid;
+                    const int f_all = at < n_pool ? at : n_pool - 1;
+                    int q = 0;
+#pragma unroll
+                    for (int m = 1; m < kTileUnits; ++m) q += f_all >= s_tile0[m] ? 1 : 0;
+                    const int f = f_all - s_tile0[q];
+                    const int2* cells = s_cells[q0 + q];
+                    int c = 0;  // the stencil cell that holds atom f of the tile
+#pragma unroll
+                    for (int step = kTileCells / 2; step > 0; step >>= 1)
+                        if (cells[c + step].y <= f) c += step;
+                    p[k] = t.xyz[cells[c].x + (f - cells[c].y)];
+                }
+#pragma unroll
+                for (int k = 0; k < kTileLoads; ++k) {
+                    const int at = base + k * kBlockFull + tid;
+                    if (at < n_pool) {
+                        s_pos[3 * at + 0] = p[k].x;
+                        s_pos[3 * at + 1] = p[k].y;
+                        s_pos[3 * at + 2] = p[k].z;
+                    }
+                }
+            }
+            __syncthreads();
+            const LjSysImage& image = image_ro[sys];
+            const int img = image.img;
+            if (img == 2) {
+                lj_tile_rows<VIRIAL, SYS, 2>(a, t, n_rows, s_staged, s_row0, s_tile0, s_pos, s_shift,
+                                             cells_ro + 9 * (size_t)sys, image.hinv, image.diag, sys, sys_base, s_acc);
+            } else if (img == 1) {
+                lj_tile_rows<VIRIAL, SYS, 1>(a, t, n_rows, s_staged, s_row0, s_tile0, s_pos, s_shift,
+                                             cells_ro + 9 * (size_t)sys, image.hinv, image.diag, sys, sys_base, s_acc);
+            } else {
+                // a cell too narrow for derived images: the shifts are read, the neighbors come from memory
+                for (int q = 0; q < n_staged; ++q) {
+                    const int4 un = s_staged[q];
+                    lj_rows<8, VIRIAL, true, SYS, false, true, 0, false>(a, un.x, un.x + un.y, sys_base, nullptr, 0, 0,
+                                                                         s_shift, sys, image.hinv, image.diag, s_acc);
+                }
+            }
+            __syncthreads();  // (the pool and the plan are rewritten next)
+            q0 += n_staged;
+        }
+        if (SYS) {
+            // (the systems of the next units may be others: the sums of these go out now)
+            if (threadIdx.x < kSysSlots * NV) {
+                const int slot = threadIdx.x / NV, k = threadIdx.x % NV;
+                const double v = s_acc[slot][k];
+                if (v != 0.0 && sys_base + slot < a.n_systems) {
+                    const int where = (k == 0) ? 0 : (k <= 3 ? k : (k <= 5 ? k + 1 : 9));
+                    atomic_add_f64(a.sys_acc + 10 * (size_t)(sys_base + slot) + where, v);
+                }
+                s_acc[slot][k] = 0.0;
+            }
+            __syncthreads();
         }
     }
 }
@@ -1040,8 +1044,7 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
                                      double epsilon, double sigma, double cutoff, double switch_width,
                                      int32_t half_list, float* atomic_energies, float* forces, float* virials,
                                      float* system_energies, void* workspace, size_t workspace_bytes, void* stream,
-                                     int32_t reuse_tables = 0, const float* ordered_positions = nullptr,
-                                     const int32_t* round_segments = nullptr, const int32_t* round_counts = nullptr) {
+                                     int32_t reuse_tables = 0, const LjTiles* tiles = nullptr) {
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj: negative size");
     if (!(switch_width >= 0.0) || switch_width > cutoff)
@@ -1139,25 +1142,22 @@ static int32_t lj_energy_forces_impl(const float* positions, const float* cells,
             a.sys_first = sys_first;
             a.sys_last = sys_last;
             a.sys_image = sys_image;
-            // large systems walked in the neighbor build's cell order with that build's hints, images derived, rows of
-            // 16-byte words, per-system sums wanted: the kernel that stages a round's neighborhood by hash
-            const bool hashed = a.order && ordered_positions && round_segments && round_counts && a.list_rc > 0.0 &&
-                                shifts && sys && a.inv_sw == 0.0 && n_systems > 0 && n_atoms / n_systems > kLdsAtoms &&
-                                max_neighbors >= 4 && max_neighbors % 4 == 0 && aligned16(a.nm) &&
-                                aligned16(ordered_positions);
-            if (hashed) {
-                LjArgs b = a;
-                b.rows_per_block = NVAMD_LJ_HASH_ROWS;
-                b.n_blocks = (unsigned)((n_atoms + b.rows_per_block - 1) / b.rows_per_block);
-                dim3 grid((b.n_blocks + 7) / 8 * 8), blk(kBlockFull);
-                const LjRounds hints{reinterpret_cast<const float4*>(ordered_positions),
-                                     reinterpret_cast<const int2*>(round_segments), round_counts};
+            // the tiles of the neighbor search walked again: images derived, per-system sums wanted
+            if (tiles) {
+                // (persistent workgroups, three to a CU; the number of units lives on the device)
+                int dev = 0, cus = 256;
+                hipGetDevice(&dev);
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+                dim3 grid((unsigned)((3 * cus + 7) / 8 * 8)), blk(kBlockFull);
                 if (vir)
-                    hipLaunchKernelGGL((lj_hashed_kernel<true, true>), grid, blk, 0, st, b, hints, b.bidx, b.order,
-                                       b.sys_first, b.sys_last, b.cells, b.sys_image);
+                    hipLaunchKernelGGL((lj_tiles_kernel<true, true>), grid, blk, 0, st, a, *tiles, tiles->records,
+                                       tiles->count, a.cells, a.sys_image);
+                else if (sys)
+                    hipLaunchKernelGGL((lj_tiles_kernel<false, true>), grid, blk, 0, st, a, *tiles, tiles->records,
+                                       tiles->count, a.cells, a.sys_image);
                 else
-                    hipLaunchKernelGGL((lj_hashed_kernel<false, true>), grid, blk, 0, st, b, hints, b.bidx, b.order,
-                                       b.sys_first, b.sys_last, b.cells, b.sys_image);
+                    hipLaunchKernelGGL((lj_tiles_kernel<false, false>), grid, blk, 0, st, a, *tiles, tiles->records,
+                                       tiles->count, a.cells, a.sys_image);
             } else
             switch (lanes_per_row(max_neighbors)) {
                 case 8: launch_full<8>(a, vir, shifts, sys, st); break;
@@ -1210,27 +1210,34 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_repeat(const float* positions, const
                                  system_energies, workspace, workspace_bytes, stream, reuse_tables ? 1 : 0);
 }
 
-NVAMD_EXPORT int32_t nvamd_lj_energy_forces_rounds(const float* positions, const float* cells,
-                                                    const int32_t* neighbor_matrix,
-                                                    const int32_t* neighbor_matrix_shifts,
-                                                    const int32_t* num_neighbors, const int32_t* batch_idx,
-                                                    const int32_t* row_order, const float* ordered_positions,
-                                                    const int32_t* round_segments, const int32_t* round_counts,
-                                                    double neighbor_list_cutoff, int32_t n_atoms, int32_t max_neighbors,
-                                                    int32_t n_systems, int32_t fill_value, double epsilon, double sigma,
-                                                    double cutoff, double switch_width, int32_t reuse_tables,
-                                                    float* atomic_energies, float* forces, float* virials,
-                                                    float* system_energies, void* workspace, size_t workspace_bytes,
-                                                    void* stream) {
-    const int given = (ordered_positions ? 1 : 0) + (round_segments ? 1 : 0) + (round_counts ? 1 : 0);
-    if (given != 0 && (given != 3 || !row_order))
-        return fail(NVAMD_ERR_INVALID_ARGUMENT,
-                    "lj: ordered_positions, round_segments and round_counts come together, with the row_order they belong to");
+NVAMD_EXPORT int32_t nvamd_lj_energy_forces_tiles(const float* positions, const float* cells,
+                                                   const int32_t* neighbor_matrix,
+                                                   const int32_t* neighbor_matrix_shifts,
+                                                   const int32_t* num_neighbors, const int32_t* batch_idx,
+                                                   const int32_t* row_order, const uint16_t* tile_index,
+                                                   const float* ordered_positions, const int32_t* tile_records,
+                                                   const int32_t* tile_count, double neighbor_list_cutoff,
+                                                   int32_t n_atoms, int32_t max_neighbors, int32_t n_systems,
+                                                   int32_t fill_value, double epsilon, double sigma, double cutoff,
+                                                   int32_t reuse_tables, float* atomic_energies, float* forces,
+                                                   float* virials, float* system_energies, void* workspace,
+                                                   size_t workspace_bytes, void* stream) {
+    if (n_atoms > 0 && n_systems > 0) {
+        if (!row_order || !tile_index || !ordered_positions || !tile_records || !tile_count)
+            return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj tiles: null buffer");
+        if (!cells || !neighbor_matrix_shifts || !(neighbor_list_cutoff > 0.0))
+            return fail(NVAMD_ERR_INVALID_ARGUMENT, "lj tiles: cells, shifts and the build's cutoff are needed");
+        if (max_neighbors < 8 || max_neighbors % 8 != 0 || !aligned16(neighbor_matrix) || !aligned16(tile_index) ||
+            !aligned16(ordered_positions))
+            return fail(NVAMD_ERR_UNSUPPORTED, "lj tiles: rows of 16-byte words are needed (max_neighbors a multiple of 8)");
+    }
+    const LjTiles tiles{tile_index, reinterpret_cast<const float4*>(ordered_positions),
+                        reinterpret_cast<const int2*>(tile_records), tile_count};
     return lj_energy_forces_impl(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors, batch_idx,
                                  row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
-                                 sigma, cutoff, switch_width, /*half_list=*/0, atomic_energies, forces, virials,
+                                 sigma, cutoff, /*switch_width=*/0.0, /*half_list=*/0, atomic_energies, forces, virials,
                                  system_energies, workspace, workspace_bytes, stream, reuse_tables ? 1 : 0,
-                                 ordered_positions, round_segments, round_counts);
+                                 (n_atoms > 0 && n_systems > 0) ? &tiles : nullptr);
 }
 
 // ---- the variant that allocates nothing ------------------------------------------------------

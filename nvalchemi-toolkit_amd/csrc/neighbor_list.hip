@@ -51,9 +51,9 @@ constexpr int kMaxCellsPerAxis = 1024;
 static_assert(kMaxCellsPerAxis <= 1024, "a search unit's cell coordinates are packed 10 bits each");
 constexpr int kMinCellCap = 8;    // a system may use at least this many cells
 constexpr int kMaxStencilRadius = 32;  // cells searched per axis and direction, at most
-constexpr int kPairStageAtoms = 4096;  // the pair kernel stages the positions of systems up to this size whole
-constexpr int kRoundRows = 64;         // rows of the pair kernel's rounds over large systems
-constexpr int kRoundSegments = NVAMD_PAIR_ROUND_SEGMENTS;  // slices of the sorted arrays named per round, at most
+constexpr int kTileRecord = NVAMD_NL_TILE_RECORD_INTS / 2;  // 8-byte words of a unit's record for the pair kernel
+static_assert(kTileRecord == 2 + kStencilBatch, "two words of header, then one word per stencil cell");
+static_assert(kTile <= NVAMD_NL_TILE_ATOMS, "a tile index must stay below what the header promises");
 
 struct NlSys {
     double h[9];       // rows = lattice vectors (identity without a cell)
@@ -110,8 +110,7 @@ struct NlHeader {
     int error;   // of the build in hand: NVAMD_NL_STATUS_* bits
     int total_units;
     int sticky;  // the bits of all earlier builds through this workspace since they were last cleared
-    int kept_xyz;  // the build in hand left the atoms' own coordinates in cell order (sorted_xyz)
-    int pad[11];
+    int pad[12];
 };
 
 struct NlWorkspace {
@@ -128,7 +127,6 @@ struct NlWorkspace {
     int* block_sums;     // scan partials
     float4* sorted_pos;  // (N) cell-local xyz + original index bits
     int4* sorted_aux;    // (N) wrap integers
-    float4* sorted_xyz;  // (N) the atoms' own float32 coordinates + original index bits, in cell order (large systems only)
     int max_cells;
     int n_scan_blocks;
 };
@@ -162,7 +160,6 @@ size_t carve(NlWorkspace* ws, char* base, int n_atoms, int n_systems) {
     p = take((nsb + 1) * sizeof(int)); if (ws) ws->block_sums = reinterpret_cast<int*>(p);
     p = take(N * sizeof(float4)); if (ws) ws->sorted_pos = reinterpret_cast<float4*>(p);
     p = take(N * sizeof(int4)); if (ws) ws->sorted_aux = reinterpret_cast<int4*>(p);
-    p = take(N * sizeof(float4)); if (ws) ws->sorted_xyz = reinterpret_cast<float4*>(p);
     if (ws) {
         ws->max_cells = (int)C;
         ws->n_scan_blocks = (int)nsb;
@@ -182,7 +179,12 @@ struct NlArgs {
     int n_atoms, n_systems, K, half, tail_mode;
     int unit_group;  // units are dealt to the XCDs in groups of this many (a power of two)
     int center_chunk;  // centre atoms per unit of work at most (<= kCenterChunk; smaller for small batches: more units)
-    int keep_xyz;      // also leave the atoms' own coordinates in cell order (for the pair kernel of large systems)
+    // What a pair kernel needs to walk the search's own tiles again (all null unless asked for):
+    uint16_t* tile_index;  // (N, K) per listed pair: where the neighbor stood in the tile of the centre atom's unit
+    float4* tile_xyz;      // (N) the atoms' own float32 coordinates + original index bits, in cell order
+    int2* tile_records;    // (max cells, kTileRecord) per unit: (first row, rows), (system, atoms in the tile or -1),
+                           // then per stencil cell (first slot of the cell order, offset in the tile)
+    int32_t* tile_count;   // (1) units of this build
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -251,7 +253,6 @@ __global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspac
     if (t == 0) {
         ws.hdr->sticky |= ws.hdr->error;
         ws.hdr->error = 0;
-        ws.hdr->kept_xyz = a.keep_xyz;
     }
     if (t >= a.n_systems) return;
     NlSys s;
@@ -533,9 +534,9 @@ __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspac
     int slot = ws.cell_start[b.cell] + ws.atom_rank[i];
     ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
     ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
-    if (a.keep_xyz) {
+    if (a.tile_xyz) {
         const Pos3 r = load_pos(a, (size_t)i);
-        ws.sorted_xyz[slot] = make_float4((float)r.x, (float)r.y, (float)r.z, __int_as_float(i));
+        a.tile_xyz[slot] = make_float4((float)r.x, (float)r.y, (float)r.z, __int_as_float(i));
     }
 }
 
@@ -710,9 +711,9 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         const int slot = start + rank;
         ws.sorted_pos[slot] = make_float4(b.u[0], b.u[1], b.u[2], __int_as_float(i));
         ws.sorted_aux[slot] = make_int4(b.w[0], b.w[1], b.w[2], 0);
-        if (a.keep_xyz) {
+        if (a.tile_xyz) {
             const Pos3 r = load_pos(a, (size_t)i);
-            ws.sorted_xyz[slot] = make_float4((float)r.x, (float)r.y, (float)r.z, __int_as_float(i));
+            a.tile_xyz[slot] = make_float4((float)r.x, (float)r.y, (float)r.z, __int_as_float(i));
         }
     };
     if (kept) {
@@ -764,12 +765,11 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
 }
 
 // Before nl_system_sort_kernel: the unit counter and the error flag start at zero.
-__global__ void nl_reset_kernel(NlWorkspace ws, int keep_xyz) {
+__global__ void nl_reset_kernel(NlWorkspace ws) {
     ws.hdr->total_units = 0;
     ws.hdr->total_cells = 0;  // not used on the per-system path: cell ids are not dense
     ws.hdr->sticky |= ws.hdr->error;
     ws.hdr->error = 0;
-    ws.hdr->kept_xyz = keep_xyz;
 }
 
 // ---- 7 search -------------------------------------------------------------------------------
@@ -833,7 +833,7 @@ __device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, i
 // candidates a centre cell of the run has to look at are one contiguous range of the LDS tile;
 // what a range picks up beyond its own layers (ranges are widened to multiples of 64) lies
 // further than the stencil radius away and can never pass the distance test.
-template <bool HALF, bool F64>
+template <bool HALF, bool F64, bool TILES>
 // The tables that every lane of a workgroup reads at the same address (unit records, the per-system
 // constants, the run's cell ranges) come in as read-only arguments of their own besides the workspace:
 // nothing in the kernel can be seen to write them, so they are fetched through the scalar cache, which
@@ -857,6 +857,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     __shared__ unsigned short hits[kWavesPerBlock][kHitCap + 2];
 
     const int total_units = ws.hdr->total_units;
+    if (TILES && blockIdx.x == 0 && threadIdx.x == 0) *a.tile_count = total_units;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
     const float rc2f = (float)a.rc2;
@@ -908,7 +909,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
         // One batch of stencil cells: the last wave enumerates up to 64 of them, one per lane, and scans
         // their sizes.  (The other waves load centre atoms meanwhile: the round trips to memory run
         // side by side.)  The cells' ranges need nothing but the unit record.
-        auto enumerate_stencil = [&](const int sb) {
+        auto enumerate_stencil = [&](const int sb, const bool first) {
             const int si = sb + lane;
             int start = 0, count = 0, q0 = 0, q1 = 0, q2 = 0;
             float o0 = 0.f, o1 = 0.f, o2 = 0.f;
@@ -958,18 +959,29 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
             if (lane == kWave - 1) st_prefix[kStencilBatch] = incl;
             st_q[lane][0] = q0; st_q[lane][1] = q1; st_q[lane][2] = q2;
             st_off[lane][0] = o0; st_off[lane][1] = o1; st_off[lane][2] = o2;
+            if (TILES && first) {
+                // the unit's record for the pair kernel: the tile is laid out by these numbers alone, the same for
+                // all passes of a unit; "no tile" unless the whole stencil is one batch and one tile
+                int2* const record = a.tile_records + (size_t)u * kTileRecord;
+                const int total = __shfl(incl, kWave - 1, kWave);
+                record[2 + lane] = make_int2(start, incl - count);
+                if (lane == 0) record[1] = make_int2(sidx, (one_batch && total <= kTile) ? total : -1);
+            }
         };
         // The first batch is enumerated before the run's own cell ranges have arrived.  (Nobody reads
         // the tables of the previous unit any more: its last pass ended with a barrier.)
-        if (wave == kWavesPerBlock - 1) enumerate_stencil(0);
+        if (wave == kWavesPerBlock - 1) enumerate_stencil(0, true);
         const int n_center = run_off[kMaxRun];
-        if (n_center == 0) continue;
-
         // the run's centre atoms, one pass at a time; or the one pass this unit stands for
         const int first_centre = __builtin_amdgcn_readfirstlane(grid.w);
         const int cc_begin = first_centre >= 0 ? (first_centre & 0xffffff) : 0;
         const int cc_share = first_centre >= 0 ? (first_centre >> 24) : n_center;
         const int cc_end = (cc_begin + cc_share) < n_center ? (cc_begin + cc_share) : n_center;
+        // the unit's rows for the pair kernel (slots of the cell order); the rest of its record is written with the
+        // stencil tables
+        if (TILES && threadIdx.x == 0)
+            a.tile_records[(size_t)u * kTileRecord] = make_int2(c_begin + cc_begin, cc_end > cc_begin ? cc_end - cc_begin : 0);
+        if (n_center == 0) continue;
         for (int cc0 = cc_begin; cc0 < cc_end; cc0 += kCenterChunk) {
             const int n_cc = (cc_end - cc0) < kCenterChunk ? (cc_end - cc0) : kCenterChunk;
             int pad_end = 0;
@@ -995,7 +1007,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
             }
 
             for (int sb = 0; sb < n_stencil; sb += kStencilBatch) {
-                if (wave == kWavesPerBlock - 1 && !(sb == 0 && cc0 == cc_begin)) enumerate_stencil(sb);
+                if (wave == kWavesPerBlock - 1 && !(sb == 0 && cc0 == cc_begin)) enumerate_stencil(sb, false);
                 __syncthreads();
                 const int batch_total = st_prefix[kStencilBatch];
                 const int n_entries = (n_stencil - sb) < kStencilBatch ? (n_stencil - sb) : kStencilBatch;
@@ -1170,6 +1182,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                                                                   __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
                                 if (in && slot < a.K) {
                                     row[slot] = j;
+                                    if (TILES) a.tile_index[(size_t)i_atom * a.K + slot] = (uint16_t)k;
                                     if (srow) {
                                         srow[3 * slot + 0] = s0;
                                         srow[3 * slot + 1] = s1;
@@ -1280,93 +1293,6 @@ __global__ __launch_bounds__(kBlock) void nl_atom_order_kernel(const float4* __r
     order[k] = __float_as_int(sorted_pos[k].w);
 }
 
-// ---- what the pair kernel of large systems takes over from a build -----------------------------------------
-// The atoms in cell order with their own coordinates (a copy out of the workspace, which the next build overwrites) ...
-__global__ __launch_bounds__(kBlock) void nl_ordered_positions_kernel(NlWorkspace ws, int n_atoms,
-                                                                      int32_t* __restrict__ order,
-                                                                      float4* __restrict__ ordered) {
-    const int k = blockIdx.x * kBlock + threadIdx.x;
-    if (k >= n_atoms) return;
-    const bool kept = ws.hdr->kept_xyz != 0;
-    const float4 p = kept ? ws.sorted_xyz[k] : ws.sorted_pos[k];
-    order[k] = __float_as_int(p.w);
-    ordered[k] = p;  // (without kept coordinates the rounds below all say "no hint": nobody reads the xyz)
-}
-
-// ... and, for every round of kRoundRows consecutive slots of the cell order, the slices of that order that hold
-// every atom within the stencil of the round's cells: a handful of (first slot, length) pairs, because a column of
-// cells along axis 2 is one slice.  A count of -1 says "no hint" (the round spans two systems, its system was not
-// built with kept coordinates, or it needs more slices than the table has room for).
-__global__ __launch_bounds__(kBlock) void nl_pair_rounds_kernel(NlWorkspace ws, const int32_t* __restrict__ bidx,
-                                                                int n_atoms, int n_rounds, int2* __restrict__ segments,
-                                                                int32_t* __restrict__ counts) {
-    const int w = blockIdx.x * kBlock + threadIdx.x;
-    if (w >= n_rounds) return;
-    const int s_lo = w * kRoundRows, s_hi = (s_lo + kRoundRows < n_atoms ? s_lo + kRoundRows : n_atoms) - 1;
-    const int sidx = bidx[s_lo];
-    int n = -1;
-    if (ws.hdr->kept_xyz && bidx[s_hi] == sidx) {
-        const NlSys& S = ws.sys[sidx];
-        const int nc0 = S.nc[0], nc1 = S.nc[1], nc2 = S.nc[2];
-        const int* start = ws.cell_start + S.cell_offset;  // S.n_cells + 1 entries
-        auto cell_of = [&](int slot) {  // the last cell that begins at or before the slot
-            int lo = 0, hi = S.n_cells;
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) >> 1;
-                if (start[mid] <= slot) lo = mid; else hi = mid;
-            }
-            return lo;
-        };
-        if (S.n_cells > 0) {
-            const int c_a = cell_of(s_lo), c_b = cell_of(s_hi);
-            const int col_a = c_a / nc2, col_b = c_b / nc2;
-            int2* out = segments + (size_t)w * kRoundSegments;
-            n = 0;
-            for (int col = col_a; col <= col_b && n >= 0; ++col) {
-                const int z_lo = (col == col_a ? c_a - col_a * nc2 : 0) - S.R[2];
-                const int z_hi = (col == col_b ? c_b - col_b * nc2 : nc2 - 1) + S.R[2];
-                const int cx = col / nc1, cy = col - cx * nc1;
-                for (int dx = -S.R[0]; dx <= S.R[0] && n >= 0; ++dx) {
-                    int gx = cx + dx;
-                    if (S.per[0]) gx -= floordiv(gx, nc0) * nc0; else if (gx < 0 || gx >= nc0) continue;
-                    for (int dy = -S.R[1]; dy <= S.R[1] && n >= 0; ++dy) {
-                        int gy = cy + dy;
-                        if (S.per[1]) gy -= floordiv(gy, nc1) * nc1; else if (gy < 0 || gy >= nc1) continue;
-                        const int base = (gx * nc1 + gy) * nc2;
-                        // the range of cells along axis 2, in one piece or (through the periodic boundary) in two
-                        int p_lo[2], p_hi[2], pieces = 1;
-                        p_lo[0] = z_lo; p_hi[0] = z_hi;
-                        if (!S.per[2]) {
-                            p_lo[0] = z_lo < 0 ? 0 : z_lo;
-                            p_hi[0] = z_hi > nc2 - 1 ? nc2 - 1 : z_hi;
-                        } else if (z_hi - z_lo + 1 >= nc2) {
-                            p_lo[0] = 0; p_hi[0] = nc2 - 1;
-                        } else if (z_lo < 0) {
-                            // (z_lo > -nc2 here: the span is shorter than the axis)
-                            pieces = 2;
-                            p_lo[0] = z_lo + nc2; p_hi[0] = nc2 - 1;
-                            p_lo[1] = 0; p_hi[1] = z_hi;
-                        } else if (z_hi > nc2 - 1) {
-                            pieces = 2;
-                            p_lo[0] = z_lo; p_hi[0] = nc2 - 1;
-                            p_lo[1] = 0; p_hi[1] = z_hi - nc2;
-                        }
-                        for (int k = 0; k < pieces; ++k) {
-                            if (p_hi[k] < p_lo[k]) continue;
-                            const int first = start[base + p_lo[k]];
-                            const int len = start[base + p_hi[k] + 1] - first;
-                            if (len <= 0) continue;
-                            if (n >= kRoundSegments) { n = -1; break; }
-                            out[n++] = make_int2(first, len);
-                        }
-                    }
-                }
-            }
-        }
-    }
-    counts[w] = n;
-}
-
 }  // namespace
 }  // namespace nvamd
 
@@ -1386,29 +1312,6 @@ NVAMD_EXPORT int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace
     hipLaunchKernelGGL(nl_atom_order_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0,
                        static_cast<hipStream_t>(stream), ws.sorted_pos, batch_idx, rebuild_flags, n_atoms, atom_order);
     NVAMD_LAUNCH_CHECK("atom order launch");
-    return NVAMD_OK;
-}
-
-NVAMD_EXPORT int32_t nvamd_nl_pair_hints(const void* workspace, size_t workspace_bytes, const int32_t* batch_idx,
-                                         int32_t n_atoms, int32_t n_systems, int32_t* atom_order,
-                                         float* ordered_positions, int32_t* round_segments, int32_t* round_counts,
-                                         void* stream) {
-    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "pair hints: negative size");
-    if (n_atoms == 0 || n_systems == 0) return NVAMD_OK;
-    if (!batch_idx || !atom_order || !ordered_positions || !round_segments || !round_counts)
-        return fail(NVAMD_ERR_INVALID_ARGUMENT, "pair hints: null buffer");
-    size_t need = carve(nullptr, nullptr, n_atoms, n_systems);
-    if (!workspace || workspace_bytes < need)
-        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "pair hints: workspace %zu < %zu bytes", workspace_bytes, need);
-    NlWorkspace ws;
-    carve(&ws, static_cast<char*>(const_cast<void*>(workspace)), n_atoms, n_systems);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(nl_ordered_positions_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws,
-                       n_atoms, atom_order, reinterpret_cast<float4*>(ordered_positions));
-    const int n_rounds = (n_atoms + kRoundRows - 1) / kRoundRows;
-    hipLaunchKernelGGL(nl_pair_rounds_kernel, dim3((n_rounds + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws, batch_idx,
-                       n_atoms, n_rounds, reinterpret_cast<int2*>(round_segments), round_counts);
-    NVAMD_LAUNCH_CHECK("pair hints launch");
     return NVAMD_OK;
 }
 
@@ -1450,7 +1353,9 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
                              const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems, double cutoff,
                              int32_t max_neighbors, int32_t half_fill, int32_t tail_mode, int32_t sort_path,
                              int32_t* neighbor_matrix, int32_t* num_neighbors, int32_t* neighbor_matrix_shifts,
-                             void* workspace, size_t workspace_bytes, void* stream) {
+                             void* workspace, size_t workspace_bytes, void* stream, uint16_t* tile_index = nullptr,
+                             float* ordered_positions = nullptr, int32_t* tile_records = nullptr,
+                             int32_t* tile_count = nullptr) {
     if (sort_path != NVAMD_NL_SORT_AUTO && sort_path != NVAMD_NL_SORT_PER_SYSTEM && sort_path != NVAMD_NL_SORT_GLOBAL)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: unknown sort_path %d", (int)sort_path);
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
@@ -1470,6 +1375,14 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
         return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "nl: workspace %zu < %zu bytes", workspace_bytes, need);
     if (max_cells_for(n_atoms, n_systems) > 0x7fffffffull)
         return fail(NVAMD_ERR_UNSUPPORTED, "nl: too many cells");
+    if (tile_index) {
+        if (!ordered_positions || !tile_records || !tile_count)
+            return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: the tile outputs come together");
+        if (!positions || half_fill || rebuild_flags || max_neighbors % 8 != 0)
+            return fail(NVAMD_ERR_UNSUPPORTED,
+                        "nl: tiles are written for float32 positions, a full list, a build of every system and "
+                        "max_neighbors a multiple of 8");
+    }
 
     NlWorkspace ws;
     carve(&ws, static_cast<char*>(workspace), n_atoms, n_systems);
@@ -1491,8 +1404,10 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     while (a.unit_group < 64 && (long long)a.unit_group * 8192 <= (long long)n_atoms) a.unit_group *= 2;
     // A small batch does not fill the chip with units of kCenterChunk centre atoms: smaller units, about 4096 of them
     a.center_chunk = NVAMD_NL_CHUNK(n_atoms);
-    // systems too large for the pair kernel to stage whole: their atoms' own coordinates stay behind in cell order
-    a.keep_xyz = (positions != nullptr && n_atoms / n_systems > kPairStageAtoms) ? 1 : 0;
+    a.tile_index = tile_index;
+    a.tile_xyz = reinterpret_cast<float4*>(ordered_positions);
+    a.tile_records = reinterpret_cast<int2*>(tile_records);
+    a.tile_count = tile_count;
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
@@ -1507,7 +1422,7 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
                                                             : (sort_path == NVAMD_NL_SORT_PER_SYSTEM);
     if (per_system) {
         // many small systems: set-up to scatter in one workgroup per system
-        hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws, a.keep_xyz);
+        hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws);
         hipLaunchKernelGGL(nl_system_sort_kernel, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
     } else {
         size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
@@ -1525,8 +1440,11 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     size_t cells_bound = max_cells_for(n_atoms, n_systems);
     if (cells_bound < n_search) n_search = (unsigned)((cells_bound + 7) / 8 * 8);
 #define NVAMD_NL_SEARCH(H, D) \
-    hipLaunchKernelGGL((nl_search_kernel<H, D>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start)
-    if (a.pos64) {
+    hipLaunchKernelGGL((nl_search_kernel<H, D, false>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start)
+    if (a.tile_index) {
+        hipLaunchKernelGGL((nl_search_kernel<false, false, true>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys,
+                           ws.cell_start);
+    } else if (a.pos64) {
         if (a.half) NVAMD_NL_SEARCH(true, true);
         else NVAMD_NL_SEARCH(false, true);
     } else {
@@ -1548,6 +1466,26 @@ NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* ce
     return nl_build_impl(positions, cell, nullptr, nullptr, pbc, batch_ptr, batch_idx, rebuild_flags, n_atoms, n_systems,
                          cutoff, max_neighbors, half_fill, tail_mode, sort_path, neighbor_matrix, num_neighbors,
                          neighbor_matrix_shifts, workspace, workspace_bytes, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_build_tiles(const float* positions, const float* cell, const uint8_t* pbc,
+                                          const int32_t* batch_ptr, const int32_t* batch_idx, int32_t n_atoms,
+                                          int32_t n_systems, double cutoff, int32_t max_neighbors, int32_t tail_mode,
+                                          int32_t sort_path, int32_t* neighbor_matrix, int32_t* num_neighbors,
+                                          int32_t* neighbor_matrix_shifts, uint16_t* tile_index, float* ordered_positions,
+                                          int32_t* tile_records, int32_t* tile_count, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    if (n_atoms > 0 && n_systems > 0 && (!tile_index || !ordered_positions || !tile_records || !tile_count))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl tiles: null buffer");
+    return nl_build_impl(positions, cell, nullptr, nullptr, pbc, batch_ptr, batch_idx, nullptr, n_atoms, n_systems, cutoff,
+                         max_neighbors, 0, tail_mode, sort_path, neighbor_matrix, num_neighbors, neighbor_matrix_shifts,
+                         workspace, workspace_bytes, stream, tile_index, ordered_positions, tile_records, tile_count);
+}
+
+NVAMD_EXPORT int32_t nvamd_nl_tile_records(int32_t n_atoms, int32_t n_systems, size_t* records) {
+    if (!records || n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl tile records: bad argument");
+    *records = max_cells_for(n_atoms, n_systems);
+    return NVAMD_OK;
 }
 
 NVAMD_EXPORT int32_t nvamd_nl_build_f64(const double* positions, const double* cell, const uint8_t* pbc,

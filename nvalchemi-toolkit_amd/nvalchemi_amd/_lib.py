@@ -56,8 +56,9 @@ _SIGNATURES = {
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_lj_energy_forces_hinted": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_repeat": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
-    "nvamd_lj_energy_forces_rounds": (_i32, [_vp] * 10 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
-    "nvamd_nl_pair_hints": (_i32, [_vp, _c.c_size_t, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "nvamd_lj_energy_forces_tiles": (_i32, [_vp] * 11 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 3 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
+    "nvamd_nl_build_tiles": (_i32, [_vp] * 5 + [_i32, _i32, _c.c_double, _i32, _i32, _i32] + [_vp] * 8 + [_c.c_size_t, _vp]),
+    "nvamd_nl_tile_records": (_i32, [_i32, _i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_lj_energy_forces_static": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_vp] * 5),
     "nvamd_nl_atom_order": (_i32, [_vp, _c.c_size_t, _vp, _vp, _i32, _i32, _vp, _vp]),
     "nvamd_segment_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
@@ -241,7 +242,10 @@ nl_sort_path = NL_SORT_AUTO
 
 def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, max_neighbors,
              half_fill, tail_mode, neighbor_matrix, num_neighbors, neighbor_matrix_shifts,
-             workspace: torch.Tensor | None = None, sort_path: int | None = None) -> None:
+             workspace: torch.Tensor | None = None, sort_path: int | None = None, pair_tiles=None) -> None:
+    """``pair_tiles``: ``(tile_index (N,K) i16, ordered_positions (N,4) f32, tile_records (R, NL_TILE_RECORD_INTS) i32,
+    tile_count (1) i32)``, R = ``nl_tile_records(N, B)``: also leave behind what the pair kernel of large systems
+    walks (float32 positions, full list, every system built, K a multiple of 8)."""
     lib = library()
     if sort_path is None:
         sort_path = nl_sort_path
@@ -263,11 +267,30 @@ def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, 
     ws = workspace if workspace is not None else workspaces.get(positions.device, "nl", need)
     if ws.device != positions.device or ws.numel() * ws.element_size() < need:
         raise ValueError("neighbor-list workspace too small or on another device")
+    if pair_tiles is not None:
+        if real != torch.float32 or half_fill or rebuild_flags is not None:
+            raise ValueError("pair tiles need float32 positions, a full list and a build of every system")
+        index, ordered, records, count = pair_tiles
+        _check(lib.nvamd_nl_build_tiles(
+            p_pos, p_cell, p_pbc, p_ptr, p_idx, N, B, float(cutoff), K, int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
+            _dev(index, "tile_index", torch.int16, (N, K)), _dev(ordered, "ordered_positions", torch.float32, (N, 4)),
+            _dev(records, "tile_records", torch.int32, (nl_tile_records(N, B), NL_TILE_RECORD_INTS)),
+            _dev(count, "tile_count", torch.int32, (1,)),
+            ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)), "nvamd_nl_build_tiles")
+        return
     entry = lib.nvamd_nl_build_f64 if real == torch.float64 else lib.nvamd_nl_build_path
     _check(entry(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,
                  int(bool(half_fill)), int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
                  ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)),
            "nvamd_nl_build")
+
+
+NL_TILE_RECORD_INTS = 132
+
+
+def nl_tile_records(n_atoms: int, n_systems: int) -> int:
+    """Rows of the ``tile_records`` table that a build of this size may write."""
+    return _size(library().nvamd_nl_tile_records, int(n_atoms), int(n_systems))
 
 
 NL_STATUS_CELL_TOO_THIN = 1
@@ -338,9 +361,9 @@ def nl_matrix_to_coo(neighbor_matrix, neighbor_matrix_shifts, edge_ptr, neighbor
 def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors,
                      batch_idx, fill_value, epsilon, sigma, cutoff, switch_width, half_list,
                      atomic_energies, forces, virials=None, system_energies=None, row_order=None,
-                     neighbor_list_cutoff: float = 0.0, pair_hints=None) -> None:
-    """``pair_hints``: ``(ordered_positions (N,4) f32, round_segments, round_counts)`` of ``nl_pair_hints`` for the
-    positions in hand and the ``row_order`` given with them (full list only; ignored otherwise)."""
+                     neighbor_list_cutoff: float = 0.0, pair_tiles=None) -> None:
+    """``pair_tiles``: the four ``pair_tiles`` tensors of the ``nl_build`` that made this matrix from the positions in
+    hand, with the ``row_order`` of that build (full list, no switching, shifts given; ignored otherwise)."""
     lib = library()
     N = positions.shape[0]
     K = neighbor_matrix.shape[1]
@@ -371,27 +394,27 @@ def lj_energy_forces(positions, cells, neighbor_matrix, neighbor_matrix_shifts, 
         state = (positions.device.index, _stream(positions.device))
         reuse = _lj_tables.get(state) == tables
         _lj_tables[state] = tables
-        if pair_hints is not None and row_order is not None:
-            ordered, segments, counts = pair_hints
-            R = (N + PAIR_ROUND_ROWS - 1) // PAIR_ROUND_ROWS
-            _check(lib.nvamd_lj_energy_forces_rounds(
+        if (pair_tiles is not None and row_order is not None and neighbor_matrix_shifts is not None
+                and float(switch_width) == 0.0 and float(neighbor_list_cutoff) > 0.0 and K % 8 == 0):
+            index, ordered, records, count = pair_tiles
+            _check(lib.nvamd_lj_energy_forces_tiles(
                 _dev(positions, "positions", torch.float32, (N, 3)),
                 _dev(cells, "cells", torch.float32, (B, 3, 3)),
                 _dev(neighbor_matrix, "neighbor_matrix", torch.int32, (N, K)),
-                _opt(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
+                _dev(neighbor_matrix_shifts, "neighbor_matrix_shifts", torch.int32, (N, K, 3)),
                 _dev(num_neighbors, "num_neighbors", torch.int32, (N,)),
                 _dev(batch_idx, "batch_idx", torch.int32, (N,)),
                 _dev(row_order, "row_order", torch.int32, (N,)),
+                _dev(index, "tile_index", torch.int16, (N, K)),
                 _dev(ordered, "ordered_positions", torch.float32, (N, 4)),
-                _dev(segments, "round_segments", torch.int32, (R, PAIR_ROUND_SEGMENTS, 2)),
-                _dev(counts, "round_counts", torch.int32, (R,)), float(neighbor_list_cutoff),
-                N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), float(switch_width),
-                int(reuse),
+                _dev(records, "tile_records", torch.int32, (nl_tile_records(N, B), NL_TILE_RECORD_INTS)),
+                _dev(count, "tile_count", torch.int32, (1,)), float(neighbor_list_cutoff),
+                N, K, B, int(fill_value), float(epsilon), float(sigma), float(cutoff), int(reuse),
                 _dev(atomic_energies, "atomic_energies", torch.float32, (N,)),
                 _dev(forces, "forces", torch.float32, (N, 3)),
                 _opt(virials, "virials", torch.float32, (B, 9)),
                 _opt(system_energies, "system_energies", torch.float32, (B,)),
-                ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_rounds")
+                ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_lj_energy_forces_tiles")
             return
         _check(lib.nvamd_lj_energy_forces_repeat(
             _dev(positions, "positions", torch.float32, (N, 3)),
@@ -458,25 +481,6 @@ def lj_energy_forces_static(positions, cells, neighbor_matrix, neighbor_matrix_s
         _opt(virials, "virials", torch.float32, (B, 9)),
         _opt(system_energies, "system_energies", torch.float32, (B,)),
         _stream(positions.device)), "nvamd_lj_energy_forces_static")
-
-
-PAIR_ROUND_ROWS, PAIR_ROUND_SEGMENTS = 64, 40
-
-
-def nl_pair_hints(batch_idx, n_systems: int, atom_order, ordered_positions, round_segments, round_counts) -> None:
-    """What the pair kernel takes over from the last neighbor build on this device and stream (same sizes): the cell
-    order, the positions in that order, and per round of 64 rows the slices of the order that hold its neighborhood."""
-    lib = library()
-    N = batch_idx.shape[0]
-    R = (N + PAIR_ROUND_ROWS - 1) // PAIR_ROUND_ROWS
-    need = _size(lib.nvamd_nl_workspace_bytes, N, int(n_systems))
-    ws = workspaces.get(batch_idx.device, "nl", need)
-    _check(lib.nvamd_nl_pair_hints(
-        ws.data_ptr(), ws.numel(), _dev(batch_idx, "batch_idx", torch.int32, (N,)), N, int(n_systems),
-        _dev(atom_order, "atom_order", torch.int32, (N,)),
-        _dev(ordered_positions, "ordered_positions", torch.float32, (N, 4)),
-        _dev(round_segments, "round_segments", torch.int32, (R, PAIR_ROUND_SEGMENTS, 2)),
-        _dev(round_counts, "round_counts", torch.int32, (R,)), _stream(batch_idx.device)), "nvamd_nl_pair_hints")
 
 
 def nl_atom_order(batch_idx, n_systems: int, atom_order, rebuild_flags=None) -> None:

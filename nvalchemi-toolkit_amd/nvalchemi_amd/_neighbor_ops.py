@@ -62,7 +62,8 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
                   num_neighbors: torch.Tensor | None = None,
                   neighbor_matrix_shifts: torch.Tensor | None = None,
                   rebuild_flags: torch.Tensor | None = None, method: str | None = None,
-                  tail_mode: int = 1, **scratch) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+                  tail_mode: int = 1, pair_tiles: tuple | None = None,
+                  **scratch) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
     """Build the dense neighbor list in place and return ``(neighbor_matrix, num_neighbors,
     neighbor_matrix_shifts)``.
 
@@ -74,6 +75,8 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
     kernel serves every case); scratch keyword tensors of the reference's strategies are
     ignored.  ``tail_mode=1`` rewrites the padding of every rebuilt row; ``0`` only clears
     what the previous build left (persistent buffers that only this function writes).
+    ``pair_tiles`` (not in the reference): four preallocated tensors in which the build also leaves what the
+    pair kernel of large systems walks, see ``_lib.nl_build``.
     """
     if method not in _METHODS:
         raise ValueError(f"unknown neighbor list method {method!r}")
@@ -106,7 +109,8 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
         neighbor_matrix_shifts = torch.zeros((N, K, 3), dtype=torch.int32, device=dev)
     _lib.nl_build(positions.contiguous(), cell, pbc, batch_ptr.to(torch.int32).contiguous(),
                   batch_idx.to(torch.int32).contiguous(), rebuild_flags, cutoff, K, half_fill, tail_mode,
-                  neighbor_matrix, num_neighbors, neighbor_matrix_shifts if cell is not None else None)
+                  neighbor_matrix, num_neighbors, neighbor_matrix_shifts if cell is not None else None,
+                  pair_tiles=pair_tiles)
     return neighbor_matrix, num_neighbors, neighbor_matrix_shifts
 
 

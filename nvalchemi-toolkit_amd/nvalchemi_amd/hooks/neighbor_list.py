@@ -84,6 +84,9 @@ class NeighborListHook:
         # Verlet-skin state: positions at the last build of each system, per-system flags
         self._ref_positions: torch.Tensor | None = None
         self._rebuild_flags: torch.Tensor | None = None
+        # what a full build leaves for the pair kernel of large systems, and whether the last build wrote it
+        self._tiles: tuple | None = None
+        self._tiles_fresh: bool = False
 
     def __call__(self, ctx: HookContext, stage: Enum) -> None:
         self._rebuild(ctx.batch)
@@ -172,7 +175,7 @@ class NeighborListHook:
 
         return (ptr(self._neighbor_matrix), ptr(self._num_neighbors), ptr(self._neighbor_matrix_shifts),
                 ptr(self._ref_positions), ptr(self._rebuild_flags), ptr(getattr(self, "_atom_order", None)),
-                ptr(getattr(self, "_ordered_positions", None)))
+                None if self._tiles is None else tuple(ptr(t) for t in self._tiles))
 
     def overflowed(self, clear: bool = True) -> bool:
         """Whether any build since the last call left an atom with more neighbors than the rows hold
@@ -193,50 +196,58 @@ class NeighborListHook:
         atoms' cell order of this build on the batch (``_neighbor_row_order``): a pair kernel that
         walks its rows in that order gathers neighbor positions from the caches instead of HBM.
         Not part of the reference; purely a hint (any model may ignore it)."""
+        tiles = self._tiles if self._tiles_fresh else None
+        self._tiles_fresh = False
         if N == 0 or batch.max_num_nodes <= self._ROW_ORDER_MIN_ATOMS:
             if getattr(batch, "_neighbor_row_order", None) is not None:
                 object.__setattr__(batch, "_neighbor_row_order", None)
-            if getattr(batch, "_neighbor_pair_hints", None) is not None:
-                object.__setattr__(batch, "_neighbor_pair_hints", None)
+            if getattr(batch, "_neighbor_pair_tiles", None) is not None:
+                object.__setattr__(batch, "_neighbor_pair_tiles", None)
             self._atom_order = None
             return
         fresh = (getattr(self, "_atom_order", None) is None or self._atom_order.shape[0] != N
                  or self._atom_order.device != batch.positions.device)
         if fresh:
             self._atom_order = torch.empty(N, dtype=torch.int32, device=batch.positions.device)
-        if self.skin <= 0.0 and batch.positions.dtype == torch.float32 and N // max(B, 1) > self._ROW_ORDER_MIN_ATOMS:
-            # Every call is a full build on the positions in hand: besides the order, the pair kernel can take the
-            # positions in that order and, per round of 64 rows, the slices of the order that hold the round's
-            # neighborhood (it then reads its neighbors with contiguous loads instead of one gather per pair).
-            R = (N + _lib.PAIR_ROUND_ROWS - 1) // _lib.PAIR_ROUND_ROWS
-            if fresh or getattr(self, "_ordered_positions", None) is None or self._ordered_positions.shape[0] != N:
-                dev = batch.positions.device
-                self._ordered_positions = torch.empty(N, 4, dtype=torch.float32, device=dev)
-                self._round_segments = torch.empty(R, _lib.PAIR_ROUND_SEGMENTS, 2, dtype=torch.int32, device=dev)
-                self._round_counts = torch.empty(R, dtype=torch.int32, device=dev)
-            _lib.nl_pair_hints(batch.batch_idx, B, self._atom_order, self._ordered_positions, self._round_segments,
-                               self._round_counts)
-            object.__setattr__(batch, "_neighbor_row_order", self._atom_order)
-            # (tied to the positions of this build: storage and version)
-            object.__setattr__(batch, "_neighbor_pair_hints",
-                               (self._ordered_positions, self._round_segments, self._round_counts,
-                                batch.positions.data_ptr(), batch.positions._version))
-            return
-        if getattr(batch, "_neighbor_pair_hints", None) is not None:
-            object.__setattr__(batch, "_neighbor_pair_hints", None)
         flags = None
         if not fresh and self.skin > 0.0 and self._ref_positions is not None:
             flags = self._rebuild_flags  # systems that were not rebuilt keep the order of their last build
         _lib.nl_atom_order(batch.batch_idx, B, self._atom_order, flags)
         object.__setattr__(batch, "_neighbor_row_order", self._atom_order)
+        # what the last build left for the pair kernel, tied to the positions and the matrix of that build
+        # (storage and version)
+        object.__setattr__(batch, "_neighbor_pair_tiles",
+                           None if tiles is None else
+                           tiles + (batch.positions.data_ptr(), batch.positions._version,
+                                    self._neighbor_matrix.data_ptr()))
+
+    def _pair_tiles_for(self, batch, cell, rebuild_flags):
+        """Buffers for what a full build leaves to the pair kernel of systems too large to stage whole (the atoms in
+        cell order, the search's tiles, each pair's place in its tile), or None where that does not apply: lists kept
+        over several steps, half lists, float64, open systems, small systems."""
+        N, B = batch.num_nodes, batch.num_graphs
+        K = self._max_neighbors
+        if (self.skin > 0.0 or rebuild_flags is not None or self.config.half_list or cell is None or N == 0
+                or batch.positions.dtype != torch.float32 or N // max(B, 1) <= self._ROW_ORDER_MIN_ATOMS or K % 8 != 0):
+            return None
+        dev = batch.positions.device
+        t = self._tiles
+        if t is None or tuple(t[0].shape) != (N, K) or t[0].device != dev or t[2].shape[0] != _lib.nl_tile_records(N, B):
+            t = (torch.empty(N, K, dtype=torch.int16, device=dev), torch.empty(N, 4, dtype=torch.float32, device=dev),
+                 torch.empty(_lib.nl_tile_records(N, B), _lib.NL_TILE_RECORD_INTS, dtype=torch.int32, device=dev),
+                 torch.zeros(1, dtype=torch.int32, device=dev))
+            self._tiles = t
+        return t
 
     def _build(self, batch, cutoff, cell, pbc, rebuild_flags) -> None:
+        tiles = self._pair_tiles_for(batch, cell, rebuild_flags)
         neighbor_list(positions=batch.positions, cutoff=cutoff, cell=cell, pbc=pbc,
                       max_neighbors=self._max_neighbors, half_fill=self.config.half_list,
                       batch_ptr=batch.batch_ptr, batch_idx=batch.batch_idx,
                       neighbor_matrix=self._neighbor_matrix, num_neighbors=self._num_neighbors,
                       neighbor_matrix_shifts=self._neighbor_matrix_shifts, rebuild_flags=rebuild_flags,
-                      method=self._neighbor_list_method, tail_mode=0)
+                      method=self._neighbor_list_method, tail_mode=0, pair_tiles=tiles)
+        self._tiles_fresh = tiles is not None
 
     # ------------------------------------------------------------------
     def _alloc_output_tensors(self, N: int, batch, pbc: torch.Tensor | None) -> None:

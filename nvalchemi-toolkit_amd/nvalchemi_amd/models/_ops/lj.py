@@ -97,7 +97,7 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
                                   cutoff: float, switch_width: float, half_list: bool,
                                   compute_virial: bool = False, out: dict | None = None,
                                   row_order: Tensor | None = None, neighbor_list_cutoff: float = 0.0,
-                                  pair_hints: tuple | None = None):
+                                  pair_tiles: tuple | None = None):
     """Fused launch: ``(atomic_energies (N), forces (N,3), system_energies (B), virials (B,9) |
     None)``.  ``neighbor_matrix_shifts=None`` means all shifts are zero (no ``(N,K,3)`` zeros
     tensor is needed).  ``out`` may carry preallocated result tensors under those names.
@@ -105,9 +105,9 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
     order of the neighbor build) only changes the order in which rows are worked on.
     ``neighbor_list_cutoff`` (the radius the matrix was searched with, 0.0 if unknown) lets the
     kernel derive shifts from positions, instead of reading them, in systems whose cell is wider
-    than twice that radius in every direction; the results are the same.  ``pair_hints`` (what the
-    neighbor hook leaves for systems too large to stage: the positions in ``row_order`` and the slices of that
-    order that hold each round's neighborhood) changes where neighbor positions are read from, nothing else."""
+    than twice that radius in every direction; the results are the same.  ``pair_tiles`` (what the
+    neighbor hook leaves for systems too large to stage: the positions in ``row_order``, the tiles of the search
+    and each pair's place in its tile) changes where neighbor positions are read from, nothing else."""
     _check_dtype(positions)
     N = positions.shape[0]
     B = cells.shape[0]
@@ -130,5 +130,5 @@ def lj_energy_forces_system_batch(positions: Tensor, cells: Tensor, neighbor_mat
     _lib.lj_energy_forces(positions, cells.to(dt), neighbor_matrix, _shifts_or_none(neighbor_matrix_shifts),
                           num_neighbors, batch_idx, fill_value, epsilon, sigma, cutoff, switch_width,
                           half_list, e, f, virials=w, system_energies=es, row_order=row_order,
-                          neighbor_list_cutoff=neighbor_list_cutoff, pair_hints=None if half_list else pair_hints)
+                          neighbor_list_cutoff=neighbor_list_cutoff, pair_tiles=None if half_list else pair_tiles)
     return e, f, es, w

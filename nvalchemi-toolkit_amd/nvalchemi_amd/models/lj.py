@@ -142,13 +142,14 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
         return None
 
     @staticmethod
-    def _pair_hints_of(data, positions: torch.Tensor):
+    def _pair_tiles_of(data, positions: torch.Tensor, neighbor_matrix: torch.Tensor):
         """What the neighbor hook left for the pair kernel of large systems, if it was made from exactly these
-        positions (same storage, no write since)."""
-        hints = getattr(data, "_neighbor_pair_hints", None)
-        if (isinstance(hints, tuple) and len(hints) == 5 and hints[3] == positions.data_ptr()
-                and hints[4] == positions._version):
-            return hints[:3]
+        positions (same storage, no write since) together with exactly this matrix."""
+        tiles = getattr(data, "_neighbor_pair_tiles", None)
+        if (isinstance(tiles, tuple) and len(tiles) == 7 and tiles[4] == positions.data_ptr()
+                and tiles[5] == positions._version and tiles[6] == neighbor_matrix.data_ptr()
+                and tuple(tiles[0].shape) == tuple(neighbor_matrix.shape)):
+            return tiles[:4]
         return None
 
     @staticmethod
@@ -203,7 +204,7 @@ class LennardJonesModelWrapper(nn.Module, BaseModelMixin):
             self.switch_width, self.half_list, compute_virial=compute_stress, out=bufs,
             row_order=self._row_order_of(data, N, positions.device),
             neighbor_list_cutoff=self._search_cutoff_of(data, neighbor_matrix),
-            pair_hints=self._pair_hints_of(data, inp["positions"]))
+            pair_tiles=self._pair_tiles_of(data, inp["positions"], neighbor_matrix))
         if own_energy:
             sys_e = sys_e.clone()  # a fresh tensor for the caller, as in the reference (:482)
         model_output: dict[str, Any] = {"energy": sys_e.unsqueeze(-1), "forces": forces}
