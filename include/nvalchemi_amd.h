@@ -298,7 +298,7 @@ int32_t nvamd_lj_energy_forces_repeat(const float* positions, const float* cells
                                       float* system_energies, void* workspace, size_t workspace_bytes,
                                       void* stream);
 
-/* nvamd_lj_energy_forces_repeat over the tiles of nvamd_nl_build_tiles, for the positions that build read.  No
+/* nvamd_lj_energy_forces_repeat over the tiles of nvamd_nl_build_extras, for the positions that build read.  No
  * counterpart in the reference.  The rows are walked unit by unit of the build's search; a unit's tile (the atoms
  * of its stencil cells, a few hundred) is copied from ordered_positions into LDS with contiguous reads, laid out
  * by the unit's record, and each listed pair finds its neighbor there through its 16-bit tile_index: no gather from
@@ -414,10 +414,11 @@ int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const
                             const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
                             int32_t* atom_order, void* stream);
 
-/* nvamd_nl_build_path that also leaves behind what a pair kernel needs to walk the search's own tiles again
- * (nvamd_lj_energy_forces_tiles).  No counterpart in the reference.  The search handles the atoms of a run of
- * cells (a "unit") against one tile: the atoms of the run's stencil cells, staged in LDS in a fixed order.  Beyond
- * the outputs of nvamd_nl_build_path:
+/* nvamd_nl_build_path (float32 positions) with two extras, each optional.  No counterpart in the reference.
+ *
+ * (1) The four tile outputs (all given or all NULL): what a pair kernel needs to walk the search's own tiles again
+ * (nvamd_lj_energy_forces_tiles).  The search handles the atoms of a run of cells (a "unit") against one tile: the
+ * atoms of the run's stencil cells, staged in LDS in a fixed order.
  *   tile_index (N, max_neighbors) u16    per listed pair, where the neighbor stood in the tile of the row's unit
  *   ordered_positions (N, 4) f32         the atoms in cell order: float32 coordinates as read, and the bits of the
  *                                        atom's index in the fourth word
@@ -426,18 +427,29 @@ int32_t nvamd_nl_atom_order(const void* workspace, size_t workspace_bytes, const
  *                                        or -1: the unit's stencil is not one tile], then per stencil cell
  *                                        [its first slot of the cell order, its offset in the tile]
  *   tile_count (1) i32                   units of this build
- * Float32 positions, full list, every system built (no rebuild_flags), max_neighbors a multiple of 8.  A tile holds
- * at most NVAMD_NL_TILE_ATOMS atoms.  Valid for the positions of this build only. */
+ * Full list, every system built (no rebuild_flags), max_neighbors a multiple of 8.  A tile holds at most
+ * NVAMD_NL_TILE_ATOMS atoms.  Valid for the positions of this build only.
+ *
+ * (2) shift_groups (N) u32 or NULL: lets the build skip the stores of shifts that are zero over zeros.  Most listed
+ * pairs of a system larger than a few cutoffs have a zero shift, and three quarters of what a build writes are
+ * shifts.  Bit g of an atom's word says that slots [g << s, (g + 1) << s) of its row of neighbor_matrix_shifts may
+ * hold a shift that is not zero, s the smallest number with (max_neighbors - 1) >> s < 32; the build writes a
+ * pair's shift if it is not zero or if its slot's bit was set, and leaves the word for the next build.  The
+ * contents of neighbor_matrix_shifts come out exactly as without it.  The contract is tail_mode 0's, extended to
+ * the shifts: neighbor_matrix_shifts was zeroed once together with shift_groups and is written by this function
+ * only, always with the same shift_groups and max_neighbors (after anything else has written it, or after
+ * max_neighbors has changed, set every word to 0xffffffff once).  tail_mode must be 0. */
 #define NVAMD_NL_TILE_RECORD_INTS 132
 #define NVAMD_NL_TILE_ATOMS 1088
 int32_t nvamd_nl_tile_records(int32_t n_atoms, int32_t n_systems, size_t* records);
-int32_t nvamd_nl_build_tiles(const float* positions, const float* cell, const uint8_t* pbc,
-                             const int32_t* batch_ptr, const int32_t* batch_idx, int32_t n_atoms,
-                             int32_t n_systems, double cutoff, int32_t max_neighbors, int32_t tail_mode,
-                             int32_t sort_path, int32_t* neighbor_matrix, int32_t* num_neighbors,
-                             int32_t* neighbor_matrix_shifts, uint16_t* tile_index, float* ordered_positions,
-                             int32_t* tile_records, int32_t* tile_count, void* workspace, size_t workspace_bytes,
-                             void* stream);
+int32_t nvamd_nl_build_extras(const float* positions, const float* cell, const uint8_t* pbc,
+                              const int32_t* batch_ptr, const int32_t* batch_idx,
+                              const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                              double cutoff, int32_t max_neighbors, int32_t half_fill, int32_t tail_mode,
+                              int32_t sort_path, int32_t* neighbor_matrix, int32_t* num_neighbors,
+                              int32_t* neighbor_matrix_shifts, uint16_t* tile_index, float* ordered_positions,
+                              int32_t* tile_records, int32_t* tile_count, uint32_t* shift_groups, void* workspace,
+                              size_t workspace_bytes, void* stream);
 
 /* Per-system reductions of a per-atom float32 vector: replace the Warp launches behind
  * nvalchemi_hooks::segmented_sum / _max / _min / _mean (nvalchemi/dynamics/hooks/_utils.py:58-136;

@@ -185,6 +185,11 @@ struct NlArgs {
     int2* tile_records;    // (max cells, kTileRecord) per unit: (first row, rows), (system, atoms in the tile or -1),
                            // then per stencil cell (first slot of the cell order, offset in the tile)
     int32_t* tile_count;   // (1) units of this build
+    // Shifts written only where they have to be (null: every listed pair's shift is written).  Bit g of a row's
+    // word says that slots [g << group_shift, (g + 1) << group_shift) of the row may hold a shift that is not zero;
+    // everywhere else the shifts in memory are zero and a zero shift need not be written again.
+    uint32_t* shift_groups;  // (N)
+    int group_shift;
     double rc, rc2, rcb;
     int32_t* nm;
     int32_t* nn;
@@ -833,7 +838,7 @@ __device__ __forceinline__ void candidate_shift(const ShiftSource& src, int k, i
 // candidates a centre cell of the run has to look at are one contiguous range of the LDS tile;
 // what a range picks up beyond its own layers (ranges are widened to multiples of 64) lies
 // further than the stencil radius away and can never pass the distance test.
-template <bool HALF, bool F64, bool TILES>
+template <bool HALF, bool F64, bool TILES, bool SPARSE>
 // The tables that every lane of a workgroup reads at the same address (unit records, the per-system
 // constants, the run's cell ranges) come in as read-only arguments of their own besides the workspace:
 // nothing in the kernel can be seen to write them, so they are fetched through the scalar cache, which
@@ -1112,6 +1117,11 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                         int base = __builtin_amdgcn_readfirstlane(meta.w);  // found before this tile
                         int32_t* row = a.nm + (size_t)i_atom * a.K;
                         int32_t* srow = a.shifts ? a.shifts + (size_t)i_atom * a.K * 3 : nullptr;
+                        // which groups of the row's slots may hold a shift that is not zero (rows that are not finished
+                        // in one piece write every shift and come out as dirty all over); asked for here, used at the
+                        // first write of the row
+                        const unsigned was_dirty = (SPARSE && fused && a.shifts) ? a.shift_groups[i_atom] : 0xffffffffu;
+                        unsigned now_dirty = 0;                             // (the same in every lane)
                         int nh = 0;                                         // entries in the hit list
                         unsigned short* my_hits = hits[wave];
 
@@ -1180,10 +1190,23 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                 const unsigned long long m = __builtin_amdgcn_ballot_w64(in);
                                 const int slot = base + __builtin_amdgcn_mbcnt_hi((unsigned)(m >> 32),
                                                                                   __builtin_amdgcn_mbcnt_lo((unsigned)m, 0));
+                                bool store_shift = srow != nullptr;
+                                if (SPARSE && m != 0) {
+                                    // These entries go to slots [base, base + n): their shifts are left unwritten if all
+                                    // of them are zero and the groups they fall into held nothing but zeros; one
+                                    // decision for the whole step, taken on scalar registers.
+                                    const int s_hi = base + __popcll(m) - 1;
+                                    const int g_lo = (base < a.K - 1 ? base : a.K - 1) >> a.group_shift;
+                                    const int g_hi = (s_hi < a.K - 1 ? s_hi : a.K - 1) >> a.group_shift;
+                                    const unsigned groups = (2u << g_hi) - (1u << g_lo);
+                                    const bool any_shift = __builtin_amdgcn_ballot_w64(in && (s0 | s1 | s2) != 0) != 0;
+                                    if (any_shift) now_dirty |= groups;
+                                    store_shift = store_shift && (any_shift || (was_dirty & groups) != 0);
+                                }
                                 if (in && slot < a.K) {
                                     row[slot] = j;
                                     if (TILES) a.tile_index[(size_t)i_atom * a.K + slot] = (uint16_t)k;
-                                    if (srow) {
+                                    if (store_shift) {
                                         srow[3 * slot + 0] = s0;
                                         srow[3 * slot + 1] = s1;
                                         srow[3 * slot + 2] = s2;
@@ -1226,7 +1249,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             // ---- count, and padding over what the previous build left beyond it
                             for (int k = base + lane; k < hi_slot; k += kWave) {
                                 row[k] = a.n_atoms;
-                                if (srow) {
+                                if (srow && (!SPARSE || ((was_dirty >> (k >> a.group_shift)) & 1u))) {
                                     srow[3 * k + 0] = 0;
                                     srow[3 * k + 1] = 0;
                                     srow[3 * k + 2] = 0;
@@ -1234,6 +1257,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             }
                             if (lane == 0) {
                                 a.nn[i_atom] = base;
+                                if (SPARSE && srow) a.shift_groups[i_atom] = now_dirty;
                                 if (base > a.K) atomicOr(&ws.hdr->error, NVAMD_NL_STATUS_ROW_OVERFLOW);
                             }
                         } else if (lane == 0) {
@@ -1263,6 +1287,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                     }
                     if (lane == 0) {
                         a.nn[i_atom] = cnt;
+                        if (SPARSE && srow) a.shift_groups[i_atom] = 0xffffffffu;
                         if (cnt > a.K) atomicOr(&ws.hdr->error, NVAMD_NL_STATUS_ROW_OVERFLOW);
                     }
                 }
@@ -1355,7 +1380,7 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
                              int32_t* neighbor_matrix, int32_t* num_neighbors, int32_t* neighbor_matrix_shifts,
                              void* workspace, size_t workspace_bytes, void* stream, uint16_t* tile_index = nullptr,
                              float* ordered_positions = nullptr, int32_t* tile_records = nullptr,
-                             int32_t* tile_count = nullptr) {
+                             int32_t* tile_count = nullptr, uint32_t* shift_groups = nullptr) {
     if (sort_path != NVAMD_NL_SORT_AUTO && sort_path != NVAMD_NL_SORT_PER_SYSTEM && sort_path != NVAMD_NL_SORT_GLOBAL)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: unknown sort_path %d", (int)sort_path);
     if (n_atoms < 0 || n_systems < 0 || max_neighbors < 0)
@@ -1375,6 +1400,9 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
         return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "nl: workspace %zu < %zu bytes", workspace_bytes, need);
     if (max_cells_for(n_atoms, n_systems) > 0x7fffffffull)
         return fail(NVAMD_ERR_UNSUPPORTED, "nl: too many cells");
+    if (shift_groups && (!positions || tail_mode))
+        return fail(NVAMD_ERR_UNSUPPORTED,
+                    "nl: shift_groups go with float32 positions and tail_mode 0 (buffers that only this function writes)");
     if (tile_index) {
         if (!ordered_positions || !tile_records || !tile_count)
             return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: the tile outputs come together");
@@ -1408,6 +1436,10 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     a.tile_xyz = reinterpret_cast<float4*>(ordered_positions);
     a.tile_records = reinterpret_cast<int2*>(tile_records);
     a.tile_count = tile_count;
+    // (no shifts, nothing to keep track of)
+    a.shift_groups = neighbor_matrix_shifts ? shift_groups : nullptr;
+    a.group_shift = 0;
+    while ((max_neighbors - 1) >> a.group_shift > 31) ++a.group_shift;
     a.rc = cutoff;
     a.rc2 = cutoff * cutoff;
     a.rcb = cutoff * (1.0 + 1.0 / 1024.0);
@@ -1439,17 +1471,20 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     unsigned n_search = 8u * 2048u;
     size_t cells_bound = max_cells_for(n_atoms, n_systems);
     if (cells_bound < n_search) n_search = (unsigned)((cells_bound + 7) / 8 * 8);
-#define NVAMD_NL_SEARCH(H, D) \
-    hipLaunchKernelGGL((nl_search_kernel<H, D, false>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start)
+#define NVAMD_NL_SEARCH(H, D, T, S) \
+    hipLaunchKernelGGL((nl_search_kernel<H, D, T, S>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys, ws.cell_start)
     if (a.tile_index) {
-        hipLaunchKernelGGL((nl_search_kernel<false, false, true>), dim3(n_search), blk, 0, st, a, ws, ws.units, ws.ssys,
-                           ws.cell_start);
+        if (a.shift_groups) NVAMD_NL_SEARCH(false, false, true, true);
+        else NVAMD_NL_SEARCH(false, false, true, false);
+    } else if (a.shift_groups) {
+        if (a.half) NVAMD_NL_SEARCH(true, false, false, true);
+        else NVAMD_NL_SEARCH(false, false, false, true);
     } else if (a.pos64) {
-        if (a.half) NVAMD_NL_SEARCH(true, true);
-        else NVAMD_NL_SEARCH(false, true);
+        if (a.half) NVAMD_NL_SEARCH(true, true, false, false);
+        else NVAMD_NL_SEARCH(false, true, false, false);
     } else {
-        if (a.half) NVAMD_NL_SEARCH(true, false);
-        else NVAMD_NL_SEARCH(false, false);
+        if (a.half) NVAMD_NL_SEARCH(true, false, false, false);
+        else NVAMD_NL_SEARCH(false, false, false, false);
     }
 #undef NVAMD_NL_SEARCH
     NVAMD_LAUNCH_CHECK("neighbor list launch");
@@ -1468,18 +1503,21 @@ NVAMD_EXPORT int32_t nvamd_nl_build_path(const float* positions, const float* ce
                          neighbor_matrix_shifts, workspace, workspace_bytes, stream);
 }
 
-NVAMD_EXPORT int32_t nvamd_nl_build_tiles(const float* positions, const float* cell, const uint8_t* pbc,
-                                          const int32_t* batch_ptr, const int32_t* batch_idx, int32_t n_atoms,
-                                          int32_t n_systems, double cutoff, int32_t max_neighbors, int32_t tail_mode,
-                                          int32_t sort_path, int32_t* neighbor_matrix, int32_t* num_neighbors,
-                                          int32_t* neighbor_matrix_shifts, uint16_t* tile_index, float* ordered_positions,
-                                          int32_t* tile_records, int32_t* tile_count, void* workspace,
-                                          size_t workspace_bytes, void* stream) {
-    if (n_atoms > 0 && n_systems > 0 && (!tile_index || !ordered_positions || !tile_records || !tile_count))
-        return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl tiles: null buffer");
-    return nl_build_impl(positions, cell, nullptr, nullptr, pbc, batch_ptr, batch_idx, nullptr, n_atoms, n_systems, cutoff,
-                         max_neighbors, 0, tail_mode, sort_path, neighbor_matrix, num_neighbors, neighbor_matrix_shifts,
-                         workspace, workspace_bytes, stream, tile_index, ordered_positions, tile_records, tile_count);
+NVAMD_EXPORT int32_t nvamd_nl_build_extras(const float* positions, const float* cell, const uint8_t* pbc,
+                                           const int32_t* batch_ptr, const int32_t* batch_idx,
+                                           const uint8_t* rebuild_flags, int32_t n_atoms, int32_t n_systems,
+                                           double cutoff, int32_t max_neighbors, int32_t half_fill, int32_t tail_mode,
+                                           int32_t sort_path, int32_t* neighbor_matrix, int32_t* num_neighbors,
+                                           int32_t* neighbor_matrix_shifts, uint16_t* tile_index,
+                                           float* ordered_positions, int32_t* tile_records, int32_t* tile_count,
+                                           uint32_t* shift_groups, void* workspace, size_t workspace_bytes,
+                                           void* stream) {
+    const int given = (tile_index ? 1 : 0) + (ordered_positions ? 1 : 0) + (tile_records ? 1 : 0) + (tile_count ? 1 : 0);
+    if (given != 0 && given != 4) return fail(NVAMD_ERR_INVALID_ARGUMENT, "nl: the four tile outputs come together");
+    return nl_build_impl(positions, cell, nullptr, nullptr, pbc, batch_ptr, batch_idx, rebuild_flags, n_atoms, n_systems,
+                         cutoff, max_neighbors, half_fill, tail_mode, sort_path, neighbor_matrix, num_neighbors,
+                         neighbor_matrix_shifts, workspace, workspace_bytes, stream, tile_index, ordered_positions,
+                         tile_records, tile_count, shift_groups);
 }
 
 NVAMD_EXPORT int32_t nvamd_nl_tile_records(int32_t n_atoms, int32_t n_systems, size_t* records) {

@@ -57,7 +57,7 @@ _SIGNATURES = {
     "nvamd_lj_energy_forces_hinted": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_repeat": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_tiles": (_i32, [_vp] * 11 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 3 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
-    "nvamd_nl_build_tiles": (_i32, [_vp] * 5 + [_i32, _i32, _c.c_double, _i32, _i32, _i32] + [_vp] * 8 + [_c.c_size_t, _vp]),
+    "nvamd_nl_build_extras": (_i32, [_vp] * 6 + [_i32, _i32, _c.c_double, _i32, _i32, _i32, _i32] + [_vp] * 9 + [_c.c_size_t, _vp]),
     "nvamd_nl_tile_records": (_i32, [_i32, _i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_lj_energy_forces_static": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_vp] * 5),
     "nvamd_nl_atom_order": (_i32, [_vp, _c.c_size_t, _vp, _vp, _i32, _i32, _vp, _vp]),
@@ -242,10 +242,14 @@ nl_sort_path = NL_SORT_AUTO
 
 def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, max_neighbors,
              half_fill, tail_mode, neighbor_matrix, num_neighbors, neighbor_matrix_shifts,
-             workspace: torch.Tensor | None = None, sort_path: int | None = None, pair_tiles=None) -> None:
+             workspace: torch.Tensor | None = None, sort_path: int | None = None, pair_tiles=None,
+             shift_groups=None) -> None:
     """``pair_tiles``: ``(tile_index (N,K) i16, ordered_positions (N,4) f32, tile_records (R, NL_TILE_RECORD_INTS) i32,
     tile_count (1) i32)``, R = ``nl_tile_records(N, B)``: also leave behind what the pair kernel of large systems
-    walks (float32 positions, full list, every system built, K a multiple of 8)."""
+    walks (float32 positions, full list, every system built, K a multiple of 8).  ``shift_groups`` (N) i32: per
+    row, which groups of slots of ``neighbor_matrix_shifts`` may hold a shift that is not zero; with it the build
+    does not write zeros over zeros (float32 positions, ``tail_mode`` 0, buffers that only this function writes and
+    that were zeroed together with it)."""
     lib = library()
     if sort_path is None:
         sort_path = nl_sort_path
@@ -267,16 +271,21 @@ def nl_build(positions, cell, pbc, batch_ptr, batch_idx, rebuild_flags, cutoff, 
     ws = workspace if workspace is not None else workspaces.get(positions.device, "nl", need)
     if ws.device != positions.device or ws.numel() * ws.element_size() < need:
         raise ValueError("neighbor-list workspace too small or on another device")
-    if pair_tiles is not None:
-        if real != torch.float32 or half_fill or rebuild_flags is not None:
-            raise ValueError("pair tiles need float32 positions, a full list and a build of every system")
-        index, ordered, records, count = pair_tiles
-        _check(lib.nvamd_nl_build_tiles(
-            p_pos, p_cell, p_pbc, p_ptr, p_idx, N, B, float(cutoff), K, int(tail_mode), int(sort_path), p_nm, p_nn, p_sh,
-            _dev(index, "tile_index", torch.int16, (N, K)), _dev(ordered, "ordered_positions", torch.float32, (N, 4)),
-            _dev(records, "tile_records", torch.int32, (nl_tile_records(N, B), NL_TILE_RECORD_INTS)),
-            _dev(count, "tile_count", torch.int32, (1,)),
-            ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)), "nvamd_nl_build_tiles")
+    if pair_tiles is not None or shift_groups is not None:
+        if real != torch.float32:
+            raise ValueError("pair tiles and shift groups need float32 positions")
+        if pair_tiles is not None and (half_fill or rebuild_flags is not None):
+            raise ValueError("pair tiles need a full list and a build of every system")
+        if shift_groups is not None and tail_mode:
+            raise ValueError("shift groups go with tail_mode 0")
+        index, ordered, records, count = pair_tiles if pair_tiles is not None else (None,) * 4
+        _check(lib.nvamd_nl_build_extras(
+            p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K, int(bool(half_fill)), int(tail_mode),
+            int(sort_path), p_nm, p_nn, p_sh,
+            _opt(index, "tile_index", torch.int16, (N, K)), _opt(ordered, "ordered_positions", torch.float32, (N, 4)),
+            _opt(records, "tile_records", torch.int32, (nl_tile_records(N, B), NL_TILE_RECORD_INTS)),
+            _opt(count, "tile_count", torch.int32, (1,)), _opt(shift_groups, "shift_groups", torch.int32, (N,)),
+            ws.data_ptr(), ws.numel() * ws.element_size(), _stream(positions.device)), "nvamd_nl_build_extras")
         return
     entry = lib.nvamd_nl_build_f64 if real == torch.float64 else lib.nvamd_nl_build_path
     _check(entry(p_pos, p_cell, p_pbc, p_ptr, p_idx, p_flags, N, B, float(cutoff), K,

@@ -62,7 +62,7 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
                   num_neighbors: torch.Tensor | None = None,
                   neighbor_matrix_shifts: torch.Tensor | None = None,
                   rebuild_flags: torch.Tensor | None = None, method: str | None = None,
-                  tail_mode: int = 1, pair_tiles: tuple | None = None,
+                  tail_mode: int = 1, pair_tiles: tuple | None = None, shift_groups: torch.Tensor | None = None,
                   **scratch) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
     """Build the dense neighbor list in place and return ``(neighbor_matrix, num_neighbors,
     neighbor_matrix_shifts)``.
@@ -76,7 +76,8 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
     ignored.  ``tail_mode=1`` rewrites the padding of every rebuilt row; ``0`` only clears
     what the previous build left (persistent buffers that only this function writes).
     ``pair_tiles`` (not in the reference): four preallocated tensors in which the build also leaves what the
-    pair kernel of large systems walks, see ``_lib.nl_build``.
+    pair kernel of large systems walks, see ``_lib.nl_build``.  ``shift_groups`` (not in the reference): the
+    record that lets a build on persistent buffers skip the stores of zero shifts over zeros, see ``_lib.nl_build``.
     """
     if method not in _METHODS:
         raise ValueError(f"unknown neighbor list method {method!r}")
@@ -110,7 +111,7 @@ def neighbor_list(positions: torch.Tensor, cutoff: float, cell: torch.Tensor | N
     _lib.nl_build(positions.contiguous(), cell, pbc, batch_ptr.to(torch.int32).contiguous(),
                   batch_idx.to(torch.int32).contiguous(), rebuild_flags, cutoff, K, half_fill, tail_mode,
                   neighbor_matrix, num_neighbors, neighbor_matrix_shifts if cell is not None else None,
-                  pair_tiles=pair_tiles)
+                  pair_tiles=pair_tiles, shift_groups=shift_groups if cell is not None else None)
     return neighbor_matrix, num_neighbors, neighbor_matrix_shifts
 
 
