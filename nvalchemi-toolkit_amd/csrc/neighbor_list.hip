@@ -1204,12 +1204,14 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                                     store_shift = store_shift && (any_shift || (was_dirty & groups) != 0);
                                 }
                                 if (in && slot < a.K) {
-                                    row[slot] = j;
-                                    if (TILES) a.tile_index[(size_t)i_atom * a.K + slot] = (uint16_t)k;
+                                    // (the rows are written past the caches' retention, like the shifts below: what the
+                                    // search re-reads, the sorted atoms of neighboring units, keeps its place in L2)
+                                    __builtin_nontemporal_store(j, &row[slot]);
+                                    if (TILES) __builtin_nontemporal_store((uint16_t)k, &a.tile_index[(size_t)i_atom * a.K + slot]);
                                     if (store_shift) {
-                                        srow[3 * slot + 0] = s0;
-                                        srow[3 * slot + 1] = s1;
-                                        srow[3 * slot + 2] = s2;
+                                        __builtin_nontemporal_store(s0, &srow[3 * slot + 0]);
+                                        __builtin_nontemporal_store(s1, &srow[3 * slot + 1]);
+                                        __builtin_nontemporal_store(s2, &srow[3 * slot + 2]);
                                     }
                                 }
                                 base += __popcll(m);
