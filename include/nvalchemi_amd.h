@@ -64,6 +64,11 @@ const char* nvamd_last_error(void);
  *                        num_neighbors must hold the previous counts (zeros at first use).
  *   neighbor_matrix_shifts may be NULL when cell is NULL.
  * ---------------------------------------------------------------------------------------- */
+/* The workspace: device memory of at least this many bytes whose first 256 bytes (the header) are ZERO when it is
+ * first used (hipMemsetAsync of 256 bytes, once).  The header keeps the unit counter and the status bits of a build
+ * in one of two slots, taken in turn, and every build clears the slot of the build before it (no reset launch), so
+ * builds through one workspace must not overlap; apart from the header nothing in it outlives a call except what
+ * nvamd_nl_atom_order and nvamd_nl_status read. */
 int32_t nvamd_nl_workspace_bytes(int32_t n_atoms, int32_t n_systems, size_t* bytes);
 
 int32_t nvamd_nl_build(const float* positions, const float* cell, const uint8_t* pbc,
@@ -395,8 +400,7 @@ int32_t nvamd_wrap_positions_f64(double* positions, const double* cell, const ui
  * kernels report nothing (a caller there compares num_neighbors with max_neighbors on the host:
  * nvalchemi/neighbors.py:269-273, nvalchemi/hooks/neighbor_list.py:446-469).
  * status (2) i32 on the device: status[0] = bits of the last build, status[1] = bits of every build since the
- *   bits were last cleared (the header of a workspace that has never held a build must be zero for status[1]
- *   to mean anything).  clear != 0 clears both words after they are read.  No host synchronisation.
+ *   bits were last cleared.  clear != 0 clears both words after they are read.  No host synchronisation.
  * NVAMD_NL_STATUS_CELL_TOO_THIN: some periodic cell is singular or thinner than cutoff / 32 along an axis; the
  *   search looks at 32 images per axis and direction at most, so that system's list is truncated.
  * NVAMD_NL_STATUS_ROW_OVERFLOW: some atom has more than max_neighbors neighbors (its count says how many; the

@@ -106,12 +106,29 @@ static_assert(sizeof(NlUnit) == 32, "read as two 16-byte words");
 static_assert(kMaxStencilRadius < 64, "stencil radii are packed 6 bits each");
 
 struct NlHeader {
+    // The unit counter and the flags of a build live in one of two slots, taken in turn (flip), so that no build
+    // needs a launch that resets them: the kernels that sort (which run before any other kernel of a build reads
+    // the slot in hand) clear the other slot, the one of the build before, after moving its flags to `sticky`; the
+    // search kernel reads the sum of both counters (the other one is zero by then) and its first workgroup turns
+    // flip over for the next build (nobody else reads flip while the search runs).  A new workspace starts with a
+    // zeroed header.
     int total_cells;
-    int error;   // of the build in hand: NVAMD_NL_STATUS_* bits
-    int total_units;
-    int sticky;  // the bits of all earlier builds through this workspace since they were last cleared
-    int pad[12];
+    int flip;       // the slot of the next build (of the build in hand, until its search kernel runs)
+    int units[2];   // search units of the build that used the slot
+    int error[2];   // its NVAMD_NL_STATUS_* bits
+    int sticky;     // the bits of all builds before the last one since they were last cleared
+    int pad[9];
 };
+static_assert(sizeof(NlHeader) == 64, "inside the 256 bytes that a new workspace starts with as zeros");
+
+// First thing in a build, by one thread of a kernel that runs before the build's counters are read by anyone else:
+// the slot of the build before is folded away and cleared.
+__device__ __forceinline__ void retire_other_slot(NlHeader* hdr) {
+    const int other = hdr->flip ^ 1;
+    hdr->sticky |= hdr->error[other];
+    hdr->error[other] = 0;
+    hdr->units[other] = 0;
+}
 
 struct NlWorkspace {
     NlHeader* hdr;
@@ -255,10 +272,7 @@ __device__ __forceinline__ void system_setup(NlSys& s, const NlArgs& a, int t) {
 __global__ __launch_bounds__(kBlock) void nl_prepare_kernel(NlArgs a, NlWorkspace ws) {
     int t = blockIdx.x * kBlock + threadIdx.x;
     if (t < ws.max_cells) ws.cell_count[t] = 0;
-    if (t == 0) {
-        ws.hdr->sticky |= ws.hdr->error;
-        ws.hdr->error = 0;
-    }
+    if (t == 0) retire_other_slot(ws.hdr);
     if (t >= a.n_systems) return;
     NlSys s;
     system_setup(s, a, t);
@@ -419,7 +433,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
         int ncell = 0, nunit = 0;
         if (t < a.n_systems) {
             NlSys s = ws.sys[t];
-            choose_grid(s, a, ws.bounds + 6 * (size_t)t, &ws.hdr->error);
+            choose_grid(s, a, ws.bounds + 6 * (size_t)t, &ws.hdr->error[ws.hdr->flip]);
             ncell = s.n_cells;
             nunit = s.n_units;
             ws.sys[t] = s;
@@ -453,7 +467,7 @@ __global__ __launch_bounds__(1024) void nl_grid_kernel(NlArgs a, NlWorkspace ws)
         ws.cell_offset[a.n_systems] = (int)(unsigned)(tot & 0xffffffffull);
         ws.unit_offset[a.n_systems] = (int)(unsigned)(tot >> 32);
         ws.hdr->total_cells = (int)(unsigned)(tot & 0xffffffffull);
-        ws.hdr->total_units = (int)(unsigned)(tot >> 32);
+        ws.hdr->units[ws.hdr->flip] = (int)(unsigned)(tot >> 32);
     }
 }
 
@@ -513,7 +527,7 @@ __device__ __forceinline__ NlUnit make_unit(const NlSearchSys& q, int lu, int ru
 // Launched over max(atoms, cell bound) threads: thread t bins atom t and describes search unit t.
 __global__ __launch_bounds__(kBlock) void nl_bin_kernel(NlArgs a, NlWorkspace ws) {
     int i = blockIdx.x * kBlock + threadIdx.x;
-    if (i < ws.hdr->total_units) {
+    if (i < ws.hdr->units[ws.hdr->flip]) {
         // the system that owns unit i: the last one whose first unit is <= i
         int lo = 0, hi = a.n_systems;
         while (hi - lo > 1) {
@@ -588,6 +602,9 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
     __shared__ int s_part[kSortBlock / kWave];
     const int t = blockIdx.x;
     const int tid = threadIdx.x;
+    // (which slot of the header this build counts in: asked for now, used when the units are reserved)
+    const int slot = __builtin_amdgcn_readfirstlane(ws.hdr->flip);
+    if (t == 0 && tid == 0) retire_other_slot(ws.hdr);
     const int begin = a.ptr[t], end = a.ptr[t + 1];
     // up to kKeep atoms per thread stay in registers from here to the scatter; their positions
     // are requested now, so that they arrive while thread 0 works out the system's grid
@@ -638,7 +655,7 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         s_sys.error = s_err;
         s_sys.cell_offset = cell_base;
         ws.cell_offset[t] = cell_base;
-        if (s_err) atomicOr(&ws.hdr->error, s_err);
+        if (s_err) atomicOr(&ws.hdr->error[slot], s_err);
     }
     __syncthreads();
     {
@@ -753,7 +770,7 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
         const int before = block_exclusive_scan(mine_units, s_part, &total);
         // a contiguous piece of the unit list, wherever the counter stands (the order of the
         // systems in the list is of no consequence)
-        if (tid == 0) s_unit0 = total > 0 ? atomicAdd(&ws.hdr->total_units, total) : 0;
+        if (tid == 0) s_unit0 = total > 0 ? atomicAdd(&ws.hdr->units[slot], total) : 0;
         __syncthreads();
         NlUnit* out = ws.units + s_unit0 + before;
         for (int lu = tid; lu < n_runs; lu += kSortBlock) {
@@ -767,14 +784,6 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
             }
         }
     }
-}
-
-// Before nl_system_sort_kernel: the unit counter and the error flag start at zero.
-__global__ void nl_reset_kernel(NlWorkspace ws) {
-    ws.hdr->total_units = 0;
-    ws.hdr->total_cells = 0;  // not used on the per-system path: cell ids are not dense
-    ws.hdr->sticky |= ws.hdr->error;
-    ws.hdr->error = 0;
 }
 
 // ---- 7 search -------------------------------------------------------------------------------
@@ -861,7 +870,9 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
     __shared__ float st_off[kStencilBatch][3];
     __shared__ unsigned short hits[kWavesPerBlock][kHitCap + 2];
 
-    const int total_units = ws.hdr->total_units;
+    // (the counter of the slot that this build did not use is zero: see NlHeader)
+    const int total_units = ws.hdr->units[0] + ws.hdr->units[1];
+    if (blockIdx.x == 0 && threadIdx.x == 0) ws.hdr->flip ^= 1;
     if (TILES && blockIdx.x == 0 && threadIdx.x == 0) *a.tile_count = total_units;
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
@@ -1260,7 +1271,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                             if (lane == 0) {
                                 a.nn[i_atom] = base;
                                 if (SPARSE && srow) a.shift_groups[i_atom] = now_dirty;
-                                if (base > a.K) atomicOr(&ws.hdr->error, NVAMD_NL_STATUS_ROW_OVERFLOW);
+                                if (base > a.K) atomicOr(&ws.hdr->error[ws.hdr->units[1] > 0 ? 1 : 0], NVAMD_NL_STATUS_ROW_OVERFLOW);
                             }
                         } else if (lane == 0) {
                             ca_meta[ca].w = base;
@@ -1290,7 +1301,7 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
                     if (lane == 0) {
                         a.nn[i_atom] = cnt;
                         if (SPARSE && srow) a.shift_groups[i_atom] = 0xffffffffu;
-                        if (cnt > a.K) atomicOr(&ws.hdr->error, NVAMD_NL_STATUS_ROW_OVERFLOW);
+                        if (cnt > a.K) atomicOr(&ws.hdr->error[ws.hdr->units[1] > 0 ? 1 : 0], NVAMD_NL_STATUS_ROW_OVERFLOW);
                     }
                 }
             }
@@ -1300,12 +1311,14 @@ __global__ __launch_bounds__(kBlock, 5) void nl_search_kernel(NlArgs a, NlWorksp
 }
 
 __global__ void nl_status_kernel(NlHeader* hdr, int32_t* out, int clear) {
-    const int now = hdr->error, all = hdr->sticky | now;
+    // (between builds flip names the slot of the next build: the last one used the other)
+    const int now = hdr->error[hdr->flip ^ 1], all = hdr->sticky | hdr->error[0] | hdr->error[1];
     out[0] = now;
     out[1] = all;
     if (clear) {
         hdr->sticky = 0;
-        hdr->error = 0;
+        hdr->error[0] = 0;
+        hdr->error[1] = 0;
     }
 }
 
@@ -1456,7 +1469,6 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
                                                             : (sort_path == NVAMD_NL_SORT_PER_SYSTEM);
     if (per_system) {
         // many small systems: set-up to scatter in one workgroup per system
-        hipLaunchKernelGGL(nl_reset_kernel, dim3(1), dim3(1), 0, st, ws);
         hipLaunchKernelGGL(nl_system_sort_kernel, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
     } else {
         size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
