@@ -997,7 +997,7 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
 }
 
 int lanes_per_row(int K) {
-    if (K <= 192) return 8;
+    if (K <= 384) return 8;  // (rows are much shorter than K on average: twice the longest row of the first build)
     if (K <= 512) return 16;
     return 32;
 }

@@ -4,7 +4,7 @@ nvamd_lj_energy_forces_tiles): systems too large for the pair kernel to stage wh
 What is checked: that the build's extra outputs describe its own search (every listed pair's tile index names
 the listed neighbor; the units' rows are the atoms, once each); that the pair results are those of the entry
 point that gathers neighbors from memory, which the other tests hold against the oracle (bit for bit where
-both sum in the same order: diagonal cells, rows of up to 192 slots; to the float32 bar of 1e-5 relative /
+both sum in the same order: diagonal cells, rows of up to 384 slots; to the float32 bar of 1e-5 relative /
 1e-6 absolute elsewhere), on cubic and triclinic cells, several systems, cells too narrow for derived images,
 systems too dense for one tile; one case directly against the oracle; and the way through the hook and the
 model, including that tiles of other positions are not used.
