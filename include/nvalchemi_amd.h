@@ -182,7 +182,10 @@ int32_t nvamd_vv_velocity_finalize(float* velocities, const float* forces_new,
  *   Only the vanilla branch exists.  uphill_flag is a device array, so the library cannot look
  *   at it without a synchronisation and does not: the caller must pass zeros (the Python
  *   wrapper checks and raises for anything else).  `active` as above.
- *   workspace: nvamd_fire_workspace_bytes(n_systems).
+ *   workspace: nvamd_fire_workspace_bytes(n_systems), all ZERO when it is first used (hipMemsetAsync once): the
+ *   sums live in two slots taken in turn from call to call, each call clears the slot of the next one, so the
+ *   step is two launches (sums, update); calls through one workspace must not overlap and must all have the same
+ *   n_systems (zero it again before a call with another n_systems).
  * ---------------------------------------------------------------------------------------- */
 int32_t nvamd_fire_workspace_bytes(int32_t n_systems, size_t* bytes);
 

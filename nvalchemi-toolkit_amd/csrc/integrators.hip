@@ -171,11 +171,14 @@ __device__ __forceinline__ bool wave_segmented_max(int seg, float& v) {
 // ---- FIRE -----------------------------------------------------------------------------------
 constexpr float kFireVmax = 3.0e38f;
 
+// The sums live in one of two slots, taken in turn from call to call (flip): the kernel that sums into one slot
+// clears the other for the next call, and the update kernel, which reads the sum of both slots (the other one is
+// zero by then), turns flip over.  So no launch is needed to clear the sums; a new workspace starts as zeros.
 struct FireScratch {
-    double* acc;     // (M,3): sum F.v, sum v.v, sum F.F
+    int* flip;       // (1) the slot of this call's sums
+    double* acc;     // (M, 2, 3): per system and slot, sum F.v, sum v.v, sum F.F (a system's place does not depend on M)
     float* alpha0;   // (M) mixing parameter of before the update
     float* dt0;      // (M) time step of before the update (the MD sub-step integrates with it)
-    float* spare;    // (M)
 };
 
 __global__ __launch_bounds__(kBlock) void fire_clear_kernel(double* acc, int n) {
@@ -183,22 +186,35 @@ __global__ __launch_bounds__(kBlock) void fire_clear_kernel(double* acc, int n) 
     if (t < n) acc[t] = 0.0;
 }
 
-// Before the sums.  The accumulators start at zero (or at the caller's sums, compute_reductions = 0), and the
-// mixing parameter and the time step of before the update are set aside: the update kernel's per-atom threads
-// read them there while its per-system threads write the new ones into the caller's arrays.
-__global__ __launch_bounds__(kBlock) void fire_prepare_kernel(const float* __restrict__ alpha,
-                                                              const float* __restrict__ dt,
-                                                              const float* __restrict__ vf,
-                                                              const float* __restrict__ vv,
-                                                              const float* __restrict__ ff, FireScratch ws,
-                                                              int import_sums, int m) {
-    int s = blockIdx.x * kBlock + threadIdx.x;
-    if (s >= m) return;
-    ws.acc[3 * s + 0] = import_sums ? (double)vf[s] : 0.0;
-    ws.acc[3 * s + 1] = import_sums ? (double)vv[s] : 0.0;
-    ws.acc[3 * s + 2] = import_sums ? (double)ff[s] : 0.0;
+// What has to happen before the update besides the sums: the slot of the next call is cleared, and the mixing
+// parameter and the time step of before the update are set aside (the update kernel's per-atom threads read them
+// there while its per-system threads write the new ones into the caller's arrays).  Done for system s by whoever
+// is given it: a thread of the kernel that sums, or of the kernel below.
+__device__ __forceinline__ void fire_set_aside(const FireScratch& ws, int slot, int s, int m,
+                                               const float* __restrict__ alpha, const float* __restrict__ dt) {
+    double* other = ws.acc + 6 * (size_t)s + 3 * (slot ^ 1);
+    other[0] = 0.0;
+    other[1] = 0.0;
+    other[2] = 0.0;
     ws.alpha0[s] = alpha[s];
     ws.dt0[s] = dt[s];
+}
+
+// No kernel sums: the caller's sums (compute_reductions = 0) or zeros (no atoms) go into this call's slot.
+__global__ __launch_bounds__(kBlock) void fire_import_kernel(const float* __restrict__ alpha,
+                                                             const float* __restrict__ dt,
+                                                             const float* __restrict__ vf,
+                                                             const float* __restrict__ vv,
+                                                             const float* __restrict__ ff, FireScratch ws, int m,
+                                                             int import_sums) {
+    int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    const int slot = ws.flip[0];
+    double* mine = ws.acc + 6 * (size_t)s + 3 * slot;
+    mine[0] = import_sums ? (double)vf[s] : 0.0;
+    mine[1] = import_sums ? (double)vv[s] : 0.0;
+    mine[2] = import_sums ? (double)ff[s] : 0.0;
+    fire_set_aside(ws, slot, s, m, alpha, dt);
 }
 
 // A workgroup takes kFireQuad * kBlock atoms, a thread kFireQuad consecutive ones (read as 16-byte words when the
@@ -213,9 +229,22 @@ template <bool VEC>
 __global__ __launch_bounds__(kBlock) void fire_reduce_kernel(const float* __restrict__ vel,
                                                              const float* __restrict__ frc,
                                                              const int32_t* __restrict__ bidx,
-                                                             double* __restrict__ acc, int n_atoms,
-                                                             int chunks_per_block) {
+                                                             double* __restrict__ acc_base, int n_atoms,
+                                                             int chunks_per_block, FireScratch ws, int m,
+                                                             const float* __restrict__ alpha,
+                                                             const float* __restrict__ dt) {
     __shared__ double s_acc[kFireSlots][3];
+    // (FIRE: the sums go into the slot of this call, and the systems are dealt to the threads of the grid for what
+    // else has to happen before the update; FIRE 2.0 passes its own cleared accumulators and no scratch)
+    double* acc = acc_base;
+    int per_system = 3;  // doubles from one system's sums to the next one's
+    if (ws.flip) {
+        const int slot = ws.flip[0];
+        acc = ws.acc + 3 * slot;
+        per_system = 6;
+        for (int s = (int)blockIdx.x * kBlock + (int)threadIdx.x; s < m; s += (int)gridDim.x * kBlock)
+            fire_set_aside(ws, slot, s, m, alpha, dt);
+    }
     // a workgroup takes chunks_per_block consecutive chunks of kFireQuad * kBlock atoms
     const int block_first = (int)blockIdx.x * chunks_per_block * (kFireQuad * kBlock);  // (below n_atoms: the grid is sized so)
     if (threadIdx.x < kFireSlots * 3) (&s_acc[0][0])[threadIdx.x] = 0.0;
@@ -228,9 +257,9 @@ __global__ __launch_bounds__(kBlock) void fire_reduce_kernel(const float* __rest
             atomicAdd(&s_acc[slot][1], v[1]);
             atomicAdd(&s_acc[slot][2], v[2]);
         } else {
-            atomic_add_f64(acc + 3 * (size_t)seg + 0, v[0]);
-            atomic_add_f64(acc + 3 * (size_t)seg + 1, v[1]);
-            atomic_add_f64(acc + 3 * (size_t)seg + 2, v[2]);
+            atomic_add_f64(acc + per_system * (size_t)seg + 0, v[0]);
+            atomic_add_f64(acc + per_system * (size_t)seg + 1, v[1]);
+            atomic_add_f64(acc + per_system * (size_t)seg + 2, v[2]);
         }
     };
     for (int chunk = 0; chunk < chunks_per_block; ++chunk) {
@@ -285,21 +314,24 @@ __global__ __launch_bounds__(kBlock) void fire_reduce_kernel(const float* __rest
     if (threadIdx.x < kFireSlots * 3) {
         // (a slot that no atom touched is still zero and names a system that may not exist)
         const double t = (&s_acc[0][0])[threadIdx.x];
-        if (t != 0.0) atomic_add_f64(acc + 3 * (size_t)seg_lo + threadIdx.x, t);
+        if (t != 0.0) atomic_add_f64(acc + per_system * (size_t)(seg_lo + threadIdx.x / 3) + threadIdx.x % 3, t);
     }
 }
 
 void launch_fire_reduce(const float* velocities, const float* forces, const int32_t* batch_idx, double* acc,
-                        int n_atoms, hipStream_t st) {
+                        int n_atoms, hipStream_t st, FireScratch ws = FireScratch{nullptr, nullptr, nullptr, nullptr},
+                        int m = 0, const float* alpha = nullptr, const float* dt = nullptr) {
     // about three workgroups per compute unit at most: every workgroup ends with atomics on its systems' sums,
     // which for one large system are the same three addresses for all of them
     const int n_chunks = (n_atoms + kFireQuad * kBlock - 1) / (kFireQuad * kBlock);
     const int per = n_chunks > 1024 ? (n_chunks + 767) / 768 : 1;
     const dim3 grid_r((n_chunks + per - 1) / per), blk(kBlock);
     if (aligned16(velocities) && aligned16(forces))
-        hipLaunchKernelGGL(fire_reduce_kernel<true>, grid_r, blk, 0, st, velocities, forces, batch_idx, acc, n_atoms, per);
+        hipLaunchKernelGGL(fire_reduce_kernel<true>, grid_r, blk, 0, st, velocities, forces, batch_idx, acc, n_atoms, per,
+                           ws, m, alpha, dt);
     else
-        hipLaunchKernelGGL(fire_reduce_kernel<false>, grid_r, blk, 0, st, velocities, forces, batch_idx, acc, n_atoms, per);
+        hipLaunchKernelGGL(fire_reduce_kernel<false>, grid_r, blk, 0, st, velocities, forces, batch_idx, acc, n_atoms, per,
+                           ws, m, alpha, dt);
 }
 
 // The update: blocks below n_atom_blocks take one atom per thread, the blocks after them one system per thread.
@@ -318,7 +350,10 @@ __global__ __launch_bounds__(kBlock) void fire_update_kernel(
     if ((int)blockIdx.x >= n_atom_blocks) {
         const int s = ((int)blockIdx.x - n_atom_blocks) * kBlock + (int)threadIdx.x;
         if (s >= m) return;
-        const double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+        // (nobody reads flip in this kernel: the sums are taken from both slots, one of which is zero)
+        if (s == 0) ws.flip[0] ^= 1;
+        const double* sums = ws.acc + 6 * (size_t)s;
+        const double P = sums[0] + sums[3], VV = sums[1] + sums[4], FF = sums[2] + sums[5];
         if (write_reductions) {
             vf[s] = (float)P;
             vv[s] = (float)VV;
@@ -349,7 +384,8 @@ __global__ __launch_bounds__(kBlock) void fire_update_kernel(
     if (i >= n_atoms) return;
     const int s = bidx[i];
     if (active && !active[s]) return;
-    const double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+    const double* sums = ws.acc + 6 * (size_t)s;
+    const double P = sums[0] + sums[3], VV = sums[1] + sums[4], FF = sums[2] + sums[5];
     const float al = ws.alpha0[s], h = ws.dt0[s], ms = maxstep[s], m_i = masses[i];
     float ma = 0.0f, mb = 0.0f;
     if (P >= 0.0) {
@@ -579,7 +615,7 @@ NVAMD_EXPORT int32_t nvamd_vv_velocity_finalize(float* velocities, const float* 
 NVAMD_EXPORT int32_t nvamd_fire_workspace_bytes(int32_t n_systems, size_t* bytes) {
     if (!bytes || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire workspace: bad argument");
     size_t m = (size_t)(n_systems > 0 ? n_systems : 1);
-    *bytes = align_up(m * 3 * sizeof(double)) + 3 * align_up(m * sizeof(float));
+    *bytes = align_up(sizeof(int)) + align_up(2 * m * 3 * sizeof(double)) + 2 * align_up(m * sizeof(float));
     return NVAMD_OK;
 }
 
@@ -608,21 +644,24 @@ NVAMD_EXPORT int32_t nvamd_fire_step(float* positions, float* velocities, const 
     size_t m = (size_t)n_systems;
     char* w = static_cast<char*>(workspace);
     FireScratch ws;
+    ws.flip = reinterpret_cast<int*>(w);
+    w += align_up(sizeof(int));
     ws.acc = reinterpret_cast<double*>(w);
-    w += align_up(m * 3 * sizeof(double));
+    w += align_up(2 * m * 3 * sizeof(double));
     ws.alpha0 = reinterpret_cast<float*>(w);
     w += align_up(m * sizeof(float));
     ws.dt0 = reinterpret_cast<float*>(w);
-    w += align_up(m * sizeof(float));
-    ws.spare = reinterpret_cast<float*>(w);
     hipStream_t st = static_cast<hipStream_t>(stream);
     dim3 blk(kBlock);
     dim3 grid_m((n_systems + kBlock - 1) / kBlock);
-    // three launches: prepare (per system), sums (per four atoms), update (per atom and per system)
-    hipLaunchKernelGGL(fire_prepare_kernel, grid_m, blk, 0, st, alpha, dt, vf, vv, ff, ws, compute_reductions ? 0 : 1,
-                       n_systems);
+    // two launches: the sums (per four atoms; its threads also clear the next call's slot and set alpha and dt
+    // aside), then the update (per atom and per system).  Without atoms to sum over, or with the caller's sums,
+    // a small kernel per system stands in for the first.
     if (compute_reductions && n_atoms > 0) {
-        launch_fire_reduce(velocities, forces, batch_idx, ws.acc, n_atoms, st);
+        launch_fire_reduce(velocities, forces, batch_idx, nullptr, n_atoms, st, ws, n_systems, alpha, dt);
+    } else {
+        hipLaunchKernelGGL(fire_import_kernel, grid_m, blk, 0, st, alpha, dt, vf, vv, ff, ws, n_systems,
+                           compute_reductions ? 0 : 1);
     }
     const int n_atom_blocks = (n_atoms + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(fire_update_kernel, dim3(n_atom_blocks + (n_systems + kBlock - 1) / kBlock), blk, 0, st, positions,

@@ -190,13 +190,12 @@ class _Workspaces:
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < nbytes:
             old = buf
-            buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
-            # The neighbor build keeps status bits in its workspace's header from build to build: a fresh buffer
-            # starts with a zero header, a regrown one takes over the header of the buffer it replaces (so that an
-            # overflow recorded through the smaller buffer is still reported by nvamd_nl_status).
-            if old is None:
-                buf[:256].zero_()
-            else:
+            # Some kernels keep state in their workspace from call to call (the neighbor build its unit counter and
+            # status bits, FIRE the slot its sums are in): a buffer starts as zeros, and a regrown one takes over the
+            # first 256 bytes of the buffer it replaces, where that state lives (so that, e.g., an overflow recorded
+            # through the smaller buffer is still reported by nvamd_nl_status).
+            buf = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+            if old is not None:
                 buf[:256].copy_(old[:256])
             self._bufs[key] = buf
         return buf
@@ -550,7 +549,9 @@ def fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_a
         ws = workspaces.get(positions.device, "f64", _size(lib.nvamd_f64_workspace_bytes, M))
     else:
         entry = lib.nvamd_fire_step
-        ws = workspaces.get(positions.device, "fire", _size(lib.nvamd_fire_workspace_bytes, M))
+        # (the kernels keep the slot of their sums in this workspace from call to call, per system: one buffer per
+        # number of systems, so that no call meets what a call over more systems left behind)
+        ws = workspaces.get(positions.device, f"fire:{M}", _size(lib.nvamd_fire_workspace_bytes, M))
     _check(entry(
         _dev(positions, "positions", f32, (N, 3)), _dev(velocities, "velocities", f32, (N, 3)),
         _dev(forces, "forces", f32, (N, 3)), _dev(masses, "masses", f32, (N,)),
