@@ -14,8 +14,10 @@
 // Per-system energy and virial go through LDS accumulators and one fp64 atomic per workgroup and
 // system.  Pair math is double on the float32 inputs ("internal math is performed in float64",
 // nvalchemi/models/_ops/lj.py:49-50).
+// Systems too large to stage whole take lj_tiles_kernel instead: it walks the units of the neighbor search again
+// and stages each unit's tile, which the build leaves described (nvamd_nl_build_extras).
 // Bound: with the shifts read, HBM; with the shifts derived, the double-precision pair arithmetic
-// (about 70 vector instructions per pair) and the latency of its operands.
+// (about 64 vector instructions per pair) and the latency of its operands.
 #include <mutex>
 
 #include "common.h"

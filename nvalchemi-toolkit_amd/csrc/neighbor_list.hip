@@ -17,6 +17,10 @@
 //               wavefront per centre atom, 64 candidates per step, ballot + prefix-popcount
 //               compaction into a hit list, the list written out into the atom's row
 // (batches of many small systems take 1-6 in one workgroup per system: nl_system_sort_kernel).
+// What the search writes (rows, shifts) goes out with non-temporal stores.  For batches of large systems it can
+// also leave a description of its tiles for the pair kernel and skip the stores of zero shifts over zeros
+// (nvamd_nl_build_extras).  The unit counter and the status bits live in the workspace's header, in two slots taken
+// in turn, so that a build needs no launch to reset them.
 //
 // Which pairs are neighbors is decided in double on the original positions (geom.h).  The search
 // classifies candidates with float32 distances on cell-local coordinates whose rounding error is
