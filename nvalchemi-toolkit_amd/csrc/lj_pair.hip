@@ -564,6 +564,7 @@ struct LjTiles {
     const float4* xyz;       // (N) cell order
     const int2* records;     // (units, kTileRecord)
     const int32_t* count;    // (1)
+    int capacity;            // records that the table has room for
 };
 
 // rows [0, n_rows) of the staged units: row rr belongs to staged unit q with s_row0[q] <= rr < s_row0[q + 1]
@@ -718,7 +719,9 @@ __global__ __launch_bounds__(kBlockFull, VIRIAL ? 4 : 6) void lj_tiles_kernel(
 
     // units are dealt to the 8 XCDs in contiguous eighths (consecutive workgroups go to the XCDs round-robin), so
     // that the slices of the cell order that neighboring tiles share stay in one L2
-    const int total = count_ro[0];
+    // (a count that the table cannot hold is not this build's: nothing past the table is read)
+    const int counted = count_ro[0];
+    const int total = counted < 0 ? 0 : (counted < t.capacity ? counted : t.capacity);
     const int n_groups = (total + kTileUnits - 1) / kTileUnits;
     const int per_xcd = (n_groups + 7) / 8;
     const int xcd = blockIdx.x % 8, slot0 = blockIdx.x / 8, stride = gridDim.x / 8;
@@ -1233,8 +1236,11 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_tiles(const float* positions, const 
             !aligned16(ordered_positions))
             return fail(NVAMD_ERR_UNSUPPORTED, "lj tiles: rows of 16-byte words are needed (max_neighbors a multiple of 8)");
     }
+    size_t capacity = 0;
+    nvamd_nl_tile_records(n_atoms, n_systems, &capacity);
     const LjTiles tiles{tile_index, reinterpret_cast<const float4*>(ordered_positions),
-                        reinterpret_cast<const int2*>(tile_records), tile_count};
+                        reinterpret_cast<const int2*>(tile_records), tile_count,
+                        (int)(capacity < 0x7fffffffull ? capacity : 0x7fffffffull)};
     return lj_energy_forces_impl(positions, cells, neighbor_matrix, neighbor_matrix_shifts, num_neighbors, batch_idx,
                                  row_order, neighbor_list_cutoff, n_atoms, max_neighbors, n_systems, fill_value, epsilon,
                                  sigma, cutoff, /*switch_width=*/0.0, /*half_list=*/0, atomic_energies, forces, virials,
