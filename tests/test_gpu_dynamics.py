@@ -350,6 +350,59 @@ def test_run_replays_captured_steps_bit_equal_to_eager_steps():
         assert torch.equal(graph_batch.num_neighbors, eager_batch.num_neighbors)
 
 
+def test_replayed_steps_of_a_large_system_and_of_fire_equal_eager_ones():
+    """The same for the paths that keep state on the device from call to call: one system of more than 4096 atoms
+    (the build leaves tile records for the pair kernel and skips zero shifts over zeros; its unit counter lives in
+    two header slots taken in turn) under NVE, and FIRE (its sums live in two slots taken in turn) on small boxes."""
+    from nvalchemi_amd.dynamics import FIRE, NVE
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    def run_both(make, n_steps):
+        out = []
+        for replay in (False, True):
+            batch, dyn = make()
+            dyn.graph_replay = replay
+            dyn.run(batch, n_steps=n_steps)
+            torch.cuda.synchronize()
+            assert (getattr(dyn, "_graph_state", None) is not None) == replay
+            if replay:
+                assert dyn._graph_state["graph"] is not None and not dyn._graph_state["failed"]
+            out.append(batch)
+        for name in ("positions", "velocities", "forces"):
+            assert torch.equal(getattr(out[0], name), getattr(out[1], name)), name
+        return out[1]
+
+    # one box of 6000 atoms on a jittered lattice (so that no two atoms start close)
+    n_side = 19
+    L = n_side * 3.4
+    g = np.random.default_rng(7)
+    grid = np.stack(np.meshgrid(*[np.arange(n_side)] * 3, indexing="ij"), -1).reshape(-1, 3)[:6000]
+    P = ((grid + 0.5) * 3.4 + g.normal(0, 0.15, (6000, 3))).astype(np.float32)
+    C = (np.eye(3) * L).astype(np.float32)[None]
+    pb = np.ones((1, 3), dtype=bool)
+    ptr = np.array([0, 6000], dtype=np.int32)
+    V = g.normal(0, 0.02, (6000, 3)).astype(np.float32)
+
+    def big():
+        batch = make_batch(P, np.full(6000, 18, dtype=np.int64), np.full(6000, 39.95, dtype=np.float32), C, pb, ptr, V)
+        model = LennardJonesModelWrapper(epsilon=0.0104, sigma=3.0, cutoff=7.0)
+        return batch, NVE(model, dt=1.0, hooks=model.make_neighbor_hooks())
+
+    batch = run_both(big, 30)
+    assert getattr(batch, "_neighbor_pair_tiles", None) is not None  # (the tile path was the one taken)
+
+    P2, C2, pb2, ptr2 = fcc_boxes(seed=4, n_boxes=3, reps=3, a=3.7, jitter=0.08)
+
+    def relax():
+        n = len(P2)
+        batch = make_batch(P2, np.full(n, 29, dtype=np.int64), np.full(n, 63.546, dtype=np.float32), C2, pb2, ptr2,
+                           np.zeros_like(P2))
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=float((3.6 / np.sqrt(2)) / 2 ** (1 / 6)), cutoff=5.0)
+        return batch, FIRE(model, dt=0.5, hooks=model.make_neighbor_hooks())
+
+    run_both(relax, 40)
+
+
 def test_run_steps_eagerly_when_a_step_needs_the_host():
     """A convergence criterion ends a run from the host: such a dynamics is never captured."""
     from nvalchemi_amd.dynamics import FIRE, ConvergenceHook
