@@ -569,7 +569,7 @@ __global__ __launch_bounds__(kBlock) void nl_scatter_kernel(NlArgs a, NlWorkspac
 // Every system owns the cell ids [atom_begin + 9 s, ... + n_cells] (cells <= max(atoms, 8), plus
 // one end entry), so cell ids need no prefix sum over the systems either.  A system with more
 // cells than the LDS histogram holds is still handled, slowly, through global memory.
-constexpr int kSortBlock = 1024;
+constexpr int kSortBlock = 512;   // (four workgroups per CU: a system's set-up is a chain of dependent steps that others hide)
 constexpr int kSortCells = 8192;         // cells of a system whose histogram fits in LDS
 constexpr int kPerSystemMeanAtoms = 8192;  // the path is taken up to this many atoms per system on average
 
