@@ -55,8 +55,8 @@ RELAX_MAXSTEP = 0.07
 # half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
 # bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
 MEASURED_TRAFFIC_BYTES = {
-    "nl": 1024 * (2 * (32435 + 15217) + (852497 + 75034)),  # search + per-system sort
-    "lj": 1024 * (2 * (167674 + 23) + 15825 + 21),          # pair kernel + conversion of the per-system sums
+    "nl": 1024 * (2 * (32288 + 11792) + (850244 + 58045)),  # search + per-system sort
+    "lj": 1024 * (2 * (167656 + 23) + 15820 + 21),          # pair kernel + conversion of the per-system sums
 }
 
 
