@@ -360,7 +360,9 @@ int32_t nvamd_lj_energy_forces_static(const float* positions, const float* cells
  * double on the float64 positions.  The pair kernel's per-system energy is the sum of the float64 atomic
  * energies.  nvamd_f64_workspace_bytes(n_systems) serves nvamd_fire_step_f64, nvamd_segment_fmax_f64 and
  * nvamd_lj_energy_forces_f64 (which needs it only with virials or system_energies); the neighbor build uses
- * nvamd_nl_workspace_bytes.  Not built for float64: the thermostats, FIRE 2.0.
+ * nvamd_nl_workspace_bytes.  nvamd_fire2_step_f64 also takes nvamd_f64_workspace_bytes(n_systems);
+ * nvamd_nhc_chain_update_f64 takes nvamd_nhc_workspace_bytes(n_systems) like its float32 form.  The Langevin
+ * step draws the same normal deviates for both types (a function of the seed and the atom index, made in double).
  * ---------------------------------------------------------------------------------------- */
 int32_t nvamd_nl_build_f64(const double* positions, const double* cell, const uint8_t* pbc,
                            const int32_t* batch_ptr, const int32_t* batch_idx, const uint8_t* rebuild_flags,
@@ -398,6 +400,25 @@ int32_t nvamd_nl_rebuild_check_f64(double* reference_positions, const double* cu
                                    int32_t update_reference, uint8_t* rebuild_flags, void* stream);
 int32_t nvamd_wrap_positions_f64(double* positions, const double* cell, const uint8_t* pbc,
                                  const int32_t* batch_idx, int32_t n_atoms, int32_t n_systems, void* stream);
+int32_t nvamd_fire2_step_f64(double* positions, double* velocities, const double* forces, const int32_t* batch_idx,
+                             double* alpha, double* dt, int32_t* nsteps_inc, double* vf, double* v_sumsq,
+                             double* f_sumsq, double* max_norm, int32_t delaystep, double dtgrow, double dtshrink,
+                             double alphashrink, double alpha0, double tmax, double tmin, double maxstep,
+                             const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* workspace,
+                             size_t workspace_bytes, void* stream);
+int32_t nvamd_langevin_half_step_f64(double* positions, double* velocities, const double* forces,
+                                     const double* masses, const double* dt, const double* kT,
+                                     const double* friction, uint64_t random_seed, const int32_t* batch_idx,
+                                     const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* stream);
+int32_t nvamd_nhc_chain_update_f64(double* velocities, const double* masses, double* eta, double* eta_dot,
+                                   const double* chain_masses, const double* kT, const double* dt,
+                                   const double* ndof, double* ke2, double* total_scale, const int32_t* batch_idx,
+                                   const uint8_t* active, int32_t compute_ke, int32_t chain_length,
+                                   int32_t yoshida_order, int32_t n_atoms, int32_t n_systems, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+int32_t nvamd_nhc_position_update_f64(double* positions, const double* velocities, const double* dt,
+                                      const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms,
+                                      int32_t n_systems, void* stream);
 
 /* What the neighbor builds through this workspace had to report.  No counterpart in the reference, whose
  * kernels report nothing (a caller there compares num_neighbors with max_neighbors on the host:

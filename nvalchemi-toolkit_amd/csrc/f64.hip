@@ -1,5 +1,6 @@
-// The float64 forms of the hot path's arithmetic kernels for gfx950: velocity Verlet, FIRE, the
-// per-system maximum force and the Lennard-Jones pair kernel.
+// The float64 forms of the hot path's arithmetic kernels for gfx950: velocity Verlet, FIRE, FIRE 2.0, the
+// per-system maximum force and the Lennard-Jones pair kernel.  (The thermostats' float64 forms are
+// instantiations of their own kernels: langevin.hip, nhc.hip; the skin test and the wrap likewise.)
 //
 // The reference's custom ops take float32 or float64 arrays (nvalchemi/dynamics/_ops/_bridge.py
 // `_vec_type` / `_scalar_type`, nvalchemi/dynamics/_ops/fire.py:281-287,
@@ -402,6 +403,131 @@ __global__ __launch_bounds__(kBlock) void lj_f64_finish_kernel(const double* __r
     }
 }
 
+// ---- FIRE 2.0 (nvalchemi/dynamics/_ops/fire.py:467-557; the float32 form is in integrators.hip) ----
+//   P > 0 :  a = 1 - alpha, b = alpha sqrt(VV / FF); count += 1; past delaystep: dt grows, alpha decays
+//   P <= 0:  count = 0; alpha = alpha0; r -= (dt/2) v; v = 0; dt shrinks while it stays >= tmin
+//   v += dt F;  P > 0: v = a v + b F;  dr = dt v, scaled so that the system's largest |dr| stays within maxstep
+struct Fire2Scratch64 {
+    double* acc;                // (M,3): sum F.v, sum v.v, sum F.F
+    double* mix_a;              // (M) factor on the kicked v
+    double* mix_b;              // (M) factor on F
+    double* back;               // (M) length of the step back (0: none)
+    unsigned long long* big;    // (M) largest |dr| of the system, as the bits of a double >= 0 (NaN above all)
+    double* up;                 // (M) P > 0 (1.0 / 0.0)
+};
+
+struct Fire2Params64 {
+    int delaystep;
+    double dtgrow, dtshrink, alphashrink, alpha0, tmax, tmin, maxstep;
+};
+
+__global__ __launch_bounds__(kBlock) void fire2_params_f64_kernel(double* __restrict__ alpha, double* __restrict__ dt,
+                                                                  int32_t* __restrict__ count, double* vf, double* vv,
+                                                                  double* ff, const uint8_t* __restrict__ active,
+                                                                  Fire2Scratch64 ws, Fire2Params64 p, int m) {
+    const int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    const double P = ws.acc[3 * s + 0], VV = ws.acc[3 * s + 1], FF = ws.acc[3 * s + 2];
+    if (vf) vf[s] = P;
+    if (vv) vv[s] = VV;
+    if (ff) ff[s] = FF;
+    double ma = 1.0, mb = 0.0, bk = 0.0, up = 0.0;
+    if (!active || active[s]) {
+        if (P > 0.0) {
+            const double al = alpha[s];
+            up = 1.0;
+            ma = 1.0 - al;
+            mb = (FF > 1e-20) ? al * sqrt(VV / FF) : 0.0;
+            const int c = count[s] + 1;
+            count[s] = c;
+            if (c > p.delaystep) {
+                const double nd = dt[s] * p.dtgrow;
+                dt[s] = nd < p.tmax ? nd : p.tmax;
+                alpha[s] = al * p.alphashrink;
+            }
+        } else {
+            count[s] = 0;
+            alpha[s] = p.alpha0;
+            bk = 0.5 * dt[s];
+            const double nd = dt[s] * p.dtshrink;
+            if (nd >= p.tmin) dt[s] = nd;
+        }
+    }
+    ws.mix_a[s] = ma;
+    ws.mix_b[s] = mb;
+    ws.back[s] = bk;
+    ws.big[s] = 0ull;
+    ws.up[s] = up;
+}
+
+// new velocities (and the step back), and the largest displacement they would give
+__global__ __launch_bounds__(kBlock) void fire2_kick_f64_kernel(double* __restrict__ pos, double* __restrict__ vel,
+                                                                const double* __restrict__ frc,
+                                                                const double* __restrict__ dt,
+                                                                const int32_t* __restrict__ bidx,
+                                                                const uint8_t* __restrict__ active, Fire2Scratch64 ws,
+                                                                int n_atoms) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_atoms) return;
+    const int s = bidx[i];
+    if (active && !active[s]) return;
+    const double h = dt[s], ma = ws.mix_a[s], mb = ws.mix_b[s], bk = ws.back[s];
+    const bool up = ws.up[s] != 0.0;
+    const size_t b = 3 * (size_t)i;
+    double dr[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        const double f = frc[b + a];
+        double v = vel[b + a];
+        if (!up) {
+            const double undo = bk * v;
+            pos[b + a] = pos[b + a] - undo;
+            v = 0.0;
+        }
+        const double kick = h * f;
+        v = v + kick;
+        if (up) {
+            const double va = ma * v, fb = mb * f;
+            v = va + fb;
+        }
+        v = fmin(fmax(v, -kFireVmax64), kFireVmax64);
+        vel[b + a] = v;
+        dr[a] = h * v;
+    }
+    const double top = fmax(fmax(fabs(dr[0]), fabs(dr[1])), fabs(dr[2]));
+    double nrm = 0.0;
+    if (top > 0.0) {
+        const double a0 = dr[0] / top, a1 = dr[1] / top, a2 = dr[2] / top;
+        nrm = top * sqrt((a0 * a0 + a1 * a1) + a2 * a2);
+    }
+    // norms are >= 0 or NaN: their bit patterns order like unsigned integers, the canonical NaN above all
+    const unsigned long long key = (top != top || nrm != nrm) ? 0x7ff8000000000000ull
+                                                              : (unsigned long long)__double_as_longlong(nrm);
+    atomicMax(ws.big + s, key);
+}
+
+__global__ __launch_bounds__(kBlock) void fire2_drift_f64_kernel(double* __restrict__ pos, const double* __restrict__ vel,
+                                                                 const double* __restrict__ dt,
+                                                                 const int32_t* __restrict__ bidx,
+                                                                 const uint8_t* __restrict__ active, Fire2Scratch64 ws,
+                                                                 double maxstep, double* __restrict__ max_norm,
+                                                                 int n_atoms) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_atoms) return;
+    const int s = bidx[i];
+    if (active && !active[s]) return;
+    const double h = dt[s], big = __longlong_as_double((long long)ws.big[s]);
+    const double sc = big > maxstep ? maxstep / big : 1.0;
+    const size_t b = 3 * (size_t)i;
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        double dr = h * vel[b + a];
+        dr = dr * sc;
+        pos[b + a] = pos[b + a] + dr;
+    }
+    if (max_norm && (i == 0 || bidx[i - 1] != s)) max_norm[s] = big;
+}
+
 }  // namespace
 }  // namespace nvamd
 
@@ -424,7 +550,8 @@ NVAMD_EXPORT int32_t nvamd_vv_velocity_finalize_f64(double* velocities, const do
 
 NVAMD_EXPORT int32_t nvamd_f64_workspace_bytes(int32_t n_systems, size_t* bytes) {
     if (!bytes || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "float64 workspace: bad argument");
-    // FIRE: (M,3) sums + three (M) factors; LJ: (M,10) sums; fmax: (M) keys -- the largest of them
+    // FIRE: (M,3) sums + three (M) factors; FIRE 2.0: (M,3) sums + five (M) words; LJ: (M,10) sums; fmax: (M) keys
+    // -- the largest of them
     *bytes = align_up((size_t)(n_systems > 0 ? n_systems : 1) * 10 * sizeof(double));
     return NVAMD_OK;
 }
@@ -561,5 +688,47 @@ NVAMD_EXPORT int32_t nvamd_lj_energy_forces_f64(const double* positions, const d
         hipLaunchKernelGGL(lj_f64_finish_kernel, blocks((size_t)n_systems * 10), blk, 0, st, a.sys_acc, system_energies,
                            virials, n_systems);
     NVAMD_LAUNCH_CHECK("lj (float64) launch");
+    return NVAMD_OK;
+}
+
+NVAMD_EXPORT int32_t nvamd_fire2_step_f64(double* positions, double* velocities, const double* forces,
+                                          const int32_t* batch_idx, double* alpha, double* dt, int32_t* nsteps_inc,
+                                          double* vf, double* v_sumsq, double* f_sumsq, double* max_norm,
+                                          int32_t delaystep, double dtgrow, double dtshrink, double alphashrink,
+                                          double alpha0, double tmax, double tmin, double maxstep,
+                                          const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+    if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2: negative size");
+    if (n_systems == 0) return NVAMD_OK;
+    if (!alpha || !dt || !nsteps_inc) return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2 (float64): null per-system buffer");
+    if (n_atoms > 0 && (!positions || !velocities || !forces || !batch_idx))
+        return fail(NVAMD_ERR_INVALID_ARGUMENT, "fire2 (float64): null per-atom buffer");
+    size_t need = 0;
+    nvamd_f64_workspace_bytes(n_systems, &need);
+    if (!workspace || workspace_bytes < need)
+        return fail(NVAMD_ERR_WORKSPACE_TOO_SMALL, "fire2 (float64): workspace %zu < %zu bytes", workspace_bytes, need);
+    const int M = n_systems;
+    Fire2Scratch64 ws;  // eight of the workspace's ten words per system
+    ws.acc = static_cast<double*>(workspace);
+    ws.mix_a = ws.acc + 3 * (size_t)M;
+    ws.mix_b = ws.mix_a + M;
+    ws.back = ws.mix_b + M;
+    ws.big = reinterpret_cast<unsigned long long*>(ws.back + M);
+    ws.up = ws.back + 2 * (size_t)M;
+    const Fire2Params64 p{delaystep, dtgrow, dtshrink, alphashrink, alpha0, tmax, tmin, maxstep};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 blk(kBlock), gm((M + kBlock - 1) / kBlock), gn((n_atoms + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(fire_clear_f64_kernel, dim3((3 * M + kBlock - 1) / kBlock), blk, 0, st, ws.acc, 3 * M);
+    if (n_atoms > 0)
+        hipLaunchKernelGGL(fire_reduce_f64_kernel, gn, blk, 0, st, velocities, forces, batch_idx, ws.acc, n_atoms);
+    hipLaunchKernelGGL(fire2_params_f64_kernel, gm, blk, 0, st, alpha, dt, nsteps_inc, vf, v_sumsq, f_sumsq, active, ws,
+                       p, M);
+    if (n_atoms > 0) {
+        hipLaunchKernelGGL(fire2_kick_f64_kernel, gn, blk, 0, st, positions, velocities, forces, dt, batch_idx, active,
+                           ws, n_atoms);
+        hipLaunchKernelGGL(fire2_drift_f64_kernel, gn, blk, 0, st, positions, velocities, dt, batch_idx, active, ws,
+                           maxstep, max_norm, n_atoms);
+    }
+    NVAMD_LAUNCH_CHECK("fire2 (float64) launch");
     return NVAMD_OK;
 }

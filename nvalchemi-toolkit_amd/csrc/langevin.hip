@@ -6,7 +6,8 @@
 // B step, nvalchemi::langevin_finalize (:134-170), is the velocity half kick of velocity Verlet
 // (nvamd_vv_velocity_finalize).
 //
-// Per atom, float32 storage, one rounding per operation:
+// Per atom, in the arrays' own type (float32, or float64 through nvamd_langevin_half_step_f64: the reference's
+// op takes both, nvalchemi/dynamics/_ops/_bridge.py), one rounding per operation:
 //   B   v <- v + (F/m) (dt/2)
 //   A   r <- r + v (dt/2)
 //   O   v <- c1 v + c2 xi,   c1 = exp(-gamma dt),  c2 = sqrt((kT/m) (1 - c1^2)),  xi ~ N(0,1)^3
@@ -57,22 +58,23 @@ __device__ __forceinline__ void box_muller(uint32_t a, uint32_t b, double& n0, d
     n1 = radius * sin(angle);
 }
 
+template <typename T>
 __global__ __launch_bounds__(kBlock) void langevin_half_step_kernel(
-    float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
-    const float* __restrict__ masses, const float* __restrict__ dt, const float* __restrict__ kT,
-    const float* __restrict__ friction, uint32_t seed_lo, uint32_t seed_hi, const int32_t* __restrict__ bidx,
+    T* __restrict__ pos, T* __restrict__ vel, const T* __restrict__ frc,
+    const T* __restrict__ masses, const T* __restrict__ dt, const T* __restrict__ kT,
+    const T* __restrict__ friction, uint32_t seed_lo, uint32_t seed_hi, const int32_t* __restrict__ bidx,
     const uint8_t* __restrict__ active, int n_atoms) {
 #pragma clang fp contract(off)
     const int i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n_atoms) return;
     const int s = bidx[i];
     if (active && !active[s]) return;
-    const float m = masses[i];
-    const float h = dt[s];
-    const float hh = 0.5f * h;
+    const T m = masses[i];
+    const T h = dt[s];
+    const T hh = (T)0.5 * h;
     const double c1d = exp(-(double)friction[s] * (double)h);
-    const float c1 = (float)c1d;
-    const float c2 = (float)sqrt(((double)kT[s] / (double)m) * (1.0 - c1d * c1d));
+    const T c1 = (T)c1d;
+    const T c2 = (T)sqrt(((double)kT[s] / (double)m) * (1.0 - c1d * c1d));
     const Philox rnd = philox4x32_10((uint32_t)i, 0u, 0u, 0u, seed_lo, seed_hi);
     double xi[4];
     box_muller(rnd.c[0], rnd.c[1], xi[0], xi[1]);
@@ -80,11 +82,11 @@ __global__ __launch_bounds__(kBlock) void langevin_half_step_kernel(
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
         const size_t e = 3 * (size_t)i + a;
-        float v = vel[e], r = pos[e];
-        const float acc = frc[e] / m;
+        T v = vel[e], r = pos[e];
+        const T acc = frc[e] / m;
         v = v + acc * hh;
         r = r + v * hh;
-        v = c1 * v + c2 * (float)xi[a];
+        v = c1 * v + c2 * (T)xi[a];
         r = r + v * hh;
         vel[e] = v;
         pos[e] = r;
@@ -96,19 +98,40 @@ __global__ __launch_bounds__(kBlock) void langevin_half_step_kernel(
 
 using namespace nvamd;
 
-NVAMD_EXPORT int32_t nvamd_langevin_half_step(float* positions, float* velocities, const float* forces,
-                                              const float* masses, const float* dt, const float* kT,
-                                              const float* friction, uint64_t random_seed,
-                                              const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms,
-                                              int32_t n_systems, void* stream) {
+namespace {
+
+template <typename T>
+int32_t langevin_half_step(T* positions, T* velocities, const T* forces, const T* masses, const T* dt, const T* kT,
+                           const T* friction, uint64_t random_seed, const int32_t* batch_idx, const uint8_t* active,
+                           int32_t n_atoms, int32_t n_systems, void* stream) {
     if (n_atoms < 0 || n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "langevin: negative size");
     if (n_atoms == 0) return NVAMD_OK;
     if (!positions || !velocities || !forces || !masses || !dt || !kT || !friction || !batch_idx)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "langevin: null buffer");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(langevin_half_step_kernel, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
+    hipLaunchKernelGGL(langevin_half_step_kernel<T>, dim3((n_atoms + kBlock - 1) / kBlock), dim3(kBlock), 0, st,
                        positions, velocities, forces, masses, dt, kT, friction, (uint32_t)(random_seed & 0xffffffffu),
                        (uint32_t)(random_seed >> 32), batch_idx, active, n_atoms);
     NVAMD_LAUNCH_CHECK("langevin launch");
     return NVAMD_OK;
+}
+
+}  // namespace
+
+NVAMD_EXPORT int32_t nvamd_langevin_half_step(float* positions, float* velocities, const float* forces,
+                                              const float* masses, const float* dt, const float* kT,
+                                              const float* friction, uint64_t random_seed,
+                                              const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms,
+                                              int32_t n_systems, void* stream) {
+    return langevin_half_step<float>(positions, velocities, forces, masses, dt, kT, friction, random_seed, batch_idx,
+                                     active, n_atoms, n_systems, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_langevin_half_step_f64(double* positions, double* velocities, const double* forces,
+                                                  const double* masses, const double* dt, const double* kT,
+                                                  const double* friction, uint64_t random_seed,
+                                                  const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms,
+                                                  int32_t n_systems, void* stream) {
+    return langevin_half_step<double>(positions, velocities, forces, masses, dt, kT, friction, random_seed, batch_idx,
+                                      active, n_atoms, n_systems, stream);
 }

@@ -69,11 +69,15 @@ _SIGNATURES = {
     "nvamd_nl_rebuild_check_f64": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _c.c_double, _i32, _vp, _vp]),
     "nvamd_wrap_positions_f64": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_langevin_half_step": (_i32, [_vp] * 7 + [_c.c_uint64, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_langevin_half_step_f64": (_i32, [_vp] * 7 + [_c.c_uint64, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_fire2_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_fire2_step": (_i32, [_vp] * 11 + [_i32] + [_c.c_double] * 7 + [_vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
+    "nvamd_fire2_step_f64": (_i32, [_vp] * 11 + [_i32] + [_c.c_double] * 7 + [_vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
     "nvamd_nhc_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_nhc_chain_update": (_i32, [_vp] * 12 + [_i32] * 5 + [_vp, _c.c_size_t, _vp]),
     "nvamd_nhc_position_update": (_i32, [_vp] * 5 + [_i32, _i32, _vp]),
+    "nvamd_nhc_chain_update_f64": (_i32, [_vp] * 12 + [_i32] * 5 + [_vp, _c.c_size_t, _vp]),
+    "nvamd_nhc_position_update_f64": (_i32, [_vp] * 5 + [_i32, _i32, _vp]),
     "nvamd_nl_filter_matrix": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _f64, _vp, _vp, _vp, _vp]),
     "nvamd_nl_filter_coo_flags": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _c.c_int64, _f64, _vp, _vp]),
     "nvamd_buffer_workspace_bytes": (_i32, [_c.c_int64, _c.c_int64, _c.POINTER(_c.c_size_t)]),
@@ -782,11 +786,13 @@ def langevin_half_step(positions, velocities, forces, masses, dt, kT, friction, 
                        active=None) -> None:
     N = positions.shape[0]
     M = dt.shape[0]
-    _check(library().nvamd_langevin_half_step(
-        _dev(positions, "positions", torch.float32, (N, 3)), _dev(velocities, "velocities", torch.float32, (N, 3)),
-        _dev(forces, "forces", torch.float32, (N, 3)), _dev(masses, "masses", torch.float32, (N,)),
-        _dev(dt, "dt", torch.float32, (M,)), _dev(kT, "temperature", torch.float32, (M,)),
-        _dev(friction, "friction", torch.float32, (M,)), int(random_seed) & 0xFFFFFFFFFFFFFFFF,
+    real = _real_dtype(positions, "positions")  # float32 or float64: every float array in that one type
+    entry = library().nvamd_langevin_half_step_f64 if real == torch.float64 else library().nvamd_langevin_half_step
+    _check(entry(
+        _dev(positions, "positions", real, (N, 3)), _dev(velocities, "velocities", real, (N, 3)),
+        _dev(forces, "forces", real, (N, 3)), _dev(masses, "masses", real, (N,)),
+        _dev(dt, "dt", real, (M,)), _dev(kT, "temperature", real, (M,)),
+        _dev(friction, "friction", real, (M,)), int(random_seed) & 0xFFFFFFFFFFFFFFFF,
         _dev(batch_idx, "batch_idx", torch.int32, (N,)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
         N, M, _stream(positions.device)), "nvamd_langevin_half_step")
 
@@ -800,12 +806,14 @@ def nhc_chain_update(velocities, masses, eta, eta_dot, chain_masses, kT, dt, ndo
     N = velocities.shape[0]
     M, C = eta.shape
     ws = workspaces.get(velocities.device, "nhc", _size(lib.nvamd_nhc_workspace_bytes, M))
-    _check(lib.nvamd_nhc_chain_update(
-        _dev(velocities, "velocities", torch.float32, (N, 3)), _dev(masses, "masses", torch.float32, (N,)),
-        _dev(eta, "eta", torch.float32, (M, C)), _dev(eta_dot, "eta_dot", torch.float32, (M, C)),
-        _dev(chain_masses, "Q", torch.float32, (M, C)), _dev(kT, "temperature", torch.float32, (M,)),
-        _dev(dt, "dt", torch.float32, (M,)), _dev(ndof, "ndof", torch.float32, (M,)),
-        _dev(ke2, "ke2", torch.float32, (M,)), _dev(total_scale, "total_scale", torch.float32, (M,)),
+    real = _real_dtype(velocities, "velocities")  # float32 or float64: every float array in that one type
+    entry = lib.nvamd_nhc_chain_update_f64 if real == torch.float64 else lib.nvamd_nhc_chain_update
+    _check(entry(
+        _dev(velocities, "velocities", real, (N, 3)), _dev(masses, "masses", real, (N,)),
+        _dev(eta, "eta", real, (M, C)), _dev(eta_dot, "eta_dot", real, (M, C)),
+        _dev(chain_masses, "Q", real, (M, C)), _dev(kT, "temperature", real, (M,)),
+        _dev(dt, "dt", real, (M,)), _dev(ndof, "ndof", real, (M,)),
+        _dev(ke2, "ke2", real, (M,)), _dev(total_scale, "total_scale", real, (M,)),
         _dev(batch_idx, "batch_idx", torch.int32, (N,)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
         1 if compute_ke else 0, C, int(yoshida_order), N, M, ws.data_ptr(), ws.numel(),
         _stream(velocities.device)), "nvamd_nhc_chain_update")
@@ -814,9 +822,11 @@ def nhc_chain_update(velocities, masses, eta, eta_dot, chain_masses, kT, dt, ndo
 def nhc_position_update(positions, velocities, dt, batch_idx, active=None) -> None:
     N = positions.shape[0]
     M = dt.shape[0]
-    _check(library().nvamd_nhc_position_update(
-        _dev(positions, "positions", torch.float32, (N, 3)), _dev(velocities, "velocities", torch.float32, (N, 3)),
-        _dev(dt, "dt", torch.float32, (M,)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+    real = _real_dtype(positions, "positions")
+    entry = library().nvamd_nhc_position_update_f64 if real == torch.float64 else library().nvamd_nhc_position_update
+    _check(entry(
+        _dev(positions, "positions", real, (N, 3)), _dev(velocities, "velocities", real, (N, 3)),
+        _dev(dt, "dt", real, (M,)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         _opt(_as_u8(active), "active", torch.uint8, (M,)), N, M, _stream(positions.device)),
         "nvamd_nhc_position_update")
 
@@ -830,14 +840,20 @@ def fire2_step(positions, velocities, forces, batch_idx, alpha, dt, nsteps_inc, 
     lib = library()
     N = positions.shape[0]
     M = dt.shape[0]
-    ws = workspaces.get(positions.device, "fire2", _size(lib.nvamd_fire2_workspace_bytes, M))
-    _check(lib.nvamd_fire2_step(
-        _dev(positions, "positions", torch.float32, (N, 3)), _dev(velocities, "velocities", torch.float32, (N, 3)),
-        _dev(forces, "forces", torch.float32, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
-        _dev(alpha, "alpha", torch.float32, (M,)), _dev(dt, "dt", torch.float32, (M,)),
-        _dev(nsteps_inc, "nsteps_inc", torch.int32, (M,)), _opt(vf, "vf", torch.float32, (M,)),
-        _opt(v_sumsq, "v_sumsq", torch.float32, (M,)), _opt(f_sumsq, "f_sumsq", torch.float32, (M,)),
-        _opt(max_norm, "max_norm", torch.float32, (M,)), int(delaystep), float(dtgrow), float(dtshrink),
+    real = _real_dtype(positions, "positions")  # float32 or float64: every float array in that one type
+    if real == torch.float64:
+        entry = lib.nvamd_fire2_step_f64
+        ws = workspaces.get(positions.device, "f64", _size(lib.nvamd_f64_workspace_bytes, M))
+    else:
+        entry = lib.nvamd_fire2_step
+        ws = workspaces.get(positions.device, "fire2", _size(lib.nvamd_fire2_workspace_bytes, M))
+    _check(entry(
+        _dev(positions, "positions", real, (N, 3)), _dev(velocities, "velocities", real, (N, 3)),
+        _dev(forces, "forces", real, (N, 3)), _dev(batch_idx, "batch_idx", torch.int32, (N,)),
+        _dev(alpha, "alpha", real, (M,)), _dev(dt, "dt", real, (M,)),
+        _dev(nsteps_inc, "nsteps_inc", torch.int32, (M,)), _opt(vf, "vf", real, (M,)),
+        _opt(v_sumsq, "v_sumsq", real, (M,)), _opt(f_sumsq, "f_sumsq", real, (M,)),
+        _opt(max_norm, "max_norm", real, (M,)), int(delaystep), float(dtgrow), float(dtshrink),
         float(alphashrink), float(alpha0), float(tmax), float(tmin), float(maxstep),
         _opt(_as_u8(active), "active", torch.uint8, (M,)), N, M, ws.data_ptr(), ws.numel(),
         _stream(positions.device)), "nvamd_fire2_step")

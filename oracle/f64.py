@@ -16,6 +16,10 @@ one IEEE operation per numpy operation (numpy does not fuse multiply-adds):
                       periodic axes when the cell is given; the whole flagged system's reference refreshed)
 * ``wrap_positions``  nvalchemi/hooks/periodic.py:42-114, 159-163 (fractional coordinates mod 1, back to
                       Cartesian, per Cartesian component where that component's pbc flag is set)
+* ``langevin_half_step``  nvalchemi/dynamics/_ops/langevin.py:52-117 (B-A-O-A; the same normal deviates as the
+                      float32 oracle, which are made in double from the seed and the atom index)
+* ``nhc_chain_update / nhc_position_update``  nvalchemi/dynamics/_ops/nose_hoover.py:143-246, 291-325
+* ``fire2_step``      nvalchemi/dynamics/_ops/fire.py:467-557
 
 Pinned (tests/test_oracle_f64.py) against the float32 oracle on inputs that float32 holds exactly
 (where both must agree: to the bit for the neighbor sets, to float32 rounding elsewhere), against
@@ -27,6 +31,12 @@ the whole-system refresh) is unpinned here in the same way.  ``rebuild_check`` a
 pinned against the float32 oracle on inputs float32 holds exactly and by what the definitions fix (a wrapped
 position lies in the cell and differs from the old one by whole lattice vectors; a displacement of
 ``threshold (1 +- 1e-12)``, which float32 cannot tell from the threshold, lands on the right side).
+The thermostats and FIRE 2.0 are PARITY UNPINNED against the reference like their float32 forms (their kernels
+are in the absent library); here they are pinned against the float32 oracle on inputs float32 holds exactly
+(agreement to float32 rounding) and by what their definitions fix in double: without friction the Langevin half
+step is the velocity-Verlet drift; without forces and noise the velocity decays by exp(-gamma dt); a chain at rest
+with the kinetic energy at its target does not move; a chain of one link follows its closed form; a FIRE 2.0 step
+with P <= 0 steps half a step back, stops, and kicks once.
 """
 
 from __future__ import annotations
@@ -292,3 +302,164 @@ def wrap_positions(positions, cell, pbc, batch_idx) -> np.ndarray:
             if pbc[s][k]:
                 pos[i, k] = w[k]
     return pos
+
+
+# ---------------------------------------------------------------------------------------------
+# Langevin, Nose-Hoover chain, FIRE 2.0: the definitions of md_oracle.c's orc_langevin_half_step,
+# orc_nhc_chain_update, orc_nhc_position_update and orc_fire2_step on doubles
+# ---------------------------------------------------------------------------------------------
+def langevin_half_step(positions, velocities, forces, masses, dt, kT, friction, seed, batch_idx, active=None):
+    """In place on float64 ``positions`` / ``velocities``:
+    v += (F/m)(dt/2); r += v (dt/2); v = c1 v + c2 xi; r += v (dt/2), c1 = exp(-gamma dt),
+    c2 = sqrt((kT/m)(1 - c1^2)); xi(seed, atom) as in the float32 oracle."""
+    from . import langevin_normals
+
+    assert positions.dtype == np.float64 and velocities.dtype == np.float64
+    bi = np.asarray(batch_idx).astype(np.int64)
+    N = len(bi)
+    on = np.ones(N, bool) if active is None else np.asarray(active).astype(bool)[bi]
+    m = np.asarray(masses, dtype=np.float64)
+    h = np.asarray(dt, dtype=np.float64)[bi]
+    hh = 0.5 * h
+    c1 = np.exp(-np.asarray(friction, dtype=np.float64)[bi] * h)
+    c2 = np.sqrt((np.asarray(kT, dtype=np.float64)[bi] / m) * (1.0 - c1 * c1))
+    xi = np.array([langevin_normals(seed, i)[:3] for i in range(N)], dtype=np.float64).reshape(N, 3)
+    acc = np.asarray(forces, dtype=np.float64) / m[:, None]
+    v = velocities + acc * hh[:, None]
+    r = positions + v * hh[:, None]
+    v = c1[:, None] * v + c2[:, None] * xi
+    r = r + v * hh[:, None]
+    velocities[on] = v[on]
+    positions[on] = r[on]
+
+
+def _ys_weights(order: int):
+    if order == 3:
+        a = 1.0 / (2.0 - np.cbrt(2.0))
+        return [a, 1.0 - 2.0 * a, a]
+    if order == 5:
+        a = 1.0 / (4.0 - np.cbrt(4.0))
+        return [a, a, 1.0 - 4.0 * a, a, a]
+    return [1.0]
+
+
+def nhc_chain_update(velocities, masses, eta, eta_dot, Q, kT, dt, ndof, batch_idx, ke2=None, active=None,
+                     yoshida_order=3):
+    """In place on float64 ``velocities (N,3)``, ``eta`` and ``eta_dot (M,C)``; returns ``(ke2, total_scale)``.
+    The propagator of ``orc_nhc_chain_update`` (Martyna, Tuckerman, Tobias, Klein 1996), every value a double."""
+    import math
+
+    assert velocities.dtype == np.float64 and eta.dtype == np.float64 and eta_dot.dtype == np.float64
+    bi = np.asarray(batch_idx).astype(np.int64)
+    M, C = eta.shape
+    m = np.asarray(masses, dtype=np.float64)
+    if ke2 is None:
+        v = velocities
+        k2_all = np.bincount(bi, weights=m * ((v[:, 0] * v[:, 0] + v[:, 1] * v[:, 1]) + v[:, 2] * v[:, 2]), minlength=M)
+    else:
+        k2_all = np.asarray(ke2, dtype=np.float64).copy()
+    scale_all = np.ones(M)
+    on_s = np.ones(M, bool) if active is None else np.asarray(active).astype(bool)
+    out_k2 = k2_all.copy() if ke2 is not None else np.where(on_s, k2_all, 0.0)  # (computed sums: live systems only)
+    for s in range(M):
+        if not on_s[s]:
+            continue
+        u = [float(x) for x in eta_dot[s]]
+        x = [float(t) for t in eta[s]]
+        q = [float(t) for t in np.asarray(Q, dtype=np.float64)[s]]
+        kt, nf, h = float(kT[s]), float(ndof[s]), float(dt[s])
+        k2, scale = float(k2_all[s]), 1.0
+
+        def g_of(k):
+            return (k2 - nf * kt) / q[0] if k == 0 else (q[k - 1] * u[k - 1] * u[k - 1] - kt) / q[k]
+
+        for w in _ys_weights(yoshida_order):
+            d = w * h
+            d2, d4, d8 = 0.5 * d, 0.25 * d, 0.125 * d
+            u[C - 1] += g_of(C - 1) * d4
+            for k in range(C - 2, -1, -1):
+                aa = math.exp(-d8 * u[k + 1])
+                u[k] = (u[k] * aa + g_of(k) * d4) * aa
+            sc = math.exp(-d2 * u[0])
+            scale *= sc
+            k2 *= sc * sc
+            for k in range(C):
+                x[k] += d2 * u[k]
+            for k in range(C - 1):
+                aa = math.exp(-d8 * u[k + 1])
+                u[k] = (u[k] * aa + g_of(k) * d4) * aa
+            u[C - 1] += g_of(C - 1) * d4
+        eta_dot[s] = u
+        eta[s] = x
+        scale_all[s] = scale
+    on = on_s[bi]
+    velocities[on] = (velocities * scale_all[bi][:, None])[on]
+    return out_k2, scale_all
+
+
+def nhc_position_update(positions, velocities, dt, batch_idx, active=None):
+    """In place: r += v dt."""
+    assert positions.dtype == np.float64
+    bi = np.asarray(batch_idx).astype(np.int64)
+    on = np.ones(len(bi), bool) if active is None else np.asarray(active).astype(bool)[bi]
+    h = np.asarray(dt, dtype=np.float64)[bi][:, None]
+    positions[on] = (positions + np.asarray(velocities, dtype=np.float64) * h)[on]
+
+
+def fire2_step(positions, velocities, forces, batch_idx, alpha, dt, nsteps_inc, active=None, **params):
+    """In place on float64 ``positions``, ``velocities`` (N,3), ``alpha``, ``dt`` (M) and int32 ``nsteps_inc`` (M);
+    returns ``dict(vf, v_sumsq, f_sumsq, max_norm)``.  The step of ``orc_fire2_step``, every value a double."""
+    from . import FIRE2_DEFAULTS
+
+    for a in (positions, velocities, alpha, dt):
+        assert a.dtype == np.float64
+    p = dict(FIRE2_DEFAULTS)
+    p.update(params)
+    bi = np.asarray(batch_idx).astype(np.int64)
+    f = np.asarray(forces, dtype=np.float64)
+    M = alpha.shape[0]
+    on_s = np.ones(M, bool) if active is None else np.asarray(active).astype(bool)
+    P = np.bincount(bi, weights=(f * velocities).sum(1), minlength=M)
+    VV = np.bincount(bi, weights=(velocities * velocities).sum(1), minlength=M)
+    FF = np.bincount(bi, weights=(f * f).sum(1), minlength=M)
+    ma, mb, back, up = np.ones(M), np.zeros(M), np.zeros(M), np.zeros(M, bool)
+    for s in range(M):
+        if not on_s[s]:
+            continue
+        if P[s] > 0.0:
+            al = alpha[s]
+            up[s] = True
+            ma[s] = 1.0 - al
+            mb[s] = al * np.sqrt(VV[s] / FF[s]) if FF[s] > 1e-20 else 0.0
+            nsteps_inc[s] += 1
+            if nsteps_inc[s] > p["delaystep"]:
+                dt[s] = min(dt[s] * p["dtgrow"], p["tmax"])
+                alpha[s] = al * p["alphashrink"]
+        else:
+            nsteps_inc[s] = 0
+            alpha[s] = p["alpha0"]
+            back[s] = 0.5 * dt[s]
+            nd = dt[s] * p["dtshrink"]
+            if nd >= p["tmin"]:
+                dt[s] = nd
+    on = on_s[bi]
+    up_a = up[bi][:, None]
+    h = dt[bi][:, None]
+    r = np.where(up_a, positions, positions - back[bi][:, None] * velocities)
+    v = np.where(up_a, velocities, 0.0)
+    v = v + h * f
+    v = np.where(up_a, ma[bi][:, None] * v + mb[bi][:, None] * f, v)
+    v = np.clip(v, -1.0e300, 1.0e300)
+    dr = h * v
+    top = np.abs(dr).max(1) if len(bi) else np.zeros(0)
+    safe = np.where(top > 0.0, top, 1.0)
+    a = dr / safe[:, None]
+    nrm = np.where(top > 0.0, top * np.sqrt((a[:, 0] * a[:, 0] + a[:, 1] * a[:, 1]) + a[:, 2] * a[:, 2]), 0.0)
+    big = np.zeros(M)
+    np.maximum.at(big, bi[on], nrm[on])
+    sc = np.where(big > p["maxstep"], p["maxstep"] / np.where(big > 0.0, big, 1.0), 1.0)
+    dr = (h * v) * sc[bi][:, None]
+    velocities[on] = v[on]
+    positions[on] = (r + dr)[on]
+    max_norm = np.where(on_s, big, 0.0)
+    return {"vf": P, "v_sumsq": VV, "f_sumsq": FF, "max_norm": max_norm}

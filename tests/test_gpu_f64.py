@@ -215,6 +215,26 @@ def test_a_float64_batch_runs_through_the_package_api():
         if k == 0:
             e0 = b2.energy.clone()
     assert b2.energy.dtype == F64 and bool((b2.energy < e0).all())
+    # ... and so do FIRE 2.0 and the two thermostats: every array stays float64, the relaxation goes downhill, the
+    # thermostats heat a lattice at rest towards their temperature
+    from nvalchemi_amd.dynamics import FIRE2, NVTLangevin, NVTNoseHoover
+
+    b3 = make()
+    relax2 = FIRE2(model, dt=0.005, hooks=model.make_neighbor_hooks())
+    for k in range(30):
+        relax2.step(b3)
+        if k == 0:
+            e0 = b3.energy.clone()
+    assert b3.positions.dtype == F64 and b3.energy.dtype == F64 and bool((b3.energy < e0).all())
+    for make_dyn in (lambda: NVTLangevin(model, dt=0.05, temperature=3000.0, friction=0.5, hooks=model.make_neighbor_hooks()),
+                     lambda: NVTNoseHoover(model, dt=0.05, temperature=3000.0, thermostat_time=2.0,
+                                           hooks=model.make_neighbor_hooks())):
+        b4 = make()
+        dyn4 = make_dyn()
+        dyn4.run(b4, n_steps=40)
+        assert b4.positions.dtype == F64 and b4.velocities.dtype == F64 and dyn4._state.dt.dtype == F64
+        v = b4.velocities
+        assert bool(torch.isfinite(v).all()) and float((v * v).sum()) > 0.0
 
 
 def test_skin_test_and_wrap_on_float64_arrays():
@@ -256,3 +276,86 @@ def test_skin_test_and_wrap_on_float64_arrays():
     want = f64.wrap_positions(far, C64, pb, bi)
     got = wrap_positions_into_cell(T(far), T(C64), T(pb).bool(), T(bi))
     assert got.dtype == torch.float64 and np.array_equal(got.cpu().numpy(), want)
+
+
+def test_thermostats_and_fire2_on_float64_arrays():
+    """The Langevin half step, the Nose-Hoover chain and its drift, and FIRE 2.0 on float64 arrays against the float64
+    oracle.  Bars: the drift bit for bit; the rest to 1e-12 relative to the largest value (exp, log, sin and cos differ
+    by a rounding between the device's library and the host's; the device sums in another order), the integer
+    counters exactly."""
+    from nvalchemi_amd import _lib
+
+    rng = np.random.default_rng(21)
+    N, M = 901, 7
+    counts = rng.multinomial(N, np.ones(M) / M)
+    counts[4] = 0
+    counts[0] += N - counts.sum()
+    bi = np.repeat(np.arange(M, dtype=np.int32), counts)
+    P, V, F = rng.normal(size=(N, 3)) * 3.0, rng.normal(size=(N, 3)) * 0.05, rng.normal(size=(N, 3))  # (m v^2 about kT)
+    mass = rng.uniform(1, 30, N)
+    dt, kT, gamma = rng.uniform(0.05, 0.3, M), rng.uniform(0.02, 0.05, M), rng.uniform(0.1, 2.0, M)
+    act = np.array([1, 0, 1, 1, 1, 0, 1], dtype=np.uint8)
+    close = lambda got, want, tol=1e-12: np.abs(got.cpu().numpy() - want).max() <= tol * max(1.0, np.abs(want).max())  # noqa: E731
+
+    for active in (None, act):
+        a_t = None if active is None else T(active)
+        # Langevin
+        Pd, Vd = T(P), T(V)
+        _lib.langevin_half_step(Pd, Vd, T(F), T(mass), T(dt), T(kT), T(gamma), (1 << 40) + 12345, T(bi), a_t)
+        Pr, Vr = P.copy(), V.copy()
+        f64.langevin_half_step(Pr, Vr, F, mass, dt, kT, gamma, (1 << 40) + 12345, bi, active)
+        assert Pd.dtype == F64 and close(Pd, Pr) and close(Vd, Vr)
+        if active is not None:
+            off = active[bi] == 0
+            assert np.array_equal(Pd.cpu().numpy()[off], P[off]) and np.array_equal(Vd.cpu().numpy()[off], V[off])
+        # the chain, computing the kinetic energy and taking it from the caller
+        ndof = 3.0 * np.maximum(counts, 1)
+        for C, order in ((1, 1), (3, 3), (5, 5)):
+            Q = oracle.nhc_masses(kT, np.full(M, 0.4), ndof, C).astype(np.float64)
+            eta0, eta_dot0 = rng.normal(size=(M, C)) * 0.05, rng.normal(size=(M, C)) * 0.05
+            for supplied in (False, True):
+                Vd, e_d, d_d = T(V), T(eta0), T(eta_dot0)
+                k2_in = rng.uniform(0.5, 2.0, M) * ndof * kT
+                k2_d = T(k2_in) if supplied else torch.zeros(M, dtype=F64, device=DEV)
+                sc_d = torch.ones(M, dtype=F64, device=DEV)
+                _lib.nhc_chain_update(Vd, T(mass), e_d, d_d, T(Q), T(kT), T(dt), T(ndof), k2_d, sc_d, T(bi),
+                                      compute_ke=not supplied, yoshida_order=order, active=a_t)
+                Vr, e_r, d_r = V.copy(), eta0.copy(), eta_dot0.copy()
+                k2_r, sc_r = f64.nhc_chain_update(Vr, mass, e_r, d_r, Q, kT, dt, ndof, bi, ke2=k2_in if supplied else None,
+                                                  active=active, yoshida_order=order)
+                live = np.ones(M, bool) if active is None else active.astype(bool)
+                assert close(Vd, Vr) and close(e_d, e_r) and close(d_d, d_r), (C, order, supplied)
+                assert np.allclose(k2_d.cpu().numpy()[live], k2_r[live], rtol=1e-12)
+                assert np.allclose(sc_d.cpu().numpy()[live], sc_r[live], rtol=1e-12)
+        # the drift
+        Pd = T(P)
+        _lib.nhc_position_update(Pd, T(V), T(dt), T(bi), a_t)
+        Pr = P.copy()
+        f64.nhc_position_update(Pr, V, dt, bi, active)
+        assert np.array_equal(Pd.cpu().numpy(), Pr)
+
+    # FIRE 2.0: fifteen steps on a quadratic bowl, from velocities that point uphill in some systems; one system
+    # frozen; a maxstep that binds in the first steps
+    x0 = rng.normal(size=(N, 3))
+    Vs = np.where(np.isin(bi, [1, 3])[:, None], 0.1 * (P - x0), V)  # (systems 1 and 3 start against their forces)
+    alpha_r, dt_r, n_r = np.full(M, 0.09), np.full(M, 0.02), np.zeros(M, np.int32)
+    alpha_d, dt_d, n_d = T(alpha_r), T(dt_r), T(n_r)
+    outs = {k: torch.zeros(M, dtype=F64, device=DEV) for k in ("vf", "v_sumsq", "f_sumsq", "max_norm")}
+    Pd, Vd, Pr, Vr = T(P), T(Vs), P.copy(), Vs.copy()
+    frozen = np.array([1, 1, 1, 1, 1, 1, 0], dtype=np.uint8)
+    par = dict(delaystep=4, dtgrow=1.1, dtshrink=0.5, alphashrink=0.99, alpha0=0.09, tmax=0.1, tmin=0.001, maxstep=0.05)
+    for step in range(15):
+        Fr = -2.0 * (Pr - x0)
+        _lib.fire2_step(Pd, Vd, T(Fr), T(bi), alpha_d, dt_d, n_d, outs["vf"], outs["v_sumsq"], outs["f_sumsq"],
+                        outs["max_norm"], active=T(frozen), **par)
+        want = f64.fire2_step(Pr, Vr, Fr, bi, alpha_r, dt_r, n_r, active=frozen, **par)
+        assert close(Pd, Pr) and close(Vd, Vr), step
+        assert np.array_equal(n_d.cpu().numpy(), n_r), step
+        assert np.allclose(dt_d.cpu().numpy(), dt_r, rtol=1e-14) and np.allclose(alpha_d.cpu().numpy(), alpha_r, rtol=1e-14)
+        for k in ("vf", "v_sumsq", "f_sumsq"):
+            assert np.allclose(outs[k].cpu().numpy(), want[k], rtol=1e-12, atol=1e-12), (k, step)
+        has_atoms = (counts > 0) & (frozen != 0)
+        assert np.allclose(outs["max_norm"].cpu().numpy()[has_atoms], want["max_norm"][has_atoms], rtol=1e-12)
+        Pd.copy_(T(Pr)); Vd.copy_(T(Vr))  # (both sides continue from the same state)
+    assert n_r.max() > par["delaystep"] and (n_r[[1, 3]] < 15).all()  # (both branches and the growth were met)
+    assert np.array_equal(Pr[bi == 6], P[bi == 6])

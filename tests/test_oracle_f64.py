@@ -203,3 +203,136 @@ def test_wrap_in_double():
     W0 = f64.wrap_positions(far, C.astype(np.float64), pb0, bi)
     assert np.array_equal(W0[ptr[2]:ptr[3]], far[ptr[2]:ptr[3]])
     assert np.array_equal(W[ptr[1]:ptr[2], 1], far[ptr[1]:ptr[2], 1])
+
+
+# ---- Langevin, Nose-Hoover chain, FIRE 2.0 in double ------------------------------------------------------------
+def _thermostat_case(seed, n_systems=3, n_lo=4, n_hi=9):
+    """Per-atom and per-system arrays that float32 holds exactly (multiples of 2^-10)."""
+    g = np.random.default_rng(seed)
+    counts = g.integers(n_lo, n_hi, n_systems)
+    ptr = ptr_from_counts(counts)
+    bidx = oracle.batch_idx_from_ptr(ptr)
+    N = int(ptr[-1])
+    q = lambda a: np.round(a * 1024.0) / 1024.0  # noqa: E731
+    return dict(N=N, M=n_systems, bidx=bidx, pos=q(g.normal(size=(N, 3)) * 3.0), vel=q(g.normal(size=(N, 3)) * 0.2),
+                frc=q(g.normal(size=(N, 3))), masses=q(g.uniform(1.0, 20.0, N)), dt=q(g.uniform(0.05, 0.2, n_systems)),
+                kT=q(g.uniform(0.02, 0.05, n_systems)), friction=q(g.uniform(0.1, 2.0, n_systems)))
+
+
+def test_langevin_in_double_equals_the_float32_oracle_to_float32_rounding_and_its_closed_forms():
+    c = _thermostat_case(5)
+    active = np.array([1, 0, 1], dtype=np.uint8)
+    for act in (None, active):
+        p32, v32 = c["pos"].astype(np.float32), c["vel"].astype(np.float32)
+        oracle.langevin_half_step(p32, v32, c["frc"], c["masses"], c["dt"], c["kT"], c["friction"], 77, c["bidx"], act)
+        p64, v64 = c["pos"].copy(), c["vel"].copy()
+        f64.langevin_half_step(p64, v64, c["frc"], c["masses"], c["dt"], c["kT"], c["friction"], 77, c["bidx"], act)
+        assert np.abs(p64 - p32).max() < 2e-6 and np.abs(v64 - v32).max() < 2e-6
+        if act is not None:
+            off = act[c["bidx"]] == 0
+            assert np.array_equal(p64[off], c["pos"][off]) and np.array_equal(v64[off], c["vel"][off])
+            assert off.any() and not np.array_equal(p64[~off], c["pos"][~off])
+    # no friction: c1 = 1, c2 = 0, the noise drops out: a kick of dt/2 and two drifts of dt/2 with the kicked velocity
+    zero = np.zeros(c["M"])
+    p, v = c["pos"].copy(), c["vel"].copy()
+    f64.langevin_half_step(p, v, c["frc"], c["masses"], c["dt"], c["kT"], zero, 3, c["bidx"])
+    h = c["dt"][c["bidx"]][:, None]
+    vk = c["vel"] + (c["frc"] / c["masses"][:, None]) * (0.5 * h)
+    assert np.abs(v - vk).max() < 1e-15 and np.abs(p - (c["pos"] + vk * h)).max() < 1e-14
+    # no forces, no temperature: the velocity decays by exp(-gamma dt)
+    p, v = c["pos"].copy(), c["vel"].copy()
+    f64.langevin_half_step(p, v, np.zeros_like(c["frc"]), c["masses"], c["dt"], zero, c["friction"], 3, c["bidx"])
+    decay = np.exp(-c["friction"] * c["dt"])[c["bidx"]][:, None]
+    assert np.abs(v - c["vel"] * decay).max() < 1e-15
+    assert np.abs(p - (c["pos"] + 0.5 * h * c["vel"] * (1.0 + decay))).max() < 1e-14
+    # the noise has the amplitude sqrt(kT/m (1 - c1^2)) and the deviates of the float32 oracle
+    p, v = np.zeros((c["N"], 3)), np.zeros((c["N"], 3))
+    f64.langevin_half_step(p, v, np.zeros_like(c["frc"]), c["masses"], c["dt"], c["kT"], c["friction"], 9, c["bidx"])
+    xi = np.array([oracle.langevin_normals(9, i)[:3] for i in range(c["N"])])
+    amp = np.sqrt(c["kT"][c["bidx"]] / c["masses"] * (1.0 - np.exp(-2.0 * c["friction"] * c["dt"])[c["bidx"]]))
+    assert np.abs(v - amp[:, None] * xi).max() < 1e-14
+
+
+def test_the_chain_in_double_equals_the_float32_oracle_to_float32_rounding_and_its_closed_forms():
+    c = _thermostat_case(6, n_systems=4)
+    M, bidx = c["M"], c["bidx"]
+    ndof = 3.0 * np.bincount(bidx, minlength=M)
+    g = np.random.default_rng(1)
+    for C, order in [(1, 1), (3, 3), (4, 5)]:
+        Q = oracle.nhc_masses(c["kT"], np.full(M, 0.5), ndof, C).astype(np.float64)
+        eta0 = np.round(g.normal(size=(M, C)) * 64.0) / 1024.0
+        eta_dot0 = np.round(g.normal(size=(M, C)) * 64.0) / 1024.0
+        active = np.array([1, 1, 0, 1], dtype=np.uint8)
+        for act in (None, active):
+            v32, e32, d32 = c["vel"].astype(np.float32), eta0.astype(np.float32), eta_dot0.astype(np.float32)
+            k32, s32 = oracle.nhc_chain_update(v32, c["masses"], e32, d32, Q, c["kT"], c["dt"], ndof, bidx, active=act,
+                                               yoshida_order=order)
+            v64, e64, d64 = c["vel"].copy(), eta0.copy(), eta_dot0.copy()
+            k64, s64 = f64.nhc_chain_update(v64, c["masses"], e64, d64, Q, c["kT"], c["dt"], ndof, bidx, active=act,
+                                            yoshida_order=order)
+            live = np.ones(M, bool) if act is None else act.astype(bool)
+            assert np.abs(v64 - v32).max() < 1e-6 and np.abs(e64 - e32).max() < 1e-6 and np.abs(d64 - d32).max() < 1e-5
+            assert np.allclose(k64, k32, rtol=1e-6) and np.allclose(s64[live], s32[live], rtol=1e-6)
+            if act is not None:
+                assert np.array_equal(v64[bidx == 2], c["vel"][bidx == 2]) and np.array_equal(e64[2], eta0[2])
+    # a chain at rest with the kinetic energy at its target: the first link feels no force
+    vel = c["vel"].copy()
+    k2 = np.bincount(bidx, weights=c["masses"] * (vel * vel).sum(1), minlength=M)
+    kT = k2 / ndof
+    Q = oracle.nhc_masses(kT, np.full(M, 0.5), ndof, 3).astype(np.float64)
+    eta, eta_dot = np.zeros((M, 3)), np.zeros((M, 3))
+    # (G_1 = 0 exactly when ke2 is supplied as ndof kT; G_k = -kT / Q_k for the links above: they do move)
+    _, scale = f64.nhc_chain_update(vel, c["masses"], eta, eta_dot, Q, kT, c["dt"], ndof, bidx, ke2=ndof * kT,
+                                    yoshida_order=1)
+    assert np.all(eta_dot[:, 1:] < 0.0) and np.abs(eta_dot[:, 0]).max() < 1e-3  # (the first link only through the second)
+    # one link, one weight: u' = u + G d/4 twice around s = exp(-u d/2), with KE2 scaled by s^2 in between
+    Q1 = oracle.nhc_masses(c["kT"], np.full(M, 0.5), ndof, 1).astype(np.float64)
+    vel = c["vel"].copy()
+    k2 = np.bincount(bidx, weights=c["masses"] * (vel * vel).sum(1), minlength=M)
+    eta, eta_dot = np.zeros((M, 1)), np.full((M, 1), 0.125)
+    _, scale = f64.nhc_chain_update(vel, c["masses"], eta, eta_dot, Q1, c["kT"], c["dt"], ndof, bidx, yoshida_order=1)
+    d = c["dt"]
+    u1 = 0.125 + (k2 - ndof * c["kT"]) / Q1[:, 0] * d / 4
+    s = np.exp(-u1 * d / 2)
+    u2 = u1 + (k2 * s * s - ndof * c["kT"]) / Q1[:, 0] * d / 4
+    assert np.abs(scale - s).max() < 1e-15 and np.abs(eta_dot[:, 0] - u2).max() < 1e-14
+    assert np.abs(eta[:, 0] - u1 * d / 2).max() < 1e-16 and np.abs(vel - c["vel"] * s[bidx][:, None]).max() < 1e-15
+    # the drift
+    p = c["pos"].copy()
+    f64.nhc_position_update(p, c["vel"], c["dt"], bidx, np.array([1, 0, 1, 1], dtype=np.uint8))
+    want = c["pos"] + c["vel"] * c["dt"][bidx][:, None]
+    assert np.array_equal(p[bidx != 1], want[bidx != 1]) and np.array_equal(p[bidx == 1], c["pos"][bidx == 1])
+
+
+def test_fire2_in_double_equals_the_float32_oracle_to_float32_rounding_and_its_uphill_form():
+    c = _thermostat_case(8, n_systems=4, n_lo=5, n_hi=12)
+    M, bidx = c["M"], c["bidx"]
+    # systems 0 and 2 uphill (v against F), 1 and 3 downhill
+    vel = c["vel"].copy()
+    sign = np.where(np.isin(bidx, [0, 2]), -1.0, 1.0)[:, None]
+    vel = sign * np.abs(vel) * np.sign(c["frc"] + 1e-30)
+    active = np.array([1, 1, 1, 0], dtype=np.uint8)
+    for act in (None, active):
+        for maxstep in (0.1, 0.004):
+            a32, d32, n32 = np.full(M, 0.09, np.float32), np.full(M, 0.03125, np.float32), np.array([60, 61, 3, 7], np.int32)
+            p32, v32 = c["pos"].astype(np.float32), vel.astype(np.float32)
+            o32 = oracle.fire2_step(p32, v32, c["frc"], bidx, a32, d32, n32, active=act, maxstep=maxstep)
+            a64, d64, n64 = np.full(M, 0.09), np.full(M, 0.03125), np.array([60, 61, 3, 7], np.int32)
+            p64, v64 = c["pos"].copy(), vel.copy()
+            o64 = f64.fire2_step(p64, v64, c["frc"], bidx, a64, d64, n64, active=act, maxstep=maxstep)
+            assert np.abs(p64 - p32).max() < 2e-6 and np.abs(v64 - v32).max() < 2e-6
+            assert np.array_equal(n64, n32) and np.allclose(a64, a32, rtol=1e-6) and np.allclose(d64, d32, rtol=1e-6)
+            for k in ("vf", "v_sumsq", "f_sumsq"):
+                assert np.allclose(o64[k], o32[k], rtol=1e-6), k
+            live = np.ones(M, bool) if act is None else act.astype(bool)
+            assert np.allclose(o64["max_norm"][live], o32["max_norm"][live], rtol=1e-5)
+            assert n64[0] == 0 and n64[1] == 62 and (act is not None or n64[3] == 8)
+    # P <= 0 in double: half a step back with the old velocity, then a plain kick and drift from rest
+    a, d, n = np.full(M, 0.2), np.full(M, 0.0625), np.full(M, 9, np.int32)
+    p, v = c["pos"].copy(), vel.copy()
+    f64.fire2_step(p, v, c["frc"], bidx, a, d, n, maxstep=1e9, dtshrink=0.5, tmin=0.0)
+    up = np.isin(bidx, [0, 2])
+    assert np.array_equal(d, np.where(np.isin(np.arange(M), [0, 2]), 0.03125, 0.0625)) and a[0] == 0.09 and n[0] == 0
+    want_v = 0.03125 * c["frc"][up]
+    assert np.abs(v[up] - want_v).max() < 1e-17
+    assert np.abs(p[up] - (c["pos"][up] - 0.03125 * vel[up] + 0.03125 * want_v)).max() < 1e-15
