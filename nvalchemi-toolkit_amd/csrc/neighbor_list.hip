@@ -37,18 +37,31 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / kWave;
-constexpr int kTile = 1088;       // candidates staged in LDS at a time
+#ifndef NVAMD_NL_TILE
+#define NVAMD_NL_TILE 1088
+#endif
+constexpr int kTile = NVAMD_NL_TILE;  // candidates staged in LDS at a time
 constexpr int kStencilBatch = 64; // stencil cells enumerated at a time (one per lane of a wave)
-constexpr int kCenterChunk = 72;  // centre atoms of a run of cells handled per pass
+#ifndef NVAMD_NL_MAXCHUNK
+#define NVAMD_NL_MAXCHUNK 72
+#endif
+constexpr int kCenterChunk = NVAMD_NL_MAXCHUNK;  // centre atoms of a run of cells handled per pass
 #ifndef NVAMD_NL_CHUNK
 #define NVAMD_NL_CHUNK(n) center_chunk_for(n)
 #endif
+// Centre atoms per unit of work for a batch of n_atoms: kCenterChunk from 58 000 atoms on, 16 below 19 000 (measured
+// on batches of 500-atom FCC boxes and of 3900-atom liquid boxes of 4 000 to 250 000 atoms: smaller units fill the
+// chip sooner, larger ones stage their tile for more centre atoms; 40, whole cells of the FCC boxes, is the best
+// at 32 000 atoms for both)
 inline int center_chunk_for(int n_atoms) {
-    int c = n_atoms / 4096 / 8 * 8;
+    int c = n_atoms / 800 / 8 * 8;
     return c < 16 ? 16 : (c > kCenterChunk ? kCenterChunk : c);
 }
 constexpr int kMaxRun = 4;        // a workgroup's unit of work: up to this many cells in a row along z
-constexpr int kHitCap = 256;      // per-wave list of accepted candidates before it is written out
+#ifndef NVAMD_NL_HITCAP
+#define NVAMD_NL_HITCAP 256
+#endif
+constexpr int kHitCap = NVAMD_NL_HITCAP;      // per-wave list of accepted candidates before it is written out
 constexpr int kPackOverflow = 1 << 15;
 static_assert(kMaxRun <= 4, "a centre atom's place in its run is kept in two bits");
 constexpr int kMaxCellsPerAxis = 1024;
@@ -1449,7 +1462,7 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     a.tail_mode = tail_mode ? 1 : 0;
     a.unit_group = 1;
     while (a.unit_group < 64 && (long long)a.unit_group * 8192 <= (long long)n_atoms) a.unit_group *= 2;
-    // A small batch does not fill the chip with units of kCenterChunk centre atoms: smaller units, about 4096 of them
+    // A small batch does not fill the chip with units of kCenterChunk centre atoms: smaller units
     a.center_chunk = NVAMD_NL_CHUNK(n_atoms);
     a.tile_index = tile_index;
     a.tile_xyz = reinterpret_cast<float4*>(ordered_positions);
