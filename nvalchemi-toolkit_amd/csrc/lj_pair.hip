@@ -963,6 +963,10 @@ void launch_full(const LjArgs& a, bool virial, bool shifts, bool sys, hipStream_
     // systems' positions and to keep per-system sums in LDS, short enough to fill the chip
     int rows = 512;
     while (rows > 4 * G && (a.n_atoms + rows - 1) / rows < 256 * 6) rows /= 2;
+    // a batch that still leaves most of the chip idle: shorter runs, down to one pass of the workgroup, until there
+    // are three workgroups for every two CUs (measured on batches of 4 000 to 500 000 atoms: 23 -> 12 us at 4 000
+    // atoms, 25 -> 18 us at 32 000; from 128 000 atoms on the runs above are as fast or faster)
+    while (rows > G && (a.n_atoms + rows - 1) / rows < 384) rows /= 2;
     rows = (rows + G - 1) / G * G;
     // With work for more than two rounds of resident workgroups (three per CU, two with the virial) and systems
     // small enough to be staged, equal shares for a whole number of rounds: the last round is then as full as the
