@@ -256,6 +256,18 @@ int32_t nvamd_nhc_position_update(float* positions, const float* velocities, con
                                   const int32_t* batch_idx, const uint8_t* active, int32_t n_atoms,
                                   int32_t n_systems, void* stream);
 
+/* What ConvergenceHook does with the result of its criterion (nvalchemi/dynamics/base.py:2459-2502: systems
+ * that are converged and whose status equals source_status get target_status), for a criterion of the form
+ * value <= threshold: status[s] = target_status where values[s] <= threshold and status[s] == source_status, in
+ * one launch instead of the reference's six Torch kernels and its host read of migrate.any().  values (M) f32 (for
+ * the default criterion: the output of nvamd_segment_fmax), status (M) i64 contiguous, updated in place.  The
+ * threshold is compared in the values' type, as Torch compares a tensor with a Python float; a NaN is not
+ * converged.  nvamd_status_migrate_f64 takes double values. */
+int32_t nvamd_status_migrate(const float* values, double threshold, int64_t* status, int64_t source_status,
+                             int64_t target_status, int32_t n_systems, void* stream);
+int32_t nvamd_status_migrate_f64(const double* values, double threshold, int64_t* status, int64_t source_status,
+                                 int64_t target_status, int32_t n_systems, void* stream);
+
 /* Per-system maximum atomic force norm (the default convergence criterion,
  * nvalchemi/dynamics/base.py:258-349: vector_norm over xyz, scatter amax over atoms).
  * fmax (M) f32; systems without atoms give -inf. */

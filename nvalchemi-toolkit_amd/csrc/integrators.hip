@@ -562,6 +562,17 @@ __global__ __launch_bounds__(kBlock) void fire2_drift_kernel(float* __restrict__
     if (max_norm && (i == 0 || bidx[i - 1] != s)) max_norm[s] = big;
 }
 
+// ---- status of converged systems -----------------------------------------------------------
+// status[s] = target where values[s] <= threshold and status[s] == source (a NaN value is not converged)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void status_migrate_kernel(const T* __restrict__ values, T threshold,
+                                                                long long* __restrict__ status, long long source,
+                                                                long long target, int m) {
+    const int s = blockIdx.x * kBlock + threadIdx.x;
+    if (s >= m) return;
+    if (values[s] <= threshold && status[s] == source) status[s] = target;
+}
+
 // ---- per-system max force norm ------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void fmax_init_kernel(float* fmax, int m) {
     int s = blockIdx.x * kBlock + threadIdx.x;
@@ -745,4 +756,31 @@ NVAMD_EXPORT int32_t nvamd_segment_fmax(const float* forces, const int32_t* batc
                            forces, batch_idx, fmax, n_atoms);
     NVAMD_LAUNCH_CHECK("fmax launch");
     return NVAMD_OK;
+}
+
+namespace {
+template <typename T>
+int32_t status_migrate(const T* values, double threshold, int64_t* status, int64_t source_status, int64_t target_status,
+                       int32_t n_systems, void* stream) {
+    if (n_systems < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "status migrate: negative size");
+    if (n_systems == 0) return NVAMD_OK;
+    if (!values || !status) return fail(NVAMD_ERR_INVALID_ARGUMENT, "status migrate: null buffer");
+    hipLaunchKernelGGL(status_migrate_kernel<T>, dim3((n_systems + kBlock - 1) / kBlock), dim3(kBlock), 0,
+                       static_cast<hipStream_t>(stream), values, (T)threshold, reinterpret_cast<long long*>(status),
+                       (long long)source_status, (long long)target_status, n_systems);
+    NVAMD_LAUNCH_CHECK("status migrate launch");
+    return NVAMD_OK;
+}
+}  // namespace
+
+NVAMD_EXPORT int32_t nvamd_status_migrate(const float* values, double threshold, int64_t* status,
+                                          int64_t source_status, int64_t target_status, int32_t n_systems,
+                                          void* stream) {
+    return status_migrate<float>(values, threshold, status, source_status, target_status, n_systems, stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_status_migrate_f64(const double* values, double threshold, int64_t* status,
+                                              int64_t source_status, int64_t target_status, int32_t n_systems,
+                                              void* stream) {
+    return status_migrate<double>(values, threshold, status, source_status, target_status, n_systems, stream);
 }

@@ -54,6 +54,8 @@ _SIGNATURES = {
     "nvamd_fire_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_fire_step": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
     "nvamd_segment_fmax": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp]),
+    "nvamd_status_migrate": (_i32, [_vp, _f64, _vp, _c.c_int64, _c.c_int64, _i32, _vp]),
+    "nvamd_status_migrate_f64": (_i32, [_vp, _f64, _vp, _c.c_int64, _c.c_int64, _i32, _vp]),
     "nvamd_lj_energy_forces_hinted": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_repeat": (_i32, [_vp] * 7 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 4 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
     "nvamd_lj_energy_forces_tiles": (_i32, [_vp] * 11 + [_c.c_double] + [_i32] * 4 + [_c.c_double] * 3 + [_i32] + [_vp] * 5 + [_c.c_size_t, _vp]),
@@ -568,6 +570,18 @@ def fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_a
         _dev(ff, "ff", f32, (M,)), _dev(batch_idx, "batch_idx", i32, (N,)),
         int(bool(compute_reductions)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
         N, M, ws.data_ptr(), ws.numel(), _stream(positions.device)), "nvamd_fire_step")
+
+
+def status_migrate(values, threshold: float, status, source_status: int, target_status: int) -> None:
+    """``status[s] = target_status`` where ``values[s] <= threshold`` and ``status[s] == source_status``; ``values (M)``
+    float32 or float64, ``status`` int64 with at least M contiguous entries (the first M are looked at)."""
+    M = values.shape[0]
+    real = _real_dtype(values, "values")
+    if status.dtype != torch.int64 or not status.is_contiguous() or status.numel() < M or status.device != values.device:
+        raise ValueError("status: expected a contiguous int64 tensor of at least as many entries as values, on their device")
+    entry = library().nvamd_status_migrate_f64 if real == torch.float64 else library().nvamd_status_migrate
+    _check(entry(_dev(values, "values", real, (M,)), float(threshold), status.data_ptr(), int(source_status),
+                 int(target_status), M, _stream(values.device)), "nvamd_status_migrate")
 
 
 def segment_fmax(forces, batch_idx, fmax) -> None:

@@ -81,6 +81,24 @@ class _ConvergenceCriterion(BaseModel):
                 and target.shape[1] == 3 and target.dtype in (torch.float32, torch.float64) and target.is_cuda
                 and target.shape[0] == batch.num_nodes and batch.num_nodes != batch.num_graphs)
 
+    @staticmethod
+    def _force_norm_max(target: torch.Tensor, batch) -> torch.Tensor:
+        """Per-system max of the atomic force norms in one pass."""
+        fmax = torch.empty(batch.num_graphs, dtype=target.dtype, device=target.device)
+        _lib.segment_fmax(target.contiguous(), batch.batch_idx, fmax)
+        return fmax
+
+    def reduced_values(self, batch) -> torch.Tensor | None:
+        """The per-system values that ``__call__`` compares with the threshold, where they come from a kernel of this
+        library (the maximum force norm); ``None`` for every other criterion."""
+        target = getattr(batch, self.key, None)
+        if target is None:
+            raise KeyError("Key for convergence check not found;"
+                           f" expected={self.key!r}, available={list(batch.keys())}")
+        if self.custom_op is None and self._is_force_norm(target, batch):
+            return self._force_norm_max(target, batch)
+        return None
+
     def __call__(self, batch) -> torch.Tensor:
         target = getattr(batch, self.key, None)
         if target is None:
@@ -89,10 +107,7 @@ class _ConvergenceCriterion(BaseModel):
         if self.custom_op is not None:
             return self.custom_op(target)
         if self._is_force_norm(target, batch):
-            # per-system max of the atomic force norms in one pass
-            fmax = torch.empty(batch.num_graphs, dtype=target.dtype, device=target.device)
-            _lib.segment_fmax(target.contiguous(), batch.batch_idx, fmax)
-            return fmax <= self.threshold
+            return self._force_norm_max(target, batch) <= self.threshold
         target = self._reduce_within_entry(target)
         is_node_level = target.shape[0] == batch.num_nodes and batch.num_nodes != batch.num_graphs
         if is_node_level:
@@ -166,6 +181,16 @@ class ConvergenceHook:
 
     def __call__(self, ctx: DynamicsContext, stage: Enum) -> None:
         batch = ctx.batch
+        status = getattr(batch, "status", None)
+        migrates = self.source_status is not None and self.target_status is not None and status is not None
+        if (migrates and len(self.criteria) == 1 and status.dtype == torch.int64 and status.is_cuda
+                and status.is_contiguous() and status.numel() >= batch.num_graphs):
+            # one criterion on the maximum force norm: comparison and migration in one launch
+            values = self.criteria[0].reduced_values(batch)
+            if values is not None:
+                _lib.status_migrate(values, self.criteria[0].threshold, status.view(-1), self.source_status,
+                                    self.target_status)
+                return
         mask = self.converged_mask(batch)  # (a missing key is an error whether or not anything migrates)
         if self.source_status is None or self.target_status is None:
             return

@@ -997,3 +997,49 @@ def test_steps_inside_the_stream_context_run_on_its_stream_and_give_the_same_tra
     with fused:
         assert fused.stream is not None and a.stream is fused.stream and b.stream is fused.stream
     assert fused.stream is None and a.stream is None and b.stream is None
+
+
+def test_status_migration_in_one_launch_equals_the_torch_expression():
+    """nvamd_status_migrate against ``status[(values <= thr) & (status == source)] = target`` written out in Torch
+    (nvalchemi/dynamics/base.py:2459-2502), on values that include the threshold itself, -inf (a system without
+    atoms), +inf and NaN; float32 and float64 values; and ConvergenceHook with one force criterion (the one launch)
+    against the same hook with a second, always-true criterion (the general Torch path)."""
+    from nvalchemi_amd import _lib
+    from nvalchemi_amd.dynamics import ConvergenceHook
+    from nvalchemi_amd.hooks._context import DynamicsContext
+
+    g = torch.Generator().manual_seed(3)
+    M = 1000
+    for dtype in (torch.float32, torch.float64):
+        values = torch.rand(M, generator=g, dtype=dtype) * 0.1
+        values[:6] = torch.tensor([0.05, float("-inf"), float("inf"), float("nan"), 0.05000001, 0.04999999], dtype=dtype)
+        status = torch.randint(0, 3, (M + 7,), generator=g, dtype=torch.int64)
+        status[:6] = 1
+        want = status.clone()
+        thr = torch.tensor(0.05, dtype=dtype)
+        pick = (values <= thr) & (want[:M] == 1)
+        want[:M][pick] = 5
+        got = status.to(DEV)
+        _lib.status_migrate(values.to(DEV), 0.05, got, 1, 5)
+        assert torch.equal(got.cpu(), want), dtype
+        assert want[0] == 5 and want[1] == 5 and want[2] == 1 and want[3] == 1 and want[5] == 5
+    with pytest.raises(ValueError):
+        _lib.status_migrate(values.to(DEV), 0.05, status[:10].to(DEV), 1, 5)
+    with pytest.raises(ValueError):
+        _lib.status_migrate(values.to(DEV), 0.05, status.to(DEV).int(), 1, 5)
+
+    P, C, pb, ptr = fcc_boxes(seed=5, n_boxes=6, reps=2, a=1.5496, jitter=0.02)
+    N = len(P)
+    batch = make_batch(P, np.full(N, 18, dtype=np.int64), np.ones(N, dtype=np.float32), C, pb, ptr)
+    f = torch.randn(N, 3, generator=g) * torch.repeat_interleave(torch.tensor([0.001, 1.0, 0.01, 0.5, 0.002, 2.0]), N // 6)[:, None]
+    batch.forces.copy_(f.to(DEV))
+    start = torch.tensor([0, 0, 1, 0, 2, 0], dtype=torch.long, device=DEV).view(-1, 1)
+    one = ConvergenceHook.from_fmax(0.05, source_status=0, target_status=1)
+    two = ConvergenceHook(criteria=[{"key": "forces", "threshold": 0.05, "reduce_op": "norm"},
+                                    {"key": "energy", "threshold": 1e30}], source_status=0, target_status=1)
+    out = []
+    for hook in (one, two):
+        batch.status = start.clone()
+        hook(DynamicsContext(batch=batch, model=None, workflow=None), None)
+        out.append(batch.status.clone())
+    assert torch.equal(out[0], out[1]) and out[0].view(-1).tolist() == [1, 0, 1, 0, 2, 0]
