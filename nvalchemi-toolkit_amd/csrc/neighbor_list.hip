@@ -609,6 +609,10 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* s_part, int* tot
     return before + incl - v;
 }
 
+// kKeep: atoms per thread whose positions and bins stay in registers from the histogram to the scatter (systems of
+// up to kKeep * kSortBlock atoms are binned once).  Four for batches of small systems, where the registers of eight
+// would leave one workgroup per CU; eight when the mean system has more than 2048 atoms.
+template <int kKeep>
 __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, NlWorkspace ws) {
     __shared__ NlSys s_sys;
     __shared__ uint32_t s_bounds[6];
@@ -625,7 +629,6 @@ __global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, Nl
     const int begin = a.ptr[t], end = a.ptr[t + 1];
     // up to kKeep atoms per thread stay in registers from here to the scatter; their positions
     // are requested now, so that they arrive while thread 0 works out the system's grid
-    constexpr int kKeep = 4;
     const bool kept = !a.pos64 && (end - begin) <= kKeep * kSortBlock;
     float my_pos[kKeep][3];
     if (kept) {
@@ -1486,7 +1489,10 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
                                                             : (sort_path == NVAMD_NL_SORT_PER_SYSTEM);
     if (per_system) {
         // many small systems: set-up to scatter in one workgroup per system
-        hipLaunchKernelGGL(nl_system_sort_kernel, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
+        if (!a.pos64 && n_atoms / n_systems > 4 * kSortBlock && n_atoms / n_systems <= 8 * kSortBlock)
+            hipLaunchKernelGGL(nl_system_sort_kernel<8>, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
+        else
+            hipLaunchKernelGGL(nl_system_sort_kernel<4>, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
     } else {
         size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
         hipLaunchKernelGGL(nl_prepare_kernel, blocks(n_prep), blk, 0, st, a, ws);
