@@ -171,6 +171,15 @@ int32_t nvamd_vv_velocity_finalize(float* velocities, const float* forces_new,
                                    const int32_t* batch_idx, const uint8_t* active,
                                    int32_t n_atoms, int32_t n_systems, void* stream);
 
+/* nvamd_vv_velocity_finalize followed by nvamd_vv_position_update with the same forces, in one launch: the closing
+ * half kick of one step and the opening half kick and drift of the next, which the reference launches back to back
+ * when nothing is registered between two steps (nvalchemi/dynamics/base.py:1875-1883 for consecutive steps).  No
+ * counterpart in the reference; the results are those of the two calls in a row, bit for bit (the same operations
+ * in the same order per element).  float32 only. */
+int32_t nvamd_vv_finalize_then_update(float* positions, float* velocities, const float* forces,
+                                      const float* masses, const float* dt, const int32_t* batch_idx,
+                                      const uint8_t* active, int32_t n_atoms, int32_t n_systems, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * FIRE step.  Replaces nvalchemi::_fire_step_op (nvalchemi/dynamics/_ops/fire.py:79-140).
  *   All per-system arrays have M entries; alpha, dt, n_steps_positive, vf, vv, ff and

@@ -50,8 +50,17 @@ __device__ __forceinline__ AtomOperands load_atom(uint32_t atom, const float* __
     return o;
 }
 
+// MODE 0: the closing half kick; 1: half kick and drift; 2: the closing half kick of one step and the half kick and
+// drift of the next with the same forces, one after the other per element (the same operations in the same order
+// as launches 0 and 1 in a row: the velocity in between is rounded as it would be stored).
+template <int MODE>
+__device__ __forceinline__ void vv_elem(float& r, float& v, float f, float m, float h) {
+    if (MODE != 1) vv_post_elem(v, f, m, h);
+    if (MODE != 0) vv_pre_elem(r, v, f, m, h);
+}
+
 // One lane owns four consecutive floats of the flat (3N) stream: at most two atoms.
-template <bool PRE>
+template <int MODE>
 __global__ __launch_bounds__(kBlock) void vv_flat_kernel(
     float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
     const float* __restrict__ masses, const float* __restrict__ dt,
@@ -69,8 +78,8 @@ __global__ __launch_bounds__(kBlock) void vv_flat_kernel(
         float4 f4 = reinterpret_cast<const float4*>(frc)[t];
         float v[4] = {v4.x, v4.y, v4.z, v4.w};
         float f[4] = {f4.x, f4.y, f4.z, f4.w};
-        float r[4];
-        if (PRE) {
+        float r[4] = {0.f, 0.f, 0.f, 0.f};
+        if (MODE != 0) {
             float4 r4 = reinterpret_cast<const float4*>(pos)[t];
             r[0] = r4.x; r[1] = r4.y; r[2] = r4.z; r[3] = r4.w;
         }
@@ -78,25 +87,22 @@ __global__ __launch_bounds__(kBlock) void vv_flat_kernel(
         for (int k = 0; k < 4; ++k) {
             bool second = (rem + k) >= 3u;
             const AtomOperands& o = second ? o1 : o0;
-            if (o.on) {
-                if (PRE) vv_pre_elem(r[k], v[k], f[k], o.m, o.h);
-                else vv_post_elem(v[k], f[k], o.m, o.h);
-            }
+            if (o.on) vv_elem<MODE>(r[k], v[k], f[k], o.m, o.h);
         }
         reinterpret_cast<float4*>(vel)[t] = make_float4(v[0], v[1], v[2], v[3]);
-        if (PRE) reinterpret_cast<float4*>(pos)[t] = make_float4(r[0], r[1], r[2], r[3]);
+        if (MODE != 0) reinterpret_cast<float4*>(pos)[t] = make_float4(r[0], r[1], r[2], r[3]);
     } else {
         for (uint32_t e = e0; e < n_elems; ++e) {
             AtomOperands o = load_atom(e / 3u, masses, dt, bidx, active);
             if (!o.on) continue;
-            if (PRE) vv_pre_elem(pos[e], vel[e], frc[e], o.m, o.h);
-            else vv_post_elem(vel[e], frc[e], o.m, o.h);
+            float none = 0.f;
+            vv_elem<MODE>(MODE != 0 ? pos[e] : none, vel[e], frc[e], o.m, o.h);
         }
     }
 }
 
 // Fallback for buffers that are not 16-byte aligned: one lane per float.
-template <bool PRE>
+template <int MODE>
 __global__ __launch_bounds__(kBlock) void vv_scalar_kernel(
     float* __restrict__ pos, float* __restrict__ vel, const float* __restrict__ frc,
     const float* __restrict__ masses, const float* __restrict__ dt,
@@ -105,30 +111,30 @@ __global__ __launch_bounds__(kBlock) void vv_scalar_kernel(
     if (e >= n_elems) return;
     AtomOperands o = load_atom(e / 3u, masses, dt, bidx, active);
     if (!o.on) return;
-    if (PRE) vv_pre_elem(pos[e], vel[e], frc[e], o.m, o.h);
-    else vv_post_elem(vel[e], frc[e], o.m, o.h);
+    float none = 0.f;
+    vv_elem<MODE>(MODE != 0 ? pos[e] : none, vel[e], frc[e], o.m, o.h);
 }
 
-template <bool PRE>
+template <int MODE>
 int32_t launch_vv(float* pos, float* vel, const float* frc, const float* masses, const float* dt,
                   const int32_t* bidx, const uint8_t* active, int32_t n_atoms, void* stream) {
     if (n_atoms < 0) return fail(NVAMD_ERR_INVALID_ARGUMENT, "n_atoms < 0");
     if (n_atoms == 0) return NVAMD_OK;
-    if ((PRE && !pos) || !vel || !frc || !masses || !dt || !bidx)
+    if ((MODE != 0 && !pos) || !vel || !frc || !masses || !dt || !bidx)
         return fail(NVAMD_ERR_INVALID_ARGUMENT, "velocity Verlet: null buffer");
     if ((int64_t)n_atoms * 3 > 0x7fffffff)
         return fail(NVAMD_ERR_UNSUPPORTED, "velocity Verlet: more than 2^31/3 atoms");
     uint32_t n_elems = 3u * (uint32_t)n_atoms;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    bool vec = aligned16(vel) && aligned16(frc) && (!PRE || aligned16(pos));
+    bool vec = aligned16(vel) && aligned16(frc) && (MODE == 0 || aligned16(pos));
     if (vec) {
         uint32_t n_threads = (n_elems + 3u) / 4u;
         dim3 grid((n_threads + kBlock - 1) / kBlock);
-        hipLaunchKernelGGL(vv_flat_kernel<PRE>, grid, dim3(kBlock), 0, st, pos, vel, frc, masses, dt,
+        hipLaunchKernelGGL(vv_flat_kernel<MODE>, grid, dim3(kBlock), 0, st, pos, vel, frc, masses, dt,
                            bidx, active, n_elems);
     } else {
         dim3 grid((n_elems + kBlock - 1) / kBlock);
-        hipLaunchKernelGGL(vv_scalar_kernel<PRE>, grid, dim3(kBlock), 0, st, pos, vel, frc, masses,
+        hipLaunchKernelGGL(vv_scalar_kernel<MODE>, grid, dim3(kBlock), 0, st, pos, vel, frc, masses,
                            dt, bidx, active, n_elems);
     }
     NVAMD_LAUNCH_CHECK("velocity Verlet launch");
@@ -610,8 +616,8 @@ NVAMD_EXPORT int32_t nvamd_vv_position_update(float* positions, float* velocitie
                                               const uint8_t* active, int32_t n_atoms,
                                               int32_t n_systems, void* stream) {
     (void)n_systems;
-    return launch_vv<true>(positions, velocities, forces, masses, dt, batch_idx, active, n_atoms,
-                           stream);
+    return launch_vv<1>(positions, velocities, forces, masses, dt, batch_idx, active, n_atoms,
+                        stream);
 }
 
 NVAMD_EXPORT int32_t nvamd_vv_velocity_finalize(float* velocities, const float* forces_new,
@@ -619,8 +625,16 @@ NVAMD_EXPORT int32_t nvamd_vv_velocity_finalize(float* velocities, const float* 
                                                 const int32_t* batch_idx, const uint8_t* active,
                                                 int32_t n_atoms, int32_t n_systems, void* stream) {
     (void)n_systems;
-    return launch_vv<false>(nullptr, velocities, forces_new, masses, dt, batch_idx, active, n_atoms,
-                            stream);
+    return launch_vv<0>(nullptr, velocities, forces_new, masses, dt, batch_idx, active, n_atoms,
+                        stream);
+}
+
+NVAMD_EXPORT int32_t nvamd_vv_finalize_then_update(float* positions, float* velocities, const float* forces,
+                                                   const float* masses, const float* dt, const int32_t* batch_idx,
+                                                   const uint8_t* active, int32_t n_atoms, int32_t n_systems,
+                                                   void* stream) {
+    (void)n_systems;
+    return launch_vv<2>(positions, velocities, forces, masses, dt, batch_idx, active, n_atoms, stream);
 }
 
 NVAMD_EXPORT int32_t nvamd_fire_workspace_bytes(int32_t n_systems, size_t* bytes) {

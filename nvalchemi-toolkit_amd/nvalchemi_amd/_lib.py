@@ -50,6 +50,7 @@ _SIGNATURES = {
     "nvamd_lj_energy_forces": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _f64, _f64,
                                       _f64, _f64, _i32, _vp, _vp, _vp, _vp, _vp, _c.c_size_t, _vp]),
     "nvamd_vv_position_update": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp]),
+    "nvamd_vv_finalize_then_update": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_vv_velocity_finalize": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _vp]),
     "nvamd_fire_workspace_bytes": (_i32, [_i32, _c.POINTER(_c.c_size_t)]),
     "nvamd_fire_step": (_i32, [_vp] * 20 + [_i32, _vp, _i32, _i32, _vp, _c.c_size_t, _vp]),
@@ -541,6 +542,18 @@ def vv_velocity_finalize(velocities, forces_new, masses, dt, batch_idx, active=N
         _dev(batch_idx, "batch_idx", torch.int32, (N,)),
         _opt(_as_u8(active), "active", torch.uint8, (M,)),
         N, M, _stream(velocities.device)), "nvamd_vv_velocity_finalize")
+
+
+def vv_finalize_then_update(positions, velocities, forces, masses, dt, batch_idx, active=None) -> None:
+    """``vv_velocity_finalize`` then ``vv_position_update`` with the same forces, in one launch (float32)."""
+    N = positions.shape[0]
+    M = dt.shape[0]
+    f32 = torch.float32
+    _check(library().nvamd_vv_finalize_then_update(
+        _dev(positions, "positions", f32, (N, 3)), _dev(velocities, "velocities", f32, (N, 3)),
+        _dev(forces, "forces", f32, (N, 3)), _dev(masses, "masses", f32, (N,)), _dev(dt, "dt", f32, (M,)),
+        _dev(batch_idx, "batch_idx", torch.int32, (N,)), _opt(_as_u8(active), "active", torch.uint8, (M,)),
+        N, M, _stream(positions.device)), "nvamd_vv_finalize_then_update")
 
 
 def fire_step(positions, velocities, forces, masses, alpha, dt, alpha_start, f_alpha, dt_min, dt_max,

@@ -617,6 +617,34 @@ class BaseDynamics(HookRegistryMixin):
             key.append((id(hook), fn() if callable(fn) else None))
         return tuple(key)
 
+    def _capture(self, batch, body, key):
+        """``body()`` captured as a HIP graph on a side stream; None if it cannot be (something in it needs the
+        host, or it replaced one of the buffers that ``key`` names)."""
+        from .. import _lib
+
+        graph = torch.cuda.CUDAGraph()
+        current = torch.cuda.current_stream()
+        side = torch.cuda.Stream(device=current.device)
+        # the captured kernels use the workspaces of the stream the eager steps ran on: replays are
+        # launched into that stream, in order with its other work
+        _lib.workspaces.share(current.device, current.cuda_stream, side.cuda_stream)
+        count, converged, mask = self.step_count, self._last_converged, self._active_mask
+        side.wait_stream(current)
+        try:
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    body()
+        except Exception:  # something in the step needs the host after all: stay eager for this batch
+            return None
+        finally:
+            current.wait_stream(side)
+            _lib.workspaces.unshare(current.device, side.cuda_stream)
+            # (the capture ran nothing)
+            self.step_count, self._last_converged, self._active_mask = count, converged, mask
+        if self._graph_key(batch) != key:  # the body replaced a buffer: what was captured is already stale
+            return None
+        return graph
+
     def _graph_step(self, batch) -> bool:
         """One step by graph replay.  False: not possible now (the caller takes the step eagerly)."""
         if not self._graph_eligible(batch):
@@ -632,28 +660,8 @@ class BaseDynamics(HookRegistryMixin):
             if st["warm"] < self._GRAPH_WARM_STEPS:
                 st["warm"] += 1
                 return False
-            from .. import _lib
-
-            graph = torch.cuda.CUDAGraph()
-            current = torch.cuda.current_stream()
-            side = torch.cuda.Stream(device=current.device)
-            # the captured kernels use the workspaces of the stream the eager steps ran on: replays are
-            # launched into that stream, in order with its other work
-            _lib.workspaces.share(current.device, current.cuda_stream, side.cuda_stream)
-            count, converged = self.step_count, self._last_converged
-            side.wait_stream(current)
-            try:
-                with torch.cuda.stream(side):
-                    with torch.cuda.graph(graph, stream=side):
-                        self.step(batch)
-            except Exception:  # something in the step needs the host after all: stay eager for this batch
-                st["failed"] = True
-                return False
-            finally:
-                current.wait_stream(side)
-                _lib.workspaces.unshare(current.device, side.cuda_stream)
-                self.step_count, self._last_converged = count, converged  # (the capture ran nothing)
-            if self._graph_key(batch) != key:  # the step replaced a buffer: what was captured is already stale
+            graph = self._capture(batch, lambda: self.step(batch), key)
+            if graph is None:
                 st["failed"] = True
                 return False
             st["graph"] = graph
@@ -662,6 +670,63 @@ class BaseDynamics(HookRegistryMixin):
         self.step_count += 1
         return True
 
+    #: whole steps in the graph that joins ``post_update`` of a step with ``pre_update`` of the next
+    _GRAPH_JOINED_STEPS = 4
+
+    def _joined_steps_possible(self, batch) -> bool:
+        """Several steps may be captured as one graph whose inner boundaries are one launch each
+        (``post_then_pre_update``) when nothing can run between two steps: no hook on the four stages around the
+        boundary, and no status mask (it is worked out from ``batch.status`` at the start of every step)."""
+        if not callable(getattr(self, "post_then_pre_update", None)) or getattr(batch, "status", None) is not None:
+            return False
+        boundary = (DynamicsStage.AFTER_POST_UPDATE, DynamicsStage.AFTER_STEP, DynamicsStage.BEFORE_STEP,
+                    DynamicsStage.BEFORE_PRE_UPDATE)
+        for hook in self.hooks:
+            runs_on_stage = getattr(hook, "_runs_on_stage", None)
+            if runs_on_stage is not None:
+                if any(runs_on_stage(stage) for stage in boundary):
+                    return False
+            elif hook.stage in boundary:
+                return False
+        return True
+
+    def _joined_steps(self, batch, k: int) -> None:
+        """``k`` steps as ``step`` takes them when the stages around the step boundary are empty, with the
+        boundaries inside taken as one launch.  (Called under graph capture only.)"""
+        self._active_mask = None
+        self.pre_update(batch)
+        for j in range(k):
+            self._call_hooks(DynamicsStage.AFTER_PRE_UPDATE, batch)
+            self._call_hooks(DynamicsStage.BEFORE_COMPUTE, batch)
+            self.compute(batch)
+            self._call_hooks(DynamicsStage.AFTER_COMPUTE, batch)
+            self._call_hooks(DynamicsStage.BEFORE_POST_UPDATE, batch)
+            if j == k - 1:
+                self.post_update(batch)
+            elif not self.post_then_pre_update(batch):
+                raise RuntimeError("no joined form of post_update and pre_update for this batch")
+            self.step_count += 1
+
+    def _graph_steps(self, batch, remaining: int) -> int:
+        """As many steps by graph replay as one replay takes (``_GRAPH_JOINED_STEPS`` when that many remain and the
+        joined graph exists or can be made, else one); 0: not possible now."""
+        k = self._GRAPH_JOINED_STEPS
+        st = getattr(self, "_graph_state", None)
+        if (remaining >= k and st is not None and st.get("graph") is not None and not st.get("joined_failed")
+                and self._graph_eligible(batch) and st["key"] == self._graph_key(batch)
+                and self._joined_steps_possible(batch)):
+            if st.get("joined") is None:
+                graph = self._capture(batch, lambda: self._joined_steps(batch, k), st["key"])
+                if graph is None:
+                    st["joined_failed"] = True
+                    return 1 if self._graph_step(batch) else 0
+                st["joined"] = graph
+            st["joined"].replay()
+            self._last_converged = None
+            self.step_count += k
+            return k
+        return 1 if self._graph_step(batch) else 0
+
     def run(self, batch, n_steps: int | None = None):
         resolved = n_steps if n_steps is not None else self.n_steps
         if resolved is None:
@@ -669,10 +734,14 @@ class BaseDynamics(HookRegistryMixin):
                              f"construction time via `{type(self).__name__}(..., n_steps=N)`.")
         self._open_hooks()
         try:
-            for _ in range(resolved):
-                if self._graph_step(batch):
+            taken = 0
+            while taken < resolved:
+                replayed = self._graph_steps(batch, resolved - taken)
+                if replayed:
+                    taken += replayed
                     continue
                 batch, converged = self.step(batch)
+                taken += 1
                 if self.sampler is None and converged is not None and converged.numel() == batch.num_graphs:
                     break
         finally:

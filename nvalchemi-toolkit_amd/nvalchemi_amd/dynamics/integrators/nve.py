@@ -45,3 +45,14 @@ class NVE(BaseDynamics):
     def post_update(self, batch) -> None:
         vv_velocity_finalize_masked(batch.velocities, batch.forces, batch.atomic_masses, self._state.dt,
                                     batch.batch_idx, self._active_mask)
+
+    def post_then_pre_update(self, batch) -> bool:
+        """``post_update`` of one step and ``pre_update`` of the next in one launch; False where that form does
+        not exist (float64 arrays), and the caller makes the two calls."""
+        if batch.positions.dtype != torch.float32:
+            return False
+        from ... import _lib
+
+        _lib.vv_finalize_then_update(batch.positions, batch.velocities, batch.forces, batch.atomic_masses,
+                                     self._state.dt, batch.batch_idx, self._active_mask)
+        return True

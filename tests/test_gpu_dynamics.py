@@ -1043,3 +1043,97 @@ def test_status_migration_in_one_launch_equals_the_torch_expression():
         hook(DynamicsContext(batch=batch, model=None, workflow=None), None)
         out.append(batch.status.clone())
     assert torch.equal(out[0], out[1]) and out[0].view(-1).tolist() == [1, 0, 1, 0, 2, 0]
+
+
+def test_joined_velocity_verlet_halves_equal_the_two_calls_in_a_row():
+    """nvamd_vv_finalize_then_update against nvamd_vv_velocity_finalize followed by nvamd_vv_position_update with the
+    same forces: bit for bit, with and without a system mask, on aligned arrays (four floats per lane) and on views
+    that start off a 16-byte boundary (one float per lane), for atom counts around the lane boundaries."""
+    from nvalchemi_amd import _lib
+
+    g = torch.Generator().manual_seed(11)
+    for N in (1, 2, 5, 255, 256, 1027):
+        M = 4
+        bidx = torch.sort(torch.randint(0, M, (N,), generator=g)).values.to(torch.int32).to(DEV)
+        base = [torch.randn(N + 1, 3, generator=g).to(DEV) for _ in range(3)]
+        masses = (torch.rand(N, generator=g) * 20 + 1).to(DEV)
+        dt = (torch.rand(M, generator=g) * 0.1 + 0.01).to(DEV)
+        for active in (None, torch.tensor([True, False, True, True], device=DEV)):
+            for offset in (0, 1):  # (offset 1: the rows start 12 bytes into the allocation)
+                P0, V0, F = (b[offset:offset + N] for b in base)
+                Pa, Va = P0.clone(), V0.clone()
+                Pb, Vb = P0.clone(), V0.clone()
+                if offset:
+                    hold = [torch.empty(N + 1, 3, device=DEV) for _ in range(4)]
+                    Pa, Va, Pb, Vb = (h[1:] for h in hold)
+                    Pa.copy_(P0); Va.copy_(V0); Pb.copy_(P0); Vb.copy_(V0)
+                    assert Pa.data_ptr() % 16 != 0
+                _lib.vv_velocity_finalize(Va, F, masses, dt, bidx, active)
+                _lib.vv_position_update(Pa, Va, F, masses, dt, bidx, active)
+                _lib.vv_finalize_then_update(Pb, Vb, F, masses, dt, bidx, active)
+                assert torch.equal(Pa, Pb) and torch.equal(Va, Vb), (N, active is not None, offset)
+                if active is not None and bool((bidx == 1).any()):
+                    off = (bidx == 1)
+                    assert torch.equal(Pb[off], P0[off]) and torch.equal(Vb[off], V0[off])
+
+
+def test_runs_replayed_four_steps_at_a_time_equal_eager_ones():
+    """``run`` replays four steps per graph where it may (NVE, no hook around the step boundary, no status), with the
+    closing half kick of a step and the opening half kick and drift of the next in one launch: positions, velocities
+    and forces after 3 to 23 steps equal those of eager steps bit for bit, whatever is left over after the last
+    group of four; with a hook registered after the step, or a status on the batch, steps are replayed one at a
+    time."""
+    from nvalchemi_amd.dynamics import NVE, DynamicsStage
+    from nvalchemi_amd.models import LennardJonesModelWrapper
+
+    P, C, pb, ptr = fcc_boxes(seed=9, n_boxes=4, reps=3, a=3.7, jitter=0.08)
+    n = len(P)
+    V = np.random.default_rng(9).normal(0, 0.02, (n, 3)).astype(np.float32)
+    sigma = float((3.6 / np.sqrt(2)) / 2 ** (1 / 6))
+
+    def make():
+        batch = make_batch(P, np.full(n, 29, dtype=np.int64), np.full(n, 63.546, dtype=np.float32), C, pb, ptr, V)
+        model = LennardJonesModelWrapper(epsilon=0.01, sigma=sigma, cutoff=5.0)
+        return batch, NVE(model, dt=1.0, hooks=model.make_neighbor_hooks())
+
+    for n_steps in (3, 6, 7, 12, 23):
+        out = []
+        for replay in (False, True):
+            batch, dyn = make()
+            dyn.graph_replay = replay
+            dyn.run(batch, n_steps=n_steps)
+            torch.cuda.synchronize()
+            assert dyn.step_count == n_steps
+            if replay:
+                # (a few eager steps while the hook settles its buffers, one step replayed alone, then four at a time)
+                joined = dyn._graph_state.get("joined")
+                assert joined is None if n_steps <= 6 else (joined is not None or n_steps < 12), n_steps
+            out.append(batch)
+        for name in ("positions", "velocities", "forces", "energy"):
+            assert torch.equal(getattr(out[0], name), getattr(out[1], name)), (name, n_steps)
+    # two runs in a row use the graphs of the first
+    batch, dyn = make()
+    dyn.run(batch, n_steps=9)
+    first = dyn._graph_state["joined"]
+    dyn.run(batch, n_steps=9)
+    eager_batch, eager = make()
+    eager.graph_replay = False
+    eager.run(eager_batch, n_steps=18)
+    assert dyn._graph_state["joined"] is first and torch.equal(batch.positions, eager_batch.positions)
+
+    class Watch:
+        frequency = 1
+        graph_safe = True
+        stage = DynamicsStage.AFTER_STEP
+
+        def __call__(self, ctx, stage):
+            pass
+
+    batch, dyn = make()
+    dyn.register_hook(Watch())
+    dyn.run(batch, n_steps=12)
+    assert dyn._graph_state["graph"] is not None and dyn._graph_state.get("joined") is None
+    batch, dyn = make()
+    batch.status = torch.zeros(batch.num_graphs, 1, dtype=torch.long, device=DEV)
+    dyn.run(batch, n_steps=12)
+    assert dyn._graph_state["graph"] is not None and dyn._graph_state.get("joined") is None
