@@ -670,7 +670,7 @@ class BaseDynamics(HookRegistryMixin):
         self.step_count += 1
         return True
 
-    #: whole steps in the graph that joins ``post_update`` of a step with ``pre_update`` of the next
+    #: whole steps, at most, in a graph that joins ``post_update`` of a step with ``pre_update`` of the next
     _GRAPH_JOINED_STEPS = 4
 
     def _joined_steps_possible(self, batch) -> bool:
@@ -708,20 +708,21 @@ class BaseDynamics(HookRegistryMixin):
             self.step_count += 1
 
     def _graph_steps(self, batch, remaining: int) -> int:
-        """As many steps by graph replay as one replay takes (``_GRAPH_JOINED_STEPS`` when that many remain and the
-        joined graph exists or can be made, else one); 0: not possible now."""
-        k = self._GRAPH_JOINED_STEPS
+        """As many steps by graph replay as one replay takes: up to ``_GRAPH_JOINED_STEPS`` of those that remain where
+        steps can be joined (one graph per number of steps, made when first needed), else one; 0: not possible now."""
+        k = min(remaining, self._GRAPH_JOINED_STEPS)
         st = getattr(self, "_graph_state", None)
-        if (remaining >= k and st is not None and st.get("graph") is not None and not st.get("joined_failed")
+        if (k >= 2 and st is not None and st.get("graph") is not None and not st.get("joined_failed")
                 and self._graph_eligible(batch) and st["key"] == self._graph_key(batch)
                 and self._joined_steps_possible(batch)):
-            if st.get("joined") is None:
+            joined = st.setdefault("joined", {})
+            if k not in joined:
                 graph = self._capture(batch, lambda: self._joined_steps(batch, k), st["key"])
                 if graph is None:
                     st["joined_failed"] = True
                     return 1 if self._graph_step(batch) else 0
-                st["joined"] = graph
-            st["joined"].replay()
+                joined[k] = graph
+            joined[k].replay()
             self._last_converged = None
             self.step_count += k
             return k
