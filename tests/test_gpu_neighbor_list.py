@@ -105,6 +105,22 @@ def test_random_periodic_batches_match_brute_force(case, half):
     check_against_oracle(P, C, pb, ptr, rc, half=half)
 
 
+def test_a_batch_whose_mean_system_takes_the_sort_with_eight_atoms_per_lane():
+    """Systems of 300 to 6000 atoms with a mean between 2049 and 4096: the per-system sort keeps eight atoms per lane
+    in registers for those that fit (up to 4096 atoms) and bins the larger one twice; triclinic cells."""
+    from _systems import ptr_from_counts, random_triclinic_cell
+
+    rng = np.random.default_rng(31)
+    counts = [300, 3900, 4700, 2200, 4096]
+    cells, pos = [], []
+    for n in counts:
+        H = random_triclinic_cell(rng, (n / 0.8) ** (1.0 / 3.0))
+        pos.append((rng.uniform(0, 1, (n, 3)) @ H.astype(np.float64)).astype(np.float32))
+        cells.append(H)
+    P, C = np.concatenate(pos), np.stack(cells).astype(np.float32)
+    check_against_oracle(P, C, np.ones((len(counts), 3), dtype=bool), ptr_from_counts(counts), 2.5)
+
+
 def test_molecules_without_cell():
     P, Z, M, ptr = molecules_batch(seed=0)
     check_against_oracle(P, None, None, ptr, 5.0, K=32)
