@@ -610,10 +610,13 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* s_part, int* tot
 }
 
 // kKeep: atoms per thread whose positions and bins stay in registers from the histogram to the scatter (systems of
-// up to kKeep * kSortBlock atoms are binned once).  Four for batches of small systems, where the registers of eight
-// would leave one workgroup per CU; eight when the mean system has more than 2048 atoms.
-template <int kKeep>
-__global__ __launch_bounds__(kSortBlock) void nl_system_sort_kernel(NlArgs a, NlWorkspace ws) {
+// up to kKeep * kSortBlock atoms are binned once): four, or eight when the mean system has more than 2048 atoms.
+// kWaves: waves per SIMD the kernel is built for.  With more systems than CUs the instance of four atoms is held to
+// 128 registers (four waves per SIMD, two workgroups per CU: one system's chain of dependent steps then runs
+// beside another's, 6 % off the build of 2048 mixed systems for 19 spilled words); with fewer systems than that
+// nothing would run beside it, and it keeps its 152 registers (the spills cost 64 boxes of 500 atoms 2 %).
+template <int kKeep, int kWaves>
+__global__ __launch_bounds__(kSortBlock, kWaves) void nl_system_sort_kernel(NlArgs a, NlWorkspace ws) {
     __shared__ NlSys s_sys;
     __shared__ uint32_t s_bounds[6];
     __shared__ int s_err;
@@ -1490,9 +1493,11 @@ static int32_t nl_build_impl(const float* positions, const float* cell, const do
     if (per_system) {
         // many small systems: set-up to scatter in one workgroup per system
         if (!a.pos64 && n_atoms / n_systems > 4 * kSortBlock && n_atoms / n_systems <= 8 * kSortBlock)
-            hipLaunchKernelGGL(nl_system_sort_kernel<8>, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
+            hipLaunchKernelGGL((nl_system_sort_kernel<8, 2>), dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
+        else if (n_systems > 256)
+            hipLaunchKernelGGL((nl_system_sort_kernel<4, 4>), dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
         else
-            hipLaunchKernelGGL(nl_system_sort_kernel<4>, dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
+            hipLaunchKernelGGL((nl_system_sort_kernel<4, 2>), dim3(n_systems), dim3(kSortBlock), 0, st, a, ws);
     } else {
         size_t n_prep = (size_t)ws.max_cells > (size_t)n_systems ? (size_t)ws.max_cells : (size_t)n_systems;
         hipLaunchKernelGGL(nl_prepare_kernel, blocks(n_prep), blk, 0, st, a, ws);
