@@ -55,8 +55,8 @@ RELAX_MAXSTEP = 0.07
 # half of what a copy kernel of known size fetches and WRITE_SIZE reads its writes in KiB, so
 # bytes = 1024 * (2 * FETCH_SIZE + WRITE_SIZE).  Summed over the kernels of each entry point.
 MEASURED_TRAFFIC_BYTES = {
-    "nl": 1024 * (2 * (32580 + 6108) + (850125 + 61273)),   # search + per-system sort
-    "lj": 1024 * (2 * (167662 + 23) + 15822 + 21),          # pair kernel + conversion of the per-system sums
+    "nl": 1024 * (2 * (32561 + 6106) + (850038 + 63352)),   # search + per-system sort
+    "lj": 1024 * (2 * (165411 + 23) + 15748 + 21),          # pair kernel + conversion of the per-system sums
 }
 
 
